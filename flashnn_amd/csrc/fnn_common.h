@@ -1,0 +1,84 @@
+// Shared device/host helpers for the flashnn_amd HIP kernels (gfx950 / CDNA4 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/flashnn_hip.h"
+
+namespace fnn {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+// ---- 16-bit float <-> fp32 on raw bit patterns -------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// round-to-nearest-even; inputs here are finite
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    union { uint16_t u; _Float16 f; } c;
+    c.u = (uint16_t)h;
+    return (float)c.f;
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    union { uint16_t u; _Float16 f; } c;
+    c.f = (_Float16)f;  // v_cvt_f16_f32, round-to-nearest-even
+    return c.u;
+}
+
+template <int DT> __device__ __forceinline__ float bits_to_f32(uint32_t h) {
+    if constexpr (DT == FNN_F16) return f16_bits_to_f32(h);
+    else return bf16_bits_to_f32(h);
+}
+template <int DT> __device__ __forceinline__ uint32_t f32_to_bits(float f) {
+    if constexpr (DT == FNN_F16) return f32_to_f16_bits(f);
+    else return f32_to_bf16_bits(f);
+}
+
+// Load element i of an array whose element type is only known at run time (uniform branch).
+__device__ __forceinline__ float load_as_f32(const void* p, int64_t i, int dtype) {
+    if (dtype == FNN_F32) return ((const float*)p)[i];
+    uint32_t h = ((const uint16_t*)p)[i];
+    return dtype == FNN_F16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
+}
+
+__device__ __forceinline__ void store_from_f32(void* p, int64_t i, float v, int dtype) {
+    if (dtype == FNN_F32) ((float*)p)[i] = v;
+    else ((uint16_t*)p)[i] = (uint16_t)(dtype == FNN_F16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v));
+}
+
+// ---- wave / block reductions -------------------------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+// ---- host side ----------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+inline bool is16(int dt) { return dt == FNN_F16 || dt == FNN_BF16; }
+inline bool isflt(int dt) { return dt == FNN_F16 || dt == FNN_BF16 || dt == FNN_F32; }
+
+}  // namespace fnn

@@ -1,0 +1,394 @@
+// Weight-only GEMMs for gfx950 (fp16/bf16 activations, int8 or packed int4 weights):
+//   out[m,n] = sum_k act[m,k] * (w[n,k] - zp[g(k),n]) * scale[g(k),n]  (+ bias[n])
+//
+// Streaming kernel (decode shapes; K % 64 == 0, 16-byte aligned rows)
+//   * a 512-thread workgroup (8 waves) owns one tile of 16 weight rows (16 output channels
+//     for int8, 32 for packed int4) and up to 64 activation rows; the waves split K;
+//   * every lane streams its weight row with 16-byte loads kept PF steps ahead in
+//     registers (no LDS, no barriers in the loop), converts the integers to the
+//     activation type in registers and feeds them to v_mfma_f32_16x16x32_{f16,bf16} as the
+//     "A" operand; the activations are the "B" operand (columns beyond M are zero);
+//   * integer -> float conversion uses exponent tricks instead of per-element converts:
+//       int4:  (nibble ^ 8) | 0x4300  is the bf16 number 128 + (v + 8),
+//              (nibble ^ 8) | 0x6400  is the fp16 number 1024 + (v + 8);
+//       int8 -> fp16: byte ^ 0x80 placed under 0x64 gives 1024 + (v + 128);
+//       int8 -> bf16: v_cvt_f32_ubyte of byte ^ 0x80, upper 16 bits (exact: 8 bits).
+//     The constant offset c is removed together with the zero point:
+//       sum_k (c + v_k - zp) a_k  =  acc - (c + zp) * sum_k a_k,
+//     where sum_k a_k comes from one more MFMA against a matrix of ones;
+//   * group scales are applied whenever a K-group ends (fp32), per-channel scales once;
+//   * the 8 partial tiles are added in a fixed order through LDS (deterministic, no
+//     atomics), then bias, rounding and the store.
+//
+// Any other shape takes a guarded one-output-per-thread kernel.
+//
+// Reference semantics: flashnn/quant_gemm.py:148-206; layouts
+// flashnn/triton_kernels/gemm_a16w4.py:163-182 (nibble order), :296-297 (scale rows).
+#include "fnn_common.h"
+
+namespace fnn {
+
+struct WoArgs {
+    const void* act;
+    const int8_t* qw;
+    const void* scale;
+    const void* zp;
+    const void* bias;
+    void* out;
+    int M, N, K;          // N = output channels
+    int64_t lda, ldw, ldc;
+    int group;            // 0 = per channel
+    int out_dtype, scale_dtype, zp_dtype, bias_dtype;
+    int m_base;           // first activation row handled by this launch
+};
+
+constexpr int kWoWaves = 8;
+constexpr int kPF = 8;    // weight loads in flight per lane
+constexpr int kPFA = 2;   // activation steps in flight per lane
+
+template <int ADT> struct MfmaT;
+template <> struct MfmaT<FNN_F16> {
+    typedef v8h vec;
+    static constexpr uint32_t one2 = 0x3C003C00u;
+    __device__ static __forceinline__ v4f mma(v4u a, v4u b, v4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a),
+                                                      __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+    }
+};
+template <> struct MfmaT<FNN_BF16> {
+    typedef v8bf vec;
+    static constexpr uint32_t one2 = 0x3F803F80u;
+    __device__ static __forceinline__ v4f mma(v4u a, v4u b, v4f c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a),
+                                                       __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+    }
+};
+
+// 16 int8 (k .. k+15 of one row) -> two MFMA operands in natural k order.
+// Values come out as c + (v + 128) with c = 1024 (fp16) or 0 (bf16).
+template <int ADT>
+__device__ __forceinline__ void convert_w8(const v4u w, v4u& s0, v4u& s1) {
+    uint32_t o[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t x = w[q] ^ 0x80808080u;
+        if constexpr (ADT == FNN_F16) {
+            o[2 * q] = __builtin_amdgcn_perm(x, 0x64646464u, 0x00050004u);
+            o[2 * q + 1] = __builtin_amdgcn_perm(x, 0x64646464u, 0x00070006u);
+        } else {
+            const uint32_t f0 = __float_as_uint((float)(x & 0xFFu));
+            const uint32_t f1 = __float_as_uint((float)((x >> 8) & 0xFFu));
+            const uint32_t f2 = __float_as_uint((float)((x >> 16) & 0xFFu));
+            const uint32_t f3 = __float_as_uint((float)(x >> 24));
+            o[2 * q] = __builtin_amdgcn_perm(f1, f0, 0x07060302u);
+            o[2 * q + 1] = __builtin_amdgcn_perm(f3, f2, 0x07060302u);
+        }
+    }
+    s0 = v4u{o[0], o[1], o[2], o[3]};
+    s1 = v4u{o[4], o[5], o[6], o[7]};
+}
+
+// 16 bytes = 16 k of two channels (low nibble: even channel).  Each operand holds k in the
+// order (0,2)(1,3)(4,6)(5,7); values are c + (v + 8), c = 1024 (fp16) / 128 (bf16).
+template <int ADT>
+__device__ __forceinline__ void convert_w4(const v4u w, v4u& e0, v4u& e1, v4u& o0, v4u& o1) {
+    constexpr uint32_t mag = ADT == FNN_F16 ? 0x64006400u : 0x43004300u;
+    uint32_t e[8], o[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t x = w[q] ^ 0x88888888u;
+        e[2 * q] = (x & 0x000F000Fu) | mag;
+        e[2 * q + 1] = ((x >> 8) & 0x000F000Fu) | mag;
+        o[2 * q] = ((x >> 4) & 0x000F000Fu) | mag;
+        o[2 * q + 1] = ((x >> 12) & 0x000F000Fu) | mag;
+    }
+    e0 = v4u{e[0], e[1], e[2], e[3]};
+    e1 = v4u{e[4], e[5], e[6], e[7]};
+    o0 = v4u{o[0], o[1], o[2], o[3]};
+    o1 = v4u{o[4], o[5], o[6], o[7]};
+}
+
+// reorder 8 consecutive 16-bit values to (0,2)(1,3)(4,6)(5,7)
+__device__ __forceinline__ v4u perm_act_w4(const v4u a) {
+    return v4u{__builtin_amdgcn_perm(a[1], a[0], 0x05040100u), __builtin_amdgcn_perm(a[1], a[0], 0x07060302u),
+               __builtin_amdgcn_perm(a[3], a[2], 0x05040100u), __builtin_amdgcn_perm(a[3], a[2], 0x07060302u)};
+}
+
+template <int WBITS, int ADT, int MB, bool GROUPED>
+__global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoArgs p) {
+    typedef MfmaT<ADT> MT;
+    constexpr int NH = WBITS == 4 ? 2 : 1;      // channel halves per weight row (int4: even/odd)
+    constexpr float c_off = WBITS == 4 ? (ADT == FNN_F16 ? 1024.f + 8.f : 128.f + 8.f)
+                                       : (ADT == FNN_F16 ? 1024.f + 128.f : 128.f);
+    __shared__ float red[kWoWaves][MB][NH][4][64];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 15;   // weight row within the tile (A operand) / activation row (B operand)
+    const int lg = lane >> 4;   // k sub-block of the lane
+
+    // XCD-aware tile order: ids congruent mod 8 share an L2; give each XCD a contiguous band so
+    // that neighbouring tiles (which share cache lines of the scale rows) meet in the same L2.
+    const int wrows = WBITS == 4 ? p.N / 2 : p.N;
+    const int tiles = (wrows + 15) / 16;
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (tile >= tiles) return;
+    const int row0 = tile * 16;
+
+    const int steps = p.K / 64;
+    const int s_begin = (int)((int64_t)steps * wave / kWoWaves);
+    const int s_end = (int)((int64_t)steps * (wave + 1) / kWoWaves);
+
+    const int wrow = min(row0 + li, wrows - 1);
+    const char* wptr = (const char*)p.qw + (int64_t)wrow * p.ldw + lg * 16;
+    const uint16_t* aptr[MB];
+    bool avalid[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = p.m_base + mb * 16 + li;
+        avalid[mb] = m < p.M;
+        aptr[mb] = (const uint16_t*)p.act + (int64_t)min(m, p.M - 1) * p.lda + lg * 16;
+    }
+
+    auto load_w = [&](int step) -> v4u {
+        const int s = min(step, s_end - 1);
+        return *(const v4u*)(wptr + (int64_t)s * 64);
+    };
+    auto load_a = [&](int mb, int step, int half) -> v4u {
+        const int s = min(step, s_end - 1);
+        return avalid[mb] ? *(const v4u*)(aptr[mb] + (int64_t)s * 64 + half * 8) : v4u{0, 0, 0, 0};
+    };
+
+    v4f outv[MB][NH], accg[MB][NH], asum[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        asum[mb] = v4f{0, 0, 0, 0};
+#pragma unroll
+        for (int h = 0; h < NH; ++h) { outv[mb][h] = v4f{0, 0, 0, 0}; accg[mb][h] = v4f{0, 0, 0, 0}; }
+    }
+
+    // channel of output register r, half h of this lane
+    auto chan = [&](int h, int r) -> int {
+        const int wr = row0 + 4 * lg + r;
+        return WBITS == 4 ? 2 * wr + h : wr;
+    };
+    // fold the running group sums into the outputs with the scales of K-group `grp`
+    auto fold = [&](int grp) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = min(chan(h, r), p.N - 1);
+                const int64_t idx = GROUPED ? (int64_t)grp * p.N + n : n;
+                const float sc = load_as_f32(p.scale, idx, p.scale_dtype);
+                const float zc = c_off + (p.zp ? load_as_f32(p.zp, idx, p.zp_dtype) : 0.f);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    outv[mb][h][r] += sc * (accg[mb][h][r] - zc * asum[mb][r]);
+                    accg[mb][h][r] = 0.f;
+                }
+            }
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) asum[mb] = v4f{0, 0, 0, 0};
+    };
+
+    if (s_begin < s_end) {
+        v4u wq[kPF];
+        v4u aq[kPFA][MB][2];
+#pragma unroll
+        for (int i = 0; i < kPF; ++i) wq[i] = load_w(s_begin + i);
+#pragma unroll
+        for (int i = 0; i < kPFA; ++i)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                aq[i][mb][0] = load_a(mb, s_begin + i, 0);
+                aq[i][mb][1] = load_a(mb, s_begin + i, 1);
+            }
+        const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+        const int gsteps = GROUPED ? p.group / 64 : 1;
+
+        for (int sb = s_begin; sb < s_end; sb += kPF) {
+#pragma unroll
+            for (int i = 0; i < kPF; ++i) {
+                const int step = sb + i;
+                if (step < s_end) {
+                    const v4u w = wq[i];
+                    wq[i] = load_w(step + kPF);
+                    v4u a[MB][2];
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) {
+                        a[mb][0] = aq[i % kPFA][mb][0];
+                        a[mb][1] = aq[i % kPFA][mb][1];
+                        aq[i % kPFA][mb][0] = load_a(mb, step + kPFA, 0);
+                        aq[i % kPFA][mb][1] = load_a(mb, step + kPFA, 1);
+                    }
+                    if constexpr (WBITS == 4) {
+                        v4u e0, e1, o0, o1;
+                        convert_w4<ADT>(w, e0, e1, o0, o1);
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb) {
+                            const v4u b0 = perm_act_w4(a[mb][0]);
+                            const v4u b1 = perm_act_w4(a[mb][1]);
+                            accg[mb][0] = MT::mma(e0, b0, accg[mb][0]);
+                            accg[mb][1] = MT::mma(o0, b0, accg[mb][1]);
+                            asum[mb] = MT::mma(ones, b0, asum[mb]);
+                            accg[mb][0] = MT::mma(e1, b1, accg[mb][0]);
+                            accg[mb][1] = MT::mma(o1, b1, accg[mb][1]);
+                            asum[mb] = MT::mma(ones, b1, asum[mb]);
+                        }
+                    } else {
+                        v4u s0, s1;
+                        convert_w8<ADT>(w, s0, s1);
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb) {
+                            accg[mb][0] = MT::mma(s0, a[mb][0], accg[mb][0]);
+                            asum[mb] = MT::mma(ones, a[mb][0], asum[mb]);
+                            accg[mb][0] = MT::mma(s1, a[mb][1], accg[mb][0]);
+                            asum[mb] = MT::mma(ones, a[mb][1], asum[mb]);
+                        }
+                    }
+                    if constexpr (GROUPED) {
+                        if ((step + 1) % gsteps == 0 || step + 1 == s_end) fold(step / gsteps);
+                    }
+                }
+            }
+        }
+        if constexpr (!GROUPED) fold(0);
+    }
+
+    // ---- add the 8 partial tiles in wave order, then bias / rounding / store ----
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int h = 0; h < NH; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) red[wave][mb][h][r][lane] = outv[mb][h][r];
+    __syncthreads();
+    constexpr int ELEMS = MB * NH * 4 * 64;
+    for (int e = threadIdx.x; e < ELEMS; e += kWoWaves * 64) {
+        const int l = e & 63;
+        const int r = (e >> 6) & 3;
+        const int h = NH == 2 ? (e >> 8) & 1 : 0;
+        const int mb = e / (NH * 256);
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWoWaves; ++w) v += red[w][mb][h][r][l];
+        const int m = p.m_base + mb * 16 + (l & 15);
+        const int wr = row0 + 4 * (l >> 4) + r;
+        const int n = WBITS == 4 ? 2 * wr + h : wr;
+        if (m < p.M && n < p.N) {
+            if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+            store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ guarded fallback
+template <int WBITS, int ADT>
+__global__ __launch_bounds__(256) void gemm_wo_any_kernel(const WoArgs p) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)p.M * p.N) return;
+    const int m = (int)(idx / p.N), n = (int)(idx % p.N);
+    const uint16_t* a = (const uint16_t*)p.act + (int64_t)m * p.lda;
+    const int8_t* w = p.qw + (int64_t)(WBITS == 4 ? n >> 1 : n) * p.ldw;
+    const int g = p.group > 0 ? p.group : p.K;
+    float total = 0.f;
+    for (int k0 = 0; k0 < p.K; k0 += g) {
+        const int64_t si = p.group > 0 ? (int64_t)(k0 / g) * p.N + n : n;
+        const float sc = load_as_f32(p.scale, si, p.scale_dtype);
+        const float z = p.zp ? load_as_f32(p.zp, si, p.zp_dtype) : 0.f;
+        float part = 0.f;
+        const int k1 = min(k0 + g, p.K);
+        for (int k = k0; k < k1; ++k) {
+            int q = w[k];
+            if constexpr (WBITS == 4) q = (n & 1) ? (q >> 4) : ((int)((uint32_t)q << 28) >> 28);
+            part += bits_to_f32<ADT>(a[k]) * ((float)q - z);
+        }
+        total += sc * part;
+    }
+    if (p.bias) total += load_as_f32(p.bias, n, p.bias_dtype);
+    store_from_f32(p.out, (int64_t)m * p.ldc + n, total, p.out_dtype);
+}
+
+// ------------------------------------------------------------------------ dispatch
+template <int WBITS, int ADT, int MB>
+static void launch_stream(WoArgs& p, hipStream_t st) {
+    const int wrows = WBITS == 4 ? p.N / 2 : p.N;
+    const int tiles = (wrows + 15) / 16;
+    const dim3 grid(((tiles + 7) / 8) * 8), block(kWoWaves * 64);
+    if (p.group > 0) gemm_wo_stream_kernel<WBITS, ADT, MB, true><<<grid, block, 0, st>>>(p);
+    else gemm_wo_stream_kernel<WBITS, ADT, MB, false><<<grid, block, 0, st>>>(p);
+}
+
+template <int WBITS, int ADT>
+static void dispatch_wo(WoArgs& p, hipStream_t st) {
+    const bool fast = p.K % 64 == 0 && (p.group == 0 || p.group % 64 == 0) && p.ldw % 16 == 0 &&
+                      p.lda % 8 == 0 && ((uintptr_t)p.qw % 16) == 0 && ((uintptr_t)p.act % 16) == 0;
+    if (!fast) {
+        const int64_t total = (int64_t)p.M * p.N;
+        gemm_wo_any_kernel<WBITS, ADT><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(p);
+        return;
+    }
+    // up to 64 activation rows per pass over the weights
+    for (int m0 = 0; m0 < p.M; m0 += 64) {
+        p.m_base = m0;
+        const int rem = p.M - m0;
+        if (rem <= 16) launch_stream<WBITS, ADT, 1>(p, st);
+        else if (rem <= 32) launch_stream<WBITS, ADT, 2>(p, st);
+        else launch_stream<WBITS, ADT, 4>(p, st);
+    }
+}
+
+template <int WBITS>
+static int run_wo(const char* fn, void* out, const void* act, const void* qw, const void* scale,
+                  const void* bias, const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda,
+                  int64_t ldw, int64_t ldc, int64_t group, int act_dtype, int out_dtype,
+                  int scale_dtype, int zp_dtype, int bias_dtype, void* stream) {
+    if (!out || !act || !qw || !scale) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
+    if (M < 0 || N < 0 || K <= 0 || lda < K || ldw < K || ldc < N || group < 0) {
+        set_error("%s: bad shape M=%lld N=%lld K=%lld lda=%lld ldw=%lld ldc=%lld group=%lld", fn,
+                  (long long)M, (long long)N, (long long)K, (long long)lda, (long long)ldw,
+                  (long long)ldc, (long long)group);
+        return FNN_ERR_ARG;
+    }
+    if (WBITS == 4 && (N & 1)) { set_error("%s: N must be even for packed int4 weights", fn); return FNN_ERR_ARG; }
+    if (group > 0 && K % group != 0) { set_error("%s: K=%lld is not a multiple of the group size %lld", fn, (long long)K, (long long)group); return FNN_ERR_ARG; }
+    if (!is16(act_dtype) || !is16(out_dtype)) { set_error("%s: activations and output must be fp16 or bf16", fn); return FNN_ERR_UNSUPPORTED; }
+    if (!isflt(scale_dtype) || (zp && !isflt(zp_dtype)) || (bias && !isflt(bias_dtype))) {
+        set_error("%s: scale / zero-point / bias type must be fp16, bf16 or fp32", fn);
+        return FNN_ERR_UNSUPPORTED;
+    }
+    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) { set_error("%s: shape too large", fn); return FNN_ERR_UNSUPPORTED; }
+    if (M == 0 || N == 0) return FNN_OK;
+    WoArgs p{};
+    p.act = act; p.qw = (const int8_t*)qw; p.scale = scale; p.zp = zp; p.bias = bias; p.out = out;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldw = ldw; p.ldc = ldc; p.group = (int)group;
+    p.out_dtype = out_dtype; p.scale_dtype = scale_dtype; p.zp_dtype = zp_dtype; p.bias_dtype = bias_dtype;
+    if (act_dtype == FNN_F16) dispatch_wo<WBITS, FNN_F16>(p, (hipStream_t)stream);
+    else dispatch_wo<WBITS, FNN_BF16>(p, (hipStream_t)stream);
+    return check_launch(fn);
+}
+
+}  // namespace fnn
+
+using namespace fnn;
+
+extern "C" int fnn_gemm_a16w8(void* out, const void* act, const void* qw, const void* scale,
+                              const void* bias, const void* zp, int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldw, int64_t ldc, int64_t group, int act_dtype,
+                              int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
+                              void* stream) {
+    return run_wo<8>("fnn_gemm_a16w8", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group,
+                     act_dtype, out_dtype, scale_dtype, zp_dtype, bias_dtype, stream);
+}
+
+extern "C" int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const void* scale,
+                              const void* bias, const void* zp, int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldw, int64_t ldc, int64_t group, int act_dtype,
+                              int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
+                              void* stream) {
+    return run_wo<4>("fnn_gemm_a16w4", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group,
+                     act_dtype, out_dtype, scale_dtype, zp_dtype, bias_dtype, stream);
+}

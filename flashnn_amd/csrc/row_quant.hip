@@ -1,0 +1,284 @@
+// Row kernels: per-token dynamic int8 quantisation and fused RMSNorm + quantisation.
+//
+// One 256-thread workgroup owns one row.  The row is read from HBM once (16-byte loads)
+// and kept in VGPRs across the reduction(s), so the HBM traffic is the algorithmic
+// 2*K bytes in + K bytes out per row.  Rows that cannot use 16-byte accesses (K not a
+// multiple of 8, unaligned base/stride, or K > 16384) take a strided path that re-reads
+// the row from L2.
+//
+// Arithmetic follows the reference's torch path exactly:
+//   dynamic_quant   flashnn/quant_gemm.py:53-57  (two roundings to the input type)
+//   rmsnorm_dquant  flashnn/norm.py:45-60        (fp32 throughout)
+#include "fnn_common.h"
+
+#pragma clang fp contract(off)
+
+namespace fnn {
+
+constexpr int kRowThreads = 256;
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float r = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    return r;
+}
+
+__device__ __forceinline__ double block_sum(double v, double* red) {
+    v = wave_sum(v);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    double r = (red[0] + red[1]) + (red[2] + red[3]);
+    __syncthreads();
+    return r;
+}
+
+// q = round_half_even(round_DT(x / s)) with x/s an IEEE fp32 division.
+template <int DT> __device__ __forceinline__ int quant_in_dtype(float x, float s) {
+    float t = x / s;
+    float th = bits_to_f32<DT>(f32_to_bits<DT>(t));
+    return (int)rintf(th);
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (uint32_t)(a & 0xFF) | ((uint32_t)(b & 0xFF) << 8) | ((uint32_t)(c & 0xFF) << 16) |
+           ((uint32_t)(d & 0xFF) << 24);
+}
+
+// ------------------------------------------------------------------ dynamic quant
+template <int DT, int NV>
+__global__ __launch_bounds__(kRowThreads) void dynamic_quant_vec_kernel(
+    int8_t* __restrict__ q, uint16_t* __restrict__ scale, const uint16_t* __restrict__ x, int K,
+    int64_t ldx, int64_t ldq) {
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const v4u* xr = (const v4u*)(x + row * ldx);
+    const int nvec = K >> 3;
+    v4u v[NV];
+    uint32_t amax = 0;  // max of |x| taken on the bit patterns (monotonic for finite values)
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int idx = threadIdx.x + i * kRowThreads;
+        v[i] = idx < nvec ? xr[idx] : v4u{0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t w = v[i][j] & 0x7FFF7FFFu;
+            amax = max(amax, max(w & 0xFFFFu, w >> 16));
+        }
+    }
+    const float mx = block_max(bits_to_f32<DT>(amax), red);
+    const uint32_t sbits = f32_to_bits<DT>(mx / 127.0f);
+    const float s = bits_to_f32<DT>(sbits);
+    if (threadIdx.x == 0) scale[row] = (uint16_t)(DT == FNN_F16 ? sbits : f32_to_f16_bits(s));
+    v2u* qr = (v2u*)(q + row * ldq);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int idx = threadIdx.x + i * kRowThreads;
+        if (idx < nvec) {
+            int o[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                o[2 * j] = s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(v[i][j] & 0xFFFFu), s);
+                o[2 * j + 1] = s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(v[i][j] >> 16), s);
+            }
+            qr[idx] = v2u{pack4(o[0], o[1], o[2], o[3]), pack4(o[4], o[5], o[6], o[7])};
+        }
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kRowThreads) void dynamic_quant_any_kernel(
+    int8_t* __restrict__ q, uint16_t* __restrict__ scale, const uint16_t* __restrict__ x, int K,
+    int64_t ldx, int64_t ldq) {
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = x + row * ldx;
+    uint32_t amax = 0;
+    for (int k = threadIdx.x; k < K; k += kRowThreads) amax = max(amax, (uint32_t)(xr[k] & 0x7FFFu));
+    const float mx = block_max(bits_to_f32<DT>(amax), red);
+    const uint32_t sbits = f32_to_bits<DT>(mx / 127.0f);
+    const float s = bits_to_f32<DT>(sbits);
+    if (threadIdx.x == 0) scale[row] = (uint16_t)(DT == FNN_F16 ? sbits : f32_to_f16_bits(s));
+    int8_t* qr = q + row * ldq;
+    for (int k = threadIdx.x; k < K; k += kRowThreads)
+        qr[k] = (int8_t)(s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(xr[k]), s));
+}
+
+// ---------------------------------------------------------------- rmsnorm + quant
+__device__ __forceinline__ int quant_clamped(float n, float s) {
+    float r = rintf(n / s);
+    r = fminf(fmaxf(r, -128.f), 127.f);
+    return s == 0.f ? 0 : (int)r;
+}
+
+template <int DT, int NV>
+__global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_vec_kernel(
+    int8_t* __restrict__ q, uint16_t* __restrict__ scale, const uint16_t* __restrict__ x,
+    const void* __restrict__ gamma, int gamma_dtype, float eps, int K, int64_t ldx, int64_t ldq) {
+    __shared__ double redd[4];
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const v4u* xr = (const v4u*)(x + row * ldx);
+    const int nvec = K >> 3;
+    float n[NV][8];
+    double ssq = 0.0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int idx = threadIdx.x + i * kRowThreads;
+        const v4u v = idx < nvec ? xr[idx] : v4u{0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            n[i][2 * j] = bits_to_f32<DT>(v[j] & 0xFFFFu);
+            n[i][2 * j + 1] = bits_to_f32<DT>(v[j] >> 16);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ssq += (double)(n[i][j] * n[i][j]);  // x*x is exact in fp32
+    }
+    const float sum = (float)block_sum(ssq, redd);
+    const float mean = sum / (float)K;
+    const float rs = 1.0f / sqrtf(mean + eps);
+    float mx = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int idx = threadIdx.x + i * kRowThreads;
+        if (idx < nvec) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float g = load_as_f32(gamma, (int64_t)idx * 8 + j, gamma_dtype);
+                n[i][j] = (n[i][j] * rs) * g;
+                mx = fmaxf(mx, fabsf(n[i][j]));
+            }
+        }
+    }
+    mx = block_max(mx, red);
+    const float s = mx / 127.0f;
+    if (threadIdx.x == 0) scale[row] = (uint16_t)f32_to_bits<DT>(s);
+    v2u* qr = (v2u*)(q + row * ldq);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int idx = threadIdx.x + i * kRowThreads;
+        if (idx < nvec) {
+            int o[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = quant_clamped(n[i][j], s);
+            qr[idx] = v2u{pack4(o[0], o[1], o[2], o[3]), pack4(o[4], o[5], o[6], o[7])};
+        }
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_any_kernel(
+    int8_t* __restrict__ q, uint16_t* __restrict__ scale, const uint16_t* __restrict__ x,
+    const void* __restrict__ gamma, int gamma_dtype, float eps, int K, int64_t ldx, int64_t ldq) {
+    __shared__ double redd[4];
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = x + row * ldx;
+    double ssq = 0.0;
+    for (int k = threadIdx.x; k < K; k += kRowThreads) {
+        const float v = bits_to_f32<DT>(xr[k]);
+        ssq += (double)(v * v);
+    }
+    const float sum = (float)block_sum(ssq, redd);
+    const float mean = sum / (float)K;
+    const float rs = 1.0f / sqrtf(mean + eps);
+    float mx = 0.f;
+    for (int k = threadIdx.x; k < K; k += kRowThreads) {
+        const float nv = (bits_to_f32<DT>(xr[k]) * rs) * load_as_f32(gamma, k, gamma_dtype);
+        mx = fmaxf(mx, fabsf(nv));
+    }
+    mx = block_max(mx, red);
+    const float s = mx / 127.0f;
+    if (threadIdx.x == 0) scale[row] = (uint16_t)f32_to_bits<DT>(s);
+    int8_t* qr = q + row * ldq;
+    for (int k = threadIdx.x; k < K; k += kRowThreads) {
+        const float nv = (bits_to_f32<DT>(xr[k]) * rs) * load_as_f32(gamma, k, gamma_dtype);
+        qr[k] = (int8_t)quant_clamped(nv, s);
+    }
+}
+
+// --------------------------------------------------------------------- launchers
+static bool vec_ok(const void* x, const void* q, int64_t K, int64_t ldx, int64_t ldq) {
+    return K % 8 == 0 && K <= 8 * kRowThreads * 8 && ldx % 8 == 0 && ldq % 8 == 0 &&
+           ((uintptr_t)x % 16) == 0 && ((uintptr_t)q % 8) == 0;
+}
+
+template <int DT>
+static void launch_dq(int8_t* q, uint16_t* scale, const uint16_t* x, int64_t M, int K, int64_t ldx,
+                      int64_t ldq, hipStream_t st) {
+    const dim3 grid((unsigned)M), block(kRowThreads);
+    if (vec_ok(x, q, K, ldx, ldq)) {
+        const int nv = (K / 8 + kRowThreads - 1) / kRowThreads;
+        if (nv <= 1) dynamic_quant_vec_kernel<DT, 1><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
+        else if (nv <= 2) dynamic_quant_vec_kernel<DT, 2><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
+        else if (nv <= 4) dynamic_quant_vec_kernel<DT, 4><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
+        else dynamic_quant_vec_kernel<DT, 8><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
+    } else {
+        dynamic_quant_any_kernel<DT><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
+    }
+}
+
+template <int DT>
+static void launch_rq(int8_t* q, uint16_t* scale, const uint16_t* x, const void* gamma, int gdt,
+                      float eps, int64_t M, int K, int64_t ldx, int64_t ldq, hipStream_t st) {
+    const dim3 grid((unsigned)M), block(kRowThreads);
+    if (vec_ok(x, q, K, ldx, ldq)) {
+        const int nv = (K / 8 + kRowThreads - 1) / kRowThreads;
+        if (nv <= 1) rmsnorm_dquant_vec_kernel<DT, 1><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
+        else if (nv <= 2) rmsnorm_dquant_vec_kernel<DT, 2><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
+        else if (nv <= 4) rmsnorm_dquant_vec_kernel<DT, 4><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
+        else rmsnorm_dquant_vec_kernel<DT, 8><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
+    } else {
+        rmsnorm_dquant_any_kernel<DT><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
+    }
+}
+
+}  // namespace fnn
+
+using namespace fnn;
+
+static int check_rows(const char* fn, const void* q, const void* scale, const void* x, int64_t M,
+                      int64_t K, int64_t ldx, int64_t ldq, int x_dtype) {
+    if (!q || !scale || !x) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
+    if (M < 0 || K <= 0 || ldx < K || ldq < K) {
+        set_error("%s: bad shape M=%lld K=%lld ldx=%lld ldq=%lld", fn, (long long)M, (long long)K,
+                  (long long)ldx, (long long)ldq);
+        return FNN_ERR_ARG;
+    }
+    if (!is16(x_dtype)) { set_error("%s: input type must be fp16 or bf16", fn); return FNN_ERR_UNSUPPORTED; }
+    if (M > 0x7FFFFFFFLL || K > 0x7FFFFFFFLL) { set_error("%s: shape too large", fn); return FNN_ERR_UNSUPPORTED; }
+    return FNN_OK;
+}
+
+extern "C" int fnn_dynamic_quant(void* q, void* scale, const void* x, int64_t M, int64_t K,
+                                 int64_t ldx, int64_t ldq, int x_dtype, void* stream) {
+    int rc = check_rows("fnn_dynamic_quant", q, scale, x, M, K, ldx, ldq, x_dtype);
+    if (rc != FNN_OK) return rc;
+    if (M == 0) return FNN_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (x_dtype == FNN_F16)
+        launch_dq<FNN_F16>((int8_t*)q, (uint16_t*)scale, (const uint16_t*)x, M, (int)K, ldx, ldq, st);
+    else
+        launch_dq<FNN_BF16>((int8_t*)q, (uint16_t*)scale, (const uint16_t*)x, M, (int)K, ldx, ldq, st);
+    return check_launch("fnn_dynamic_quant");
+}
+
+extern "C" int fnn_rmsnorm_dquant(void* q, void* scale, const void* x, const void* gamma, float eps,
+                                  int64_t M, int64_t K, int64_t ldx, int64_t ldq, int x_dtype,
+                                  int gamma_dtype, void* stream) {
+    int rc = check_rows("fnn_rmsnorm_dquant", q, scale, x, M, K, ldx, ldq, x_dtype);
+    if (rc != FNN_OK) return rc;
+    if (!gamma) { set_error("fnn_rmsnorm_dquant: null gamma"); return FNN_ERR_ARG; }
+    if (!isflt(gamma_dtype)) { set_error("fnn_rmsnorm_dquant: bad gamma type"); return FNN_ERR_UNSUPPORTED; }
+    if (M == 0) return FNN_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (x_dtype == FNN_F16)
+        launch_rq<FNN_F16>((int8_t*)q, (uint16_t*)scale, (const uint16_t*)x, gamma, gamma_dtype, eps, M, (int)K, ldx, ldq, st);
+    else
+        launch_rq<FNN_BF16>((int8_t*)q, (uint16_t*)scale, (const uint16_t*)x, gamma, gamma_dtype, eps, M, (int)K, ldx, ldq, st);
+    return check_launch("fnn_rmsnorm_dquant");
+}

@@ -1,0 +1,148 @@
+"""Launcher functions with the shape of the reference's Triton launchers: the caller
+allocates the outputs, the launcher fills them on the current stream.
+
+Each one replaces the reference function named in its docstring and forwards to the C ABI
+of libflashnn_hip.so.  The argument checks raise the same exception types with the same
+messages as the reference so callers and tests behave identically.
+"""
+import torch
+
+from . import _lib
+
+
+def hip_dynamic_quantize(out, input, scale):
+    """Replaces triton_dynamic_quantize (flashnn/triton_kernels/dynamic_quant.py:73-97)."""
+    assert input.is_contiguous(), "input must be contiguous"
+    assert input.dim() == 2 and out.shape == input.shape and out.dtype == torch.int8
+    assert scale.dtype == torch.float16 and scale.numel() == input.size(0)
+    assert out.is_contiguous() and scale.is_contiguous()
+    _lib.require_gpu(out, input, scale)
+    lib = _lib.load()
+    M, K = input.shape
+    _lib.check(lib.fnn_dynamic_quant(_lib.ptr(out), _lib.ptr(scale), _lib.ptr(input), M, K,
+                                     input.stride(0) if M > 1 else K, out.stride(0) if M > 1 else K,
+                                     _lib.dtype_code(input.dtype), _lib.current_stream(input.device)))
+    return out, scale
+
+
+def hip_rmsnorm_dquant_forward(x, weight, eps):
+    """Replaces triton_rmsnorm_dquant_forward (flashnn/triton_kernels/rms_norm_dquant.py:80-96)."""
+    _lib.require_gpu(x, weight)
+    lib = _lib.load()
+    y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    x_arg = x.reshape(-1, x.shape[-1])
+    if not x_arg.is_contiguous():
+        x_arg = x_arg.contiguous()
+    M, N = x_arg.shape
+    scale = torch.empty((M,), dtype=x.dtype, device=x.device)
+    w = weight.detach()
+    if not w.is_contiguous():
+        w = w.contiguous()
+    assert w.numel() == N, "weight must have one entry per channel"
+    _lib.check(lib.fnn_rmsnorm_dquant(_lib.ptr(y), _lib.ptr(scale), _lib.ptr(x_arg), _lib.ptr(w),
+                                      float(eps), M, N, N, N, _lib.dtype_code(x.dtype),
+                                      _lib.dtype_code(w.dtype), _lib.current_stream(x.device)))
+    return y, scale.reshape(x.shape[:-1])
+
+
+def _flat_scale(t, n, what):
+    t = torch.squeeze(t)
+    if t.dim() == 0:
+        t = t.reshape(1)
+    assert t.dim() == 1 and t.numel() == n, f"{what} must have {n} entries"
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col):
+    """Replaces triton_gemm_a8w8_forward (flashnn/triton_kernels/gemm_a8w8.py:182-221).
+
+    Unlike the Triton launcher the scale type need not equal the output type: fp16, bf16 and
+    fp32 scales are accepted in any combination."""
+    assert a.dtype == torch.int8 and b.dtype == torch.int8, "Matrix A/B must be int8 type"
+    assert a.is_contiguous(), "Matrix A must be contiguous"
+    assert out.dtype == torch.float16 or out.dtype == torch.bfloat16, \
+        "Output type must be float16 or bfloat16"
+    assert a.shape[1] == b.shape[1], "Matrix B must be transposed"
+    _lib.require_gpu(out, a, b, alpha_row, alpha_col)
+    lib = _lib.load()
+    M, K = a.shape
+    N = b.shape[0]
+    assert out.shape == (M, N) and out.stride(1) == 1
+    if b.stride(1) != 1:
+        b = b.contiguous()
+    ar = _flat_scale(alpha_row, M, "alpha_row")
+    ac = _flat_scale(alpha_col, N, "alpha_col")
+    _lib.check(lib.fnn_gemm_a8w8(_lib.ptr(out), _lib.ptr(a), _lib.ptr(b), _lib.ptr(ar), _lib.ptr(ac),
+                                 M, N, K, a.stride(0) if M > 1 else K, b.stride(0) if N > 1 else K,
+                                 out.stride(0) if M > 1 else N, _lib.dtype_code(out.dtype),
+                                 _lib.dtype_code(ar.dtype), _lib.dtype_code(ac.dtype),
+                                 _lib.current_stream(a.device)))
+    return out
+
+
+def hip_gemm_a8w8_int32(a, b):
+    """Raw int32 accumulators of the A8W8 contraction (no reference launcher; parity hook)."""
+    assert a.dtype == torch.int8 and b.dtype == torch.int8, "Matrix A/B must be int8 type"
+    assert a.is_contiguous() and b.is_contiguous() and a.shape[1] == b.shape[1]
+    _lib.require_gpu(a, b)
+    lib = _lib.load()
+    M, K = a.shape
+    N = b.shape[0]
+    acc = torch.empty((M, N), dtype=torch.int32, device=a.device)
+    _lib.check(lib.fnn_gemm_a8w8_i32(_lib.ptr(acc), _lib.ptr(a), _lib.ptr(b), M, N, K, K, K, N,
+                                     _lib.current_stream(a.device)))
+    return acc
+
+
+def _weight_only(fn_name, out, act, quant_w, scale_w, bias, zero_points, n_out):
+    assert quant_w.dtype == torch.int8, "Weight must be int8 type"
+    assert act.is_contiguous(), "Activation must be contiguous"
+    assert quant_w.is_contiguous(), "Weight must be contiguous"
+    assert act.shape[1] == quant_w.shape[1], "Matrix B must be transposed"
+    _lib.require_gpu(out, act, quant_w, scale_w, bias, zero_points)
+    lib = _lib.load()
+    scale_w = scale_w.squeeze()
+    M, K = act.shape
+    N = n_out
+    assert out.shape == (M, N) and out.stride(1) == 1
+    if scale_w.dim() <= 1:
+        group = 0
+        scale_w = scale_w.reshape(-1)
+        assert scale_w.numel() == N
+    else:
+        assert scale_w.dim() == 2 and scale_w.shape[1] == N
+        group = int(K / scale_w.shape[0])
+        assert group > 0, "k_per_scale should greater than 0"
+        assert group * scale_w.shape[0] == K, "K must be a multiple of the scale rows"
+    scale_w = scale_w.contiguous()
+    zp = None
+    if zero_points is not None:
+        zp = zero_points.squeeze().reshape(scale_w.shape).contiguous()
+        if not zp.is_floating_point():
+            zp = zp.to(scale_w.dtype)
+    if bias is not None:
+        bias = bias.reshape(-1).contiguous()
+        assert bias.numel() == N
+    fn = getattr(lib, fn_name)
+    _lib.check(fn(_lib.ptr(out), _lib.ptr(act), _lib.ptr(quant_w), _lib.ptr(scale_w), _lib.ptr(bias),
+                  _lib.ptr(zp), M, N, K, act.stride(0) if M > 1 else K, K,
+                  out.stride(0) if M > 1 else N, group, _lib.dtype_code(act.dtype),
+                  _lib.dtype_code(out.dtype), _lib.dtype_code(scale_w.dtype),
+                  _lib.dtype_code(zp.dtype) if zp is not None else 0,
+                  _lib.dtype_code(bias.dtype) if bias is not None else 0,
+                  _lib.current_stream(act.device)))
+    return out
+
+
+def hip_gemm_a16w8_forward(out, act, quant_w, scale_w, bias=None, zero_points=None):
+    """Replaces triton_gemm_a16w8_forward (flashnn/triton_kernels/gemm_a16w8.py:275-338).
+    `out` need not be zeroed."""
+    return _weight_only("fnn_gemm_a16w8", out, act, quant_w, scale_w, bias, zero_points,
+                        quant_w.shape[0])
+
+
+def hip_gemm_a16w4_forward(out, act, quant_w, scale_w, bias=None, zero_points=None):
+    """Replaces triton_gemm_a16w4_forward (flashnn/triton_kernels/gemm_a16w4.py:336-406).
+    quant_w is [N/2, K] with channel 2j in the low and 2j+1 in the high nibble of row j."""
+    return _weight_only("fnn_gemm_a16w4", out, act, quant_w, scale_w, bias, zero_points,
+                        quant_w.shape[0] * 2)

@@ -1,0 +1,61 @@
+"""Seeded synthetic inputs for the benchmark configurations (CPU tensors; callers move
+them to the GPU).  Shapes and distributions follow the configurations the benchmark and
+the parity tests are quoted on."""
+import math
+
+import torch
+
+
+def _gen(seed):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    return g
+
+
+def activations(M, K, dtype, seed=0, outlier_frac=0.0, outlier_gain=20.0):
+    """~N(0,1) activations; optionally a fixed random subset of channels scaled up."""
+    g = _gen(seed)
+    x = torch.randn(M, K, generator=g, dtype=torch.float32)
+    if outlier_frac > 0:
+        n_out = math.ceil(outlier_frac * K)
+        cols = torch.randperm(K, generator=g)[:n_out]
+        x[:, cols] *= outlier_gain
+    return x.to(dtype)
+
+
+def int8_weights(N, K, seed=1):
+    """int8 weights uniform in [-127, 127] and per-output-channel fp32 scales U(1e-3, 1e-2)."""
+    g = _gen(seed)
+    w = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    s = torch.empty(N, dtype=torch.float32).uniform_(1e-3, 1e-2, generator=g)
+    return w, s
+
+
+def int4_group_weights(N, K, group, scale_dtype=torch.float16, seed=2):
+    """uint4 weights with per-group scales and uint4 zero points, expressed through the
+    operator's signed-nibble layout: returns (packed [N/2,K] int8, scales [K/group,N],
+    zero_points [K/group,N] as scale_dtype, u4 [N,K] uint8, zp_u4 [K/group,N] uint8).
+
+    A uint4 value u with zero point z equals the signed nibble (u - 8) with zero point
+    (z - 8): (u - 8) - (z - 8) = u - z.  Row j of the packed matrix holds channel 2j in the
+    low nibble and channel 2j+1 in the high nibble."""
+    g = _gen(seed)
+    u = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8)
+    zp = torch.randint(0, 16, (K // group, N), generator=g, dtype=torch.uint8)
+    s = torch.empty(K // group, N, dtype=torch.float32).uniform_(1e-3, 1e-2, generator=g).to(scale_dtype)
+    nib = (u.to(torch.int16) - 8) & 0xF
+    packed = (nib[0::2] | (nib[1::2] << 4)).to(torch.uint8).view(torch.int8).contiguous()
+    zp_ref = (zp.to(torch.float32) - 8).to(scale_dtype)
+    return packed, s, zp_ref, u, zp
+
+
+def rmsnorm_gamma(K, seed=3):
+    g = _gen(seed)
+    return torch.empty(K, dtype=torch.float32).uniform_(0.5, 1.5, generator=g)
+
+
+# (K, N) of the Llama-7B-like linear layers used for the A8W8 prefill configuration
+A8W8_PREFILL_SHAPES = {"qkv": (4096, 12288), "o": (4096, 4096), "gate_up": (4096, 22016),
+                       "down": (11008, 4096)}
+A16W8_DECODE_SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096)]
+A16W4_SHAPE = (8192, 28672)

