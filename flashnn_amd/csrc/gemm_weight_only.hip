@@ -92,15 +92,19 @@ __device__ __forceinline__ void convert_w8(const v4u w, v4u& s0, v4u& s1) {
 // order (0,2)(1,3)(4,6)(5,7); values are c + (v + 8), c = 1024 (fp16) / 128 (bf16).
 template <int ADT>
 __device__ __forceinline__ void convert_w4(const v4u w, v4u& e0, v4u& e1, v4u& o0, v4u& o1) {
-    constexpr uint32_t mag = ADT == FNN_F16 ? 0x64006400u : 0x43004300u;
+    // (x & 0x000F000F) ^ c with c = exponent bits | 0x0008 per half: the xor both flips the
+    // nibble's sign bit (two's complement -> offset by 8) and sets the exponent, because the two
+    // bit sets are disjoint.  One 3-input bit operation per pair of weights.
+    constexpr uint32_t msk = 0x000F000Fu;
+    constexpr uint32_t cst = (ADT == FNN_F16 ? 0x64006400u : 0x43004300u) ^ 0x00080008u;
     uint32_t e[8], o[8];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        const uint32_t x = w[q] ^ 0x88888888u;
-        e[2 * q] = (x & 0x000F000Fu) | mag;
-        e[2 * q + 1] = ((x >> 8) & 0x000F000Fu) | mag;
-        o[2 * q] = ((x >> 4) & 0x000F000Fu) | mag;
-        o[2 * q + 1] = ((x >> 12) & 0x000F000Fu) | mag;
+        const uint32_t x = w[q];
+        e[2 * q] = (x & msk) ^ cst;
+        e[2 * q + 1] = ((x >> 8) & msk) ^ cst;
+        o[2 * q] = ((x >> 4) & msk) ^ cst;
+        o[2 * q + 1] = ((x >> 12) & msk) ^ cst;
     }
     e0 = v4u{e[0], e[1], e[2], e[3]};
     e1 = v4u{e[4], e[5], e[6], e[7]};
@@ -285,6 +289,423 @@ __global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoA
     }
 }
 
+
+// ------------------------------------------------------------------ decode kernel (M <= 8)
+// A 256-thread workgroup (4 waves, splitting K) owns 8 weight rows (8 channels for int8,
+// 16 for packed int4): with N = 28672 int4 channels that is 1792 workgroups, exactly 7 per CU.
+// The 16 rows of the MFMA "A" operand are used twice: lane row i holds weight row (i & 7) for
+// the first (i < 8) or second (i >= 8) 16-byte half of a 32-byte K segment, so one load
+// instruction of a wave covers 8 rows x 128 contiguous bytes and every loaded byte is used.
+// The 16 columns of the "B" operand are used the same way: column j holds activation row
+// (j & 7) for the first or second half.  Of the 16x16 result only the two 8x8 blocks on
+// the diagonal (same half on both sides) are meaningful; they are added at the end.
+// Scales and zero points of the tile (all K-groups) and, when they fit, the activation rows
+// are staged in LDS once per workgroup; weights stream through registers kPF loads ahead.
+constexpr int kDecWaves = 4;
+
+template <int WBITS, int ADT, bool GROUPED, bool ACT_LDS>
+__global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_kernel(const WoArgs p) {
+    typedef MfmaT<ADT> MT;
+    constexpr int NH = WBITS == 4 ? 2 : 1;
+    constexpr int NC = 8 * NH;                 // channels per tile
+    constexpr float c_off = WBITS == 4 ? (ADT == FNN_F16 ? 1024.f + 8.f : 128.f + 8.f)
+                                       : (ADT == FNN_F16 ? 1024.f + 128.f : 128.f);
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int li = lane & 15;
+    const int lg = lane >> 4;
+    const int half = li >> 3;     // which 16-byte half of the lane group's 32-byte K segment
+    const int r8 = li & 7;        // weight row (A side) / activation row (B side)
+
+    const int wrows = WBITS == 4 ? p.N / 2 : p.N;
+    const int tiles = (wrows + 7) / 8;
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (tile >= tiles) return;
+    const int row0 = tile * 8;
+    const int n0 = row0 * NH;
+
+    const int steps = p.K / 128;
+    const int s_begin = (int)((int64_t)steps * wave / kDecWaves);
+    const int s_end = (int)((int64_t)steps * (wave + 1) / kDecWaves);
+    const int ngroups = GROUPED ? p.K / p.group : 1;
+
+    // LDS carve-up: [scale ngroups*NC f32][zoff ngroups*NC f32][red 4*NH*4*64 f32][acts]
+    float* s_lds = (float*)smem;
+    float* z_lds = s_lds + ngroups * NC;
+    float* red = z_lds + ngroups * NC;
+    uint16_t* a_lds = (uint16_t*)(red + kDecWaves * NH * 4 * 64);
+    const int a_stride = p.K + 32;   // elements; the pad staggers the rows over the banks
+
+    // ---- issue the first weight loads, then fill LDS while they are in flight ----
+    const char* wptr = (const char*)p.qw + (int64_t)min(row0 + r8, wrows - 1) * p.ldw + lg * 32 + half * 16;
+    auto load_w = [&](int step) -> v4u {
+        const int s = min(step, s_end - 1);
+        return __builtin_nontemporal_load((const v4u*)(wptr + (int64_t)s * 128));
+    };
+    v4u wq[kPF];
+    if (s_begin < s_end) {
+#pragma unroll
+        for (int i = 0; i < kPF; ++i) wq[i] = load_w(s_begin + i);
+    }
+
+    for (int e = threadIdx.x; e < ngroups * NC; e += kDecWaves * 64) {
+        const int g = e / NC, c = e % NC;
+        const int64_t idx = (int64_t)g * p.N + min(n0 + c, p.N - 1);
+        const float sc = load_as_f32(p.scale, idx, p.scale_dtype);
+        const float z = p.zp ? load_as_f32(p.zp, idx, p.zp_dtype) : 0.f;
+        s_lds[e] = sc;
+        z_lds[e] = sc * (c_off + z);
+    }
+    if constexpr (ACT_LDS) {
+        const int chunks = p.K / 8;
+        for (int e = threadIdx.x; e < p.M * chunks; e += kDecWaves * 64) {
+            const int m = e / chunks, c = e % chunks;
+            v4u v = *(const v4u*)((const uint16_t*)p.act + (int64_t)m * p.lda + c * 8);
+            if constexpr (WBITS == 4) v = perm_act_w4(v);
+            *(v4u*)(a_lds + m * a_stride + c * 8) = v;
+        }
+    }
+    __syncthreads();
+
+    // activation operand of this lane for K step `step`, sub-slot `slot` (8 values)
+    const bool avalid = r8 < p.M;
+    const int koff = lg * 32 + half * 16;
+    const uint16_t* aptr = (const uint16_t*)p.act + (int64_t)min(r8, p.M - 1) * p.lda + koff;
+    auto load_a_gbl = [&](int step, int slot) -> v4u {
+        const int s = min(step, s_end - 1);
+        return avalid ? *(const v4u*)(aptr + (int64_t)s * 128 + slot * 8) : v4u{0, 0, 0, 0};
+    };
+    auto load_a_lds = [&](int step, int slot) -> v4u {
+        return avalid ? *(const v4u*)(a_lds + r8 * a_stride + step * 128 + koff + slot * 8) : v4u{0, 0, 0, 0};
+    };
+
+    v4f outv[NH], accg[NH], asum = v4f{0, 0, 0, 0};
+#pragma unroll
+    for (int h = 0; h < NH; ++h) { outv[h] = v4f{0, 0, 0, 0}; accg[h] = v4f{0, 0, 0, 0}; }
+
+    // result register r of this lane is weight row (4*lg + r) & 7: channels NH*(4*(lg&1)+r)+h
+    auto fold = [&](int grp) {
+        const float* sp = s_lds + grp * NC + NH * 4 * (lg & 1);
+        const float* zp = z_lds + grp * NC + NH * 4 * (lg & 1);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                outv[h][r] += sp[NH * r + h] * accg[h][r] - zp[NH * r + h] * asum[r];
+                accg[h][r] = 0.f;
+            }
+        asum = v4f{0, 0, 0, 0};
+    };
+
+    if (s_begin < s_end) {
+        v4u aq[kPFA][2];
+        if constexpr (!ACT_LDS) {
+#pragma unroll
+            for (int i = 0; i < kPFA; ++i) {
+                aq[i][0] = load_a_gbl(s_begin + i, 0);
+                aq[i][1] = load_a_gbl(s_begin + i, 1);
+            }
+        }
+        const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+        const int gsteps = GROUPED ? p.group / 128 : 1;
+        for (int sb = s_begin; sb < s_end; sb += kPF) {
+#pragma unroll
+            for (int i = 0; i < kPF; ++i) {
+                const int step = sb + i;
+                if (step < s_end) {
+                    const v4u w = wq[i];
+                    wq[i] = load_w(step + kPF);
+                    v4u a0, a1;
+                    if constexpr (ACT_LDS) {
+                        a0 = load_a_lds(step, 0);
+                        a1 = load_a_lds(step, 1);
+                    } else {
+                        a0 = aq[i % kPFA][0];
+                        a1 = aq[i % kPFA][1];
+                        aq[i % kPFA][0] = load_a_gbl(step + kPFA, 0);
+                        aq[i % kPFA][1] = load_a_gbl(step + kPFA, 1);
+                        if constexpr (WBITS == 4) { a0 = perm_act_w4(a0); a1 = perm_act_w4(a1); }
+                    }
+                    if constexpr (WBITS == 4) {
+                        v4u e0, e1, o0, o1;
+                        convert_w4<ADT>(w, e0, e1, o0, o1);
+                        accg[0] = MT::mma(e0, a0, accg[0]);
+                        accg[1] = MT::mma(o0, a0, accg[1]);
+                        asum = MT::mma(ones, a0, asum);
+                        accg[0] = MT::mma(e1, a1, accg[0]);
+                        accg[1] = MT::mma(o1, a1, accg[1]);
+                        asum = MT::mma(ones, a1, asum);
+                    } else {
+                        v4u s0, s1;
+                        convert_w8<ADT>(w, s0, s1);
+                        accg[0] = MT::mma(s0, a0, accg[0]);
+                        asum = MT::mma(ones, a0, asum);
+                        accg[0] = MT::mma(s1, a1, accg[0]);
+                        asum = MT::mma(ones, a1, asum);
+                    }
+                    if constexpr (GROUPED) {
+                        if ((step + 1) % gsteps == 0 || step + 1 == s_end) fold(step / gsteps);
+                    }
+                }
+            }
+        }
+        if constexpr (!GROUPED) fold(0);
+    }
+
+    // ---- add the partial tiles of the 4 waves and the two diagonal blocks ----
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[((wave * NH + h) * 4 + r) * 64 + lane] = outv[h][r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < p.M * NC; e += kDecWaves * 64) {
+        const int m = e / NC, c = e % NC;
+        const int row = c / NH, h = c % NH;          // weight row 0..7 of the tile
+        const int r = row & 3;
+        const int lane1 = m + 16 * (row >> 2);              // result row `row`,     column m
+        const int lane2 = (m + 8) + 16 * ((row + 8) >> 2);  // result row `row`+8,   column m+8
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < kDecWaves; ++w)
+            v += red[((w * NH + h) * 4 + r) * 64 + lane1] + red[((w * NH + h) * 4 + r) * 64 + lane2];
+        const int n = n0 + c;
+        if (n < p.N) {
+            if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+            store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
+        }
+    }
+}
+
+
+// --------------------------------------------- decode kernel, activations staged in LDS
+// Same tiling as gemm_wo_decode_kernel (8 weight rows per 256-thread workgroup, the two
+// diagonal 8x8 blocks of the 16x16 MFMA result) with the per-step VALU work cut down:
+//   * G128 (group size 128 = one 128-byte K step): the 8 result columns of a block are
+//     shared by MP activation rows and 8/MP consecutive K-groups.  Column gslot*MP + m gets
+//     the activations of row m only in the steps of group slot gslot (a zeroed LDS
+//     region otherwise), so 8/MP groups accumulate side by side and the scales are
+//     applied once per 8/MP steps instead of every step;
+//   * sign flip, nibble mask and exponent insertion are one 3-input bit operation;
+//   * the wave index is made scalar so the K loop is scalar control flow, the weight
+//     address is a scalar base plus a per-lane 32-bit offset.
+template <int WBITS, int ADT, bool G128, int MP, int CH, bool FULL>
+__global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(const WoArgs p) {
+    typedef MfmaT<ADT> MT;
+    constexpr int NH = WBITS == 4 ? 2 : 1;
+    constexpr int NC = 8 * NH;
+    constexpr int GS = G128 ? 8 / MP : 1;       // K-groups accumulated side by side
+    constexpr int UN = 8;                        // weight loads in flight per lane
+    // CH = steps per straight-line chunk; FULL = every wave owns whole chunks (no guards)
+    constexpr int ZERO_BYTES = CH * 256 + 32;
+    constexpr float c_off = WBITS == 4 ? (ADT == FNN_F16 ? 1024.f + 8.f : 128.f + 8.f)
+                                       : (ADT == FNN_F16 ? 1024.f + 128.f : 128.f);
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int li = lane & 15;
+    const int lg = lane >> 4;
+    const int half = li >> 3;
+    const int j7 = li & 7;
+
+    const int wrows = WBITS == 4 ? p.N / 2 : p.N;
+    const int tiles = (wrows + 7) / 8;
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (tile >= tiles) return;
+    const int row0 = tile * 8;
+    const int n0 = row0 * NH;
+
+    const int steps = p.K / 128;
+    // waves take whole blocks of 8 steps so that group slots line up with step indices
+    const int nblk = (steps + 7) / 8;
+    const int s_begin = (nblk * wave / kDecWaves) * 8;
+    const int s_end = min((nblk * (wave + 1) / kDecWaves) * 8, steps);
+    const int ngroups = G128 ? steps : 1;
+
+    // LDS: [zeros][scale ngroups*NC f32][zoff ngroups*NC f32][red 4*NH*4*64 f32][acts]
+    float* s_lds = (float*)(smem + ZERO_BYTES);
+    float* z_lds = s_lds + ngroups * NC;
+    float* red = z_lds + ngroups * NC;
+    uint16_t* a_lds = (uint16_t*)(red + kDecWaves * NH * 4 * 64);
+    const int a_stride = p.K + 32;
+
+    const int wrow_l = min(row0 + j7, wrows - 1) - row0;
+    const uint32_t w_off = (uint32_t)wrow_l * (uint32_t)p.ldw + lg * 32 + half * 16;
+    const char* w_tile = (const char*)p.qw + (int64_t)row0 * p.ldw;
+    auto load_w = [&](int step) -> v4u {
+        const char* base = w_tile + (int64_t)min(step, s_end - 1) * 128;   // scalar
+        return __builtin_nontemporal_load((const v4u*)(base + w_off));
+    };
+    v4u wq[UN];
+    if (s_begin < s_end) {
+#pragma unroll
+        for (int i = 0; i < UN; ++i) wq[i] = load_w(s_begin + i);
+    }
+
+    for (int e = threadIdx.x; e < ZERO_BYTES / 4; e += kDecWaves * 64) ((uint32_t*)smem)[e] = 0;
+    // Fill LDS in batches: all loads of a batch are issued before the first store, so a batch
+    // costs one memory latency (a load-store loop would pay it once per element).
+    constexpr int NT = kDecWaves * 64;
+    {
+        const int total = ngroups * NC;
+        for (int e0 = 0; e0 < total; e0 += 4 * NT) {
+            float sc[4], z[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int e = e0 + u * NT + threadIdx.x;
+                const int ec = min(e, total - 1);
+                const int64_t idx = (int64_t)(ec / NC) * p.N + min(n0 + ec % NC, p.N - 1);
+                sc[u] = load_as_f32(p.scale, idx, p.scale_dtype);
+                z[u] = p.zp ? load_as_f32(p.zp, idx, p.zp_dtype) : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int e = e0 + u * NT + threadIdx.x;
+                if (e < total) { s_lds[e] = sc[u]; z_lds[e] = sc[u] * (c_off + z[u]); }
+            }
+        }
+    }
+    {
+        const int chunks = p.K / 8;   // 16-byte pieces per activation row
+        for (int m = 0; m < p.M; ++m) {
+            const v4u* src = (const v4u*)((const uint16_t*)p.act + (int64_t)m * p.lda);
+            v4u* dst = (v4u*)(a_lds + m * a_stride);
+            for (int c0 = 0; c0 < chunks; c0 += 4 * NT) {
+                v4u v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = src[min(c0 + u * NT + (int)threadIdx.x, chunks - 1)];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int c = c0 + u * NT + threadIdx.x;
+                    if (c < chunks) dst[c] = WBITS == 4 ? perm_act_w4(v[u]) : v[u];
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // B-operand source of this lane: column j7 = gslot*MP + m
+    const int m_col = G128 ? (j7 % MP) : j7;
+    const int gslot = G128 ? (j7 / MP) : 0;
+    const bool col_valid = m_col < p.M;
+    bool use[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) use[i] = col_valid && (i % GS) == gslot;
+    const int koff = lg * 32 + half * 16;
+    // byte addresses in LDS; step s adds s*256
+    uint32_t a_real = (uint32_t)((const char*)(a_lds + m_col * a_stride + koff) - smem) + s_begin * 256;
+    const uint32_t a_zero = 0;
+    uint32_t sz_addr = (uint32_t)((const char*)(s_lds + (s_begin + gslot) * (G128 ? NC : 0) + NH * 4 * (lg & 1)) - smem);
+    const uint32_t z_delta = (uint32_t)(ngroups * NC * 4);
+
+    v4f outv[NH], accg[NH], asum;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) { outv[h] = v4f{0, 0, 0, 0}; accg[h] = v4f{0, 0, 0, 0}; }
+    asum = v4f{0, 0, 0, 0};
+    const v4f zero4 = v4f{0, 0, 0, 0};
+
+    auto fold = [&](uint32_t addr) {
+        float sv[NH * 4], zv[NH * 4];
+#pragma unroll
+        for (int q = 0; q < NH; ++q) {
+            const v4f a = *(const v4f*)(smem + addr + q * 16);
+            const v4f b = *(const v4f*)(smem + addr + z_delta + q * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { sv[q * 4 + e] = a[e]; zv[q * 4 + e] = b[e]; }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+                outv[h][r] += sv[NH * r + h] * accg[h][r] - zv[NH * r + h] * asum[r];
+    };
+
+    // The K range of a wave is processed in chunks of CH steps.  A chunk is straight-line code:
+    // UN loads are in flight at its start, steps 0..CH-UN-1 each issue the load UN steps ahead,
+    // so the wait counts are exact and nothing is carried over a loop edge in registers.
+    const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+    for (int sb = s_begin; sb < s_end; sb += CH) {
+        if (sb != s_begin) {
+#pragma unroll
+            for (int i = 0; i < UN; ++i) wq[i] = load_w(sb + i);
+        }
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            const int step = sb + i;
+            if (FULL || step < s_end) {
+                const v4u w = wq[i % UN];
+                const uint32_t aa = (use[i % 8] ? a_real : a_zero) + i * 256;
+                const v4u a0 = *(const v4u*)(smem + aa);
+                const v4u a1 = *(const v4u*)(smem + aa + 16);
+                const bool first = G128 ? (i % GS == 0) : (step == s_begin);
+                if constexpr (WBITS == 4) {
+                    v4u e0, e1, o0, o1;
+                    convert_w4<ADT>(w, e0, e1, o0, o1);
+                    // refill the queue slot only after its old value is dead, so that both live
+                    // in the same registers
+                    if (i + UN < CH) wq[i % UN] = load_w(step + UN);
+                    accg[0] = MT::mma(e0, a0, first ? zero4 : accg[0]);
+                    accg[1] = MT::mma(o0, a0, first ? zero4 : accg[1]);
+                    asum = MT::mma(ones, a0, first ? zero4 : asum);
+                    accg[0] = MT::mma(e1, a1, accg[0]);
+                    accg[1] = MT::mma(o1, a1, accg[1]);
+                    asum = MT::mma(ones, a1, asum);
+                } else {
+                    v4u s0, s1;
+                    convert_w8<ADT>(w, s0, s1);
+                    if (i + UN < CH) wq[i % UN] = load_w(step + UN);
+                    accg[0] = MT::mma(s0, a0, first ? zero4 : accg[0]);
+                    asum = MT::mma(ones, a0, first ? zero4 : asum);
+                    accg[0] = MT::mma(s1, a1, accg[0]);
+                    asum = MT::mma(ones, a1, asum);
+                }
+                if constexpr (G128) {
+                    if (i % GS == GS - 1 || (!FULL && step + 1 == s_end))
+                        fold(sz_addr + (i / GS) * GS * NC * 4);
+                }
+            }
+            // keep every step's refill load inside its step: the scheduler would otherwise
+            // sink the loads to shorten their live ranges and empty the queue
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        a_real += CH * 256;
+        if constexpr (G128) sz_addr += CH * NC * 4;
+    }
+    if constexpr (!G128) {
+        if (s_begin < s_end) fold(sz_addr);
+    }
+
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[((wave * NH + h) * 4 + r) * 64 + lane] = outv[h][r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < p.M * NC; e += kDecWaves * 64) {
+        const int m = e / NC, c = e % NC;
+        const int row = c / NH, h = c % NH;
+        const int r = row & 3;
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < kDecWaves; ++w)
+#pragma unroll
+            for (int gs = 0; gs < GS; ++gs) {
+                const int col = gs * (G128 ? MP : 0) + m;
+                const int lane1 = col + 16 * (row >> 2);
+                const int lane2 = (col + 8) + 16 * ((row + 8) >> 2);
+                v += red[((w * NH + h) * 4 + r) * 64 + lane1] + red[((w * NH + h) * 4 + r) * 64 + lane2];
+            }
+        const int n = n0 + c;
+        if (n < p.N) {
+            if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+            store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ guarded fallback
 template <int WBITS, int ADT>
 __global__ __launch_bounds__(256) void gemm_wo_any_kernel(const WoArgs p) {
@@ -323,6 +744,49 @@ static void launch_stream(WoArgs& p, hipStream_t st) {
 }
 
 template <int WBITS, int ADT>
+static bool launch_decode(WoArgs& p, hipStream_t st) {
+    constexpr int NH = WBITS == 4 ? 2 : 1;
+    if (p.M > 8 || p.K % 128 != 0) return false;
+    if (p.group > 0 && (p.group % 128 != 0)) return false;
+    const int ngroups = p.group > 0 ? p.K / p.group : 1;
+    const size_t fixed = (size_t)ngroups * 8 * NH * 8 + (size_t)kDecWaves * NH * 4 * 64 * 4;
+    if (fixed > 40 * 1024) return false;
+    const size_t act_bytes = (size_t)p.M * (p.K + 32) * 2;
+    const bool act_lds = act_bytes <= 33 * 1024;
+    const int wrows = WBITS == 4 ? p.N / 2 : p.N;
+    const int tiles = (wrows + 7) / 8;
+    const dim3 grid(((tiles + 7) / 8) * 8), block(kDecWaves * 64);
+    p.m_base = 0;
+    if (act_lds && (p.group == 0 || p.group == 128)) {
+        const int steps = p.K / 128;
+        const bool full16 = steps % (kDecWaves * 16) == 0, full8 = steps % (kDecWaves * 8) == 0;
+        const size_t smem = fixed + act_bytes + 16 * 256 + 32;
+#define FNN_DEC(G, MPV)                                                                              \
+    do {                                                                                             \
+        if (full16) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, true><<<grid, block, smem, st>>>(p); \
+        else if (full8) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 8, true><<<grid, block, smem, st>>>(p); \
+        else gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, false><<<grid, block, smem, st>>>(p);  \
+    } while (0)
+        if (p.group == 0) FNN_DEC(false, 8);
+        else if (p.M == 1) FNN_DEC(true, 1);
+        else if (p.M == 2) FNN_DEC(true, 2);
+        else if (p.M <= 4) FNN_DEC(true, 4);
+        else FNN_DEC(true, 8);
+#undef FNN_DEC
+        return true;
+    }
+    const size_t smem = fixed + (act_lds ? act_bytes : 0);
+    if (p.group > 0) {
+        if (act_lds) gemm_wo_decode_kernel<WBITS, ADT, true, true><<<grid, block, smem, st>>>(p);
+        else gemm_wo_decode_kernel<WBITS, ADT, true, false><<<grid, block, smem, st>>>(p);
+    } else {
+        if (act_lds) gemm_wo_decode_kernel<WBITS, ADT, false, true><<<grid, block, smem, st>>>(p);
+        else gemm_wo_decode_kernel<WBITS, ADT, false, false><<<grid, block, smem, st>>>(p);
+    }
+    return true;
+}
+
+template <int WBITS, int ADT>
 static void dispatch_wo(WoArgs& p, hipStream_t st) {
     const bool fast = p.K % 64 == 0 && (p.group == 0 || p.group % 64 == 0) && p.ldw % 16 == 0 &&
                       p.lda % 8 == 0 && ((uintptr_t)p.qw % 16) == 0 && ((uintptr_t)p.act % 16) == 0;
@@ -331,6 +795,7 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
         gemm_wo_any_kernel<WBITS, ADT><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(p);
         return;
     }
+    if (launch_decode<WBITS, ADT>(p, st)) return;
     // up to 64 activation rows per pass over the weights
     for (int m0 = 0; m0 < p.M; m0 += 64) {
         p.m_base = m0;
