@@ -290,6 +290,49 @@ __global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoA
 }
 
 
+
+// Stage the scales and zero points of NC consecutive channels (all K-groups) in LDS as fp32:
+// s_lds[g*NC + c] = scale, z_lds[g*NC + c] = scale * (c_off + zp).  16-bit scale type SDT, same
+// type for the zero points, N a multiple of NC and 16-byte aligned tables (checked on the
+// host): every thread loads 16-byte pieces, all loads of a batch before the first store, so a
+// batch costs one memory latency.
+template <int SDT, int NC>
+__device__ __forceinline__ void fill_scales_lds(float* s_lds, float* z_lds, const WoArgs& p, int n0,
+                                                int ngroups, float c_off, int tid, int nthreads) {
+    constexpr int VPR = NC / 8;   // 16-byte pieces per group row
+    const int nvec = ngroups * VPR;
+    for (int v0 = 0; v0 < nvec; v0 += 2 * nthreads) {
+        v4u sv[2], zv[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int e = min(v0 + u * nthreads + tid, nvec - 1);
+            const int64_t off = (int64_t)(e / VPR) * p.N + n0 + (e % VPR) * 8;
+            sv[u] = *(const v4u*)((const uint16_t*)p.scale + off);
+            zv[u] = p.zp ? *(const v4u*)((const uint16_t*)p.zp + off) : v4u{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int e = v0 + u * nthreads + tid;
+            if (e < nvec) {
+                float sc[8], zo[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    sc[2 * j] = bits_to_f32<SDT>(sv[u][j] & 0xFFFFu);
+                    sc[2 * j + 1] = bits_to_f32<SDT>(sv[u][j] >> 16);
+                    zo[2 * j] = sc[2 * j] * (c_off + bits_to_f32<SDT>(zv[u][j] & 0xFFFFu));
+                    zo[2 * j + 1] = sc[2 * j + 1] * (c_off + bits_to_f32<SDT>(zv[u][j] >> 16));
+                }
+                float* sd = s_lds + (e / VPR) * NC + (e % VPR) * 8;
+                float* zd = z_lds + (e / VPR) * NC + (e % VPR) * 8;
+                *(v4f*)sd = v4f{sc[0], sc[1], sc[2], sc[3]};
+                *(v4f*)(sd + 4) = v4f{sc[4], sc[5], sc[6], sc[7]};
+                *(v4f*)zd = v4f{zo[0], zo[1], zo[2], zo[3]};
+                *(v4f*)(zd + 4) = v4f{zo[4], zo[5], zo[6], zo[7]};
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------ decode kernel (M <= 8)
 // A 256-thread workgroup (4 waves, splitting K) owns 8 weight rows (8 channels for int8,
 // 16 for packed int4): with N = 28672 int4 channels that is 1792 workgroups, exactly 7 per CU.
@@ -550,25 +593,8 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     // Fill LDS in batches: all loads of a batch are issued before the first store, so a batch
     // costs one memory latency (a load-store loop would pay it once per element).
     constexpr int NT = kDecWaves * 64;
-    {
-        const int total = ngroups * NC;
-        for (int e0 = 0; e0 < total; e0 += 4 * NT) {
-            float sc[4], z[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int e = e0 + u * NT + threadIdx.x;
-                const int ec = min(e, total - 1);
-                const int64_t idx = (int64_t)(ec / NC) * p.N + min(n0 + ec % NC, p.N - 1);
-                sc[u] = load_as_f32(p.scale, idx, p.scale_dtype);
-                z[u] = p.zp ? load_as_f32(p.zp, idx, p.zp_dtype) : 0.f;
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int e = e0 + u * NT + threadIdx.x;
-                if (e < total) { s_lds[e] = sc[u]; z_lds[e] = sc[u] * (c_off + z[u]); }
-            }
-        }
-    }
+    if (p.scale_dtype == FNN_F16) fill_scales_lds<FNN_F16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
+    else fill_scales_lds<FNN_BF16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
     {
         const int chunks = p.K / 8;   // 16-byte pieces per activation row
         for (int m = 0; m < p.M; ++m) {
@@ -706,6 +732,255 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     }
 }
 
+
+// ------------------------------------------------ GEMV kernel: one wave streams one tile
+// For many output channels (tiles >= 4 x CUs) the K split across waves is dropped: a
+// workgroup has one wave per tile of 8 weight rows, each wave walks the whole K range of its
+// tile with UN 16-byte loads in flight, and the grid is sized to one workgroup per CU
+// (N = 28672 int4 channels: 1792 tiles = 256 workgroups x 7 waves).  Long streams keep the
+// load queue full for the whole kernel, there is no cross-wave reduction, and every CU gets
+// the same number of bytes.  Activations (M <= 4 rows) are staged in LDS once per workgroup,
+// the scales of a tile once per wave; the MFMA layout, the group slots and the integer
+// conversion are those of gemm_wo_decode_lds_kernel.
+constexpr int kGemvMaxWaves = 8;
+
+template <int WBITS, int ADT, bool G128, int MP, int UN, bool FULL>
+__global__ __launch_bounds__(kGemvMaxWaves * 64) void gemm_wo_gemv_kernel(const WoArgs p, const int wpw) {
+    typedef MfmaT<ADT> MT;
+    constexpr int NH = WBITS == 4 ? 2 : 1;
+    constexpr int NC = 8 * NH;
+    constexpr int GS = G128 ? 8 / MP : 1;
+    constexpr float c_off = WBITS == 4 ? (ADT == FNN_F16 ? 1024.f + 8.f : 128.f + 8.f)
+                                       : (ADT == FNN_F16 ? 1024.f + 128.f : 128.f);
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int li = lane & 15;
+    const int lg = lane >> 4;
+    const int half = li >> 3;
+    const int j7 = li & 7;
+
+    const int wrows = WBITS == 4 ? p.N / 2 : p.N;
+    const int tiles = (wrows + 7) / 8;
+    const int tile = blockIdx.x * wpw + wave;
+    const bool tile_ok = tile < tiles;           // wave-uniform
+    const int row0 = min(tile, tiles - 1) * 8;
+    const int n0 = row0 * NH;
+
+    const int steps = p.K / 128;
+    const int ngroups = G128 ? steps : 1;
+
+    // LDS: [32 B of zeros][activations M x (K+32)][per wave: scale, zoff (ngroups*NC f32 each)]
+    const int a_stride = p.K + 32;
+    uint16_t* a_lds = (uint16_t*)(smem + 32);
+    float* s_lds = (float*)(smem + 32 + (size_t)p.M * a_stride * 2) + (size_t)wave * ngroups * NC * 2;
+    float* z_lds = s_lds + ngroups * NC;
+
+    const int wrow_l = min(row0 + j7, wrows - 1) - row0;
+    const uint32_t w_off = (uint32_t)wrow_l * (uint32_t)p.ldw + lg * 32 + half * 16;
+    const char* w_tile = (const char*)p.qw + (int64_t)row0 * p.ldw;
+    auto load_w = [&](int step) -> v4u {
+        const char* base = w_tile + (int64_t)min(step, steps - 1) * 128;   // scalar
+        return __builtin_nontemporal_load((const v4u*)(base + w_off));
+    };
+    // ---- start-up: every load is issued before the first wait ----
+    // The small tables go first (vector memory returns in order): scales and zero points of the
+    // tile, the activation rows, then the first UN weight pieces.  The tables are written to LDS
+    // while the weight loads are still in flight.
+    constexpr int VPR = NC / 8;   // 16-byte pieces per scale row of the tile
+    constexpr int SB = 2;         // scale batches staged in registers
+    constexpr int AB = 4;         // activation batches per row staged in registers
+    const int nvec = ngroups * VPR;
+    const int chunks = p.K / 8;
+    const int nt = blockDim.x;
+    const bool has_zp = p.zp != nullptr;
+    const uint16_t* zp_tab = has_zp ? (const uint16_t*)p.zp : (const uint16_t*)p.scale;
+    v4u sv[SB], zv[SB];
+#pragma unroll
+    for (int u = 0; u < SB; ++u) {
+        const int e = min(u * 64 + lane, nvec - 1);
+        const int64_t off = (int64_t)(e / VPR) * p.N + n0 + (e % VPR) * 8;
+        sv[u] = *(const v4u*)((const uint16_t*)p.scale + off);
+        zv[u] = *(const v4u*)(zp_tab + off);
+    }
+    v4u av[4][AB];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        const v4u* src = (const v4u*)((const uint16_t*)p.act + (int64_t)min(m, p.M - 1) * p.lda);
+#pragma unroll
+        for (int u = 0; u < AB; ++u) av[m][u] = src[min(u * nt + (int)threadIdx.x, chunks - 1)];
+    }
+    v4u wq[UN];
+#pragma unroll
+    for (int i = 0; i < UN; ++i) wq[i] = load_w(i);
+
+    if (threadIdx.x < 8) ((uint32_t*)smem)[threadIdx.x] = 0;
+    const bool s_f16 = p.scale_dtype == FNN_F16;
+#pragma unroll
+    for (int u = 0; u < SB; ++u) {
+        const int e = u * 64 + lane;
+        if (e < nvec) {
+            float sc[8], zo[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t sb = (sv[u][j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
+                const uint32_t zb = (zv[u][j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
+                sc[j] = s_f16 ? f16_bits_to_f32(sb) : bf16_bits_to_f32(sb);
+                const float z = s_f16 ? f16_bits_to_f32(zb) : bf16_bits_to_f32(zb);
+                zo[j] = sc[j] * (c_off + (has_zp ? z : 0.f));
+            }
+            float* sd = s_lds + (e / VPR) * NC + (e % VPR) * 8;
+            float* zd = z_lds + (e / VPR) * NC + (e % VPR) * 8;
+            *(v4f*)sd = v4f{sc[0], sc[1], sc[2], sc[3]};
+            *(v4f*)(sd + 4) = v4f{sc[4], sc[5], sc[6], sc[7]};
+            *(v4f*)zd = v4f{zo[0], zo[1], zo[2], zo[3]};
+            *(v4f*)(zd + 4) = v4f{zo[4], zo[5], zo[6], zo[7]};
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        v4u* dst = (v4u*)(a_lds + m * a_stride);
+#pragma unroll
+        for (int u = 0; u < AB; ++u) {
+            const int c = u * nt + threadIdx.x;
+            if (m < p.M && c < chunks) dst[c] = WBITS == 4 ? perm_act_w4(av[m][u]) : av[m][u];
+        }
+    }
+    // whatever did not fit the staged batches (very long K)
+    if (nvec > SB * 64) {
+        float* so = s_lds + SB * 64 / VPR * NC;
+        float* zo = z_lds + SB * 64 / VPR * NC;
+        WoArgs q = p;
+        q.scale = (const uint16_t*)p.scale + (int64_t)(SB * 64 / VPR) * p.N;
+        if (has_zp) q.zp = (const uint16_t*)p.zp + (int64_t)(SB * 64 / VPR) * p.N;
+        if (s_f16) fill_scales_lds<FNN_F16, NC>(so, zo, q, n0, ngroups - SB * 64 / VPR, c_off, lane, 64);
+        else fill_scales_lds<FNN_BF16, NC>(so, zo, q, n0, ngroups - SB * 64 / VPR, c_off, lane, 64);
+    }
+    if (chunks > AB * nt) {
+        for (int m = 0; m < p.M; ++m) {
+            const v4u* src = (const v4u*)((const uint16_t*)p.act + (int64_t)m * p.lda);
+            v4u* dst = (v4u*)(a_lds + m * a_stride);
+            for (int c = AB * nt + threadIdx.x; c < chunks; c += nt)
+                dst[c] = WBITS == 4 ? perm_act_w4(src[c]) : src[c];
+        }
+    }
+    __syncthreads();
+
+    const int m_col = G128 ? (j7 % MP) : j7;
+    const int gslot = G128 ? (j7 / MP) : 0;
+    const bool col_valid = m_col < p.M;
+    bool use[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) use[i] = col_valid && (i % GS) == gslot;
+    const int koff = lg * 32 + half * 16;
+    uint32_t a_real = (uint32_t)((const char*)(a_lds + m_col * a_stride + koff) - smem);
+    uint32_t sz_addr = (uint32_t)((const char*)(s_lds + gslot * (G128 ? NC : 0) + NH * 4 * (lg & 1)) - smem);
+    const uint32_t z_delta = (uint32_t)(ngroups * NC * 4);
+
+    v4f outv[NH], accg[NH], asum;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) { outv[h] = v4f{0, 0, 0, 0}; accg[h] = v4f{0, 0, 0, 0}; }
+    asum = v4f{0, 0, 0, 0};
+    const v4f zero4 = v4f{0, 0, 0, 0};
+
+    auto fold = [&](uint32_t addr) {
+        float sv[NH * 4], zv[NH * 4];
+#pragma unroll
+        for (int q = 0; q < NH; ++q) {
+            const v4f a = *(const v4f*)(smem + addr + q * 16);
+            const v4f b = *(const v4f*)(smem + addr + z_delta + q * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { sv[q * 4 + e] = a[e]; zv[q * 4 + e] = b[e]; }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+                outv[h][r] += sv[NH * r + h] * accg[h][r] - zv[NH * r + h] * asum[r];
+    };
+
+    // Queue slots are refilled BURST at a time, after the last of them has been consumed (so old
+    // and new value share registers): DRAM then sees 8 rows x BURST*128 contiguous bytes per
+    // burst instead of single 128-byte pieces, which keeps more of its row buffers useful.
+    constexpr int BURST = UN >= 16 ? 4 : 1;
+    auto refill = [&](int i, int sb) {
+        if (i % BURST == BURST - 1) {
+#pragma unroll
+            for (int b = 0; b < BURST; ++b) wq[i - (BURST - 1) + b] = load_w(sb + i - (BURST - 1) + b + UN);
+        }
+    };
+    const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+    for (int sb = 0; sb < steps; sb += UN) {
+#pragma unroll
+        for (int i = 0; i < UN; ++i) {
+            const int step = sb + i;
+            if (FULL || step < steps) {
+                const v4u w = wq[i];
+                const uint32_t aa = use[i % 8] ? a_real + i * 256 : 0u;
+                const v4u a0 = *(const v4u*)(smem + aa);
+                const v4u a1 = *(const v4u*)(smem + aa + 16);
+                const bool first = G128 ? (i % GS == 0) : (step == 0);
+                if constexpr (WBITS == 4) {
+                    v4u e0, e1, o0, o1;
+                    convert_w4<ADT>(w, e0, e1, o0, o1);
+                    refill(i, sb);
+                    accg[0] = MT::mma(e0, a0, first ? zero4 : accg[0]);
+                    accg[1] = MT::mma(o0, a0, first ? zero4 : accg[1]);
+                    asum = MT::mma(ones, a0, first ? zero4 : asum);
+                    accg[0] = MT::mma(e1, a1, accg[0]);
+                    accg[1] = MT::mma(o1, a1, accg[1]);
+                    asum = MT::mma(ones, a1, asum);
+                } else {
+                    v4u s0, s1;
+                    convert_w8<ADT>(w, s0, s1);
+                    refill(i, sb);
+                    accg[0] = MT::mma(s0, a0, first ? zero4 : accg[0]);
+                    asum = MT::mma(ones, a0, first ? zero4 : asum);
+                    accg[0] = MT::mma(s1, a1, accg[0]);
+                    asum = MT::mma(ones, a1, asum);
+                }
+                if constexpr (G128) {
+                    if (i % GS == GS - 1 || (!FULL && step + 1 == steps))
+                        fold(sz_addr + (i / GS) * GS * NC * 4);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);   // keep each refill load inside its step
+        }
+        a_real += UN * 256;
+        if constexpr (G128) sz_addr += UN * NC * 4;
+    }
+    if constexpr (!G128) fold(sz_addr);
+
+    // ---- per-wave reduction of the group-slot columns and the two diagonal blocks ----
+    // the wave's own scale area is free now and private to it
+    float* red = s_lds;
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[(h * 4 + r) * 64 + lane] = outv[h][r];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): this wave's LDS writes are done
+    for (int e = lane; e < p.M * NC; e += 64) {
+        const int m = e / NC, c = e % NC;
+        const int row = c / NH, h = c % NH;
+        const int r = row & 3;
+        float v = 0.f;
+#pragma unroll
+        for (int gs = 0; gs < GS; ++gs) {
+            const int col = gs * (G128 ? MP : 0) + m;
+            const int lane1 = col + 16 * (row >> 2);
+            const int lane2 = (col + 8) + 16 * ((row + 8) >> 2);
+            v += red[(h * 4 + r) * 64 + lane1] + red[(h * 4 + r) * 64 + lane2];
+        }
+        const int n = n0 + c;
+        if (tile_ok && n < p.N) {
+            if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+            store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ guarded fallback
 template <int WBITS, int ADT>
 __global__ __launch_bounds__(256) void gemm_wo_any_kernel(const WoArgs p) {
@@ -757,7 +1032,42 @@ static bool launch_decode(WoArgs& p, hipStream_t st) {
     const int tiles = (wrows + 7) / 8;
     const dim3 grid(((tiles + 7) / 8) * 8), block(kDecWaves * 64);
     p.m_base = 0;
-    if (act_lds && (p.group == 0 || p.group == 128)) {
+    // the LDS-staged kernels read the scale tables in 16-byte pieces
+    const bool tables16 = is16(p.scale_dtype) && (!p.zp || p.zp_dtype == p.scale_dtype) &&
+                          p.N % (8 * NH) == 0 && ((uintptr_t)p.scale % 16) == 0 &&
+                          (!p.zp || ((uintptr_t)p.zp % 16) == 0);
+    // many tiles: one wave per tile, one workgroup per CU
+    if (tables16 && (p.group == 0 || p.group == 128) && p.M <= 4 && tiles >= 4 * 256) {
+        int wpw = (tiles + 255) / 256;
+        const int ngr = p.group > 0 ? p.K / 128 : 1;
+        while (wpw > kGemvMaxWaves) wpw = (wpw + 1) / 2;
+        const size_t need = 32 + act_bytes + (size_t)wpw * ngr * 8 * NH * 8;
+        // ask for more than half of the 160 KB so that two workgroups never share a CU
+        const size_t smem = need > 84 * 1024 ? need : 84 * 1024;
+        // the wave's scale area doubles as its reduction scratch (NH*4*64 floats)
+        if (need <= 150 * 1024 && (size_t)ngr * 8 * NH * 2 >= (size_t)NH * 4 * 64) {
+            const dim3 g2((tiles + wpw - 1) / wpw), b2(wpw * 64);
+            const bool full = (p.K / 128) % 8 == 0;
+#define FNN_GEMV(G, MPV)                                                                                  \
+    do {                                                                                                  \
+        auto kfn = full ? gemm_wo_gemv_kernel<WBITS, ADT, G, MPV, 8, true>                               \
+                        : gemm_wo_gemv_kernel<WBITS, ADT, G, MPV, 8, false>;                             \
+        static bool attr_set[2] = {false, false};                                                         \
+        if (!attr_set[full]) {                                                                            \
+            (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            attr_set[full] = true;                                                                        \
+        }                                                                                                 \
+        kfn<<<g2, b2, smem, st>>>(p, wpw);                                                                \
+    } while (0)
+            if (p.group == 0) FNN_GEMV(false, 8);
+            else if (p.M == 1) FNN_GEMV(true, 1);
+            else if (p.M == 2) FNN_GEMV(true, 2);
+            else FNN_GEMV(true, 4);
+#undef FNN_GEMV
+            return true;
+        }
+    }
+    if (tables16 && act_lds && (p.group == 0 || p.group == 128)) {
         const int steps = p.K / 128;
         const bool full16 = steps % (kDecWaves * 16) == 0, full8 = steps % (kDecWaves * 8) == 0;
         const size_t smem = fixed + act_bytes + 16 * 256 + 32;

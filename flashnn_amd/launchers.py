@@ -118,8 +118,8 @@ def _weight_only(fn_name, out, act, quant_w, scale_w, bias, zero_points, n_out):
     zp = None
     if zero_points is not None:
         zp = zero_points.squeeze().reshape(scale_w.shape).contiguous()
-        if not zp.is_floating_point():
-            zp = zp.to(scale_w.dtype)
+        if zp.dtype != scale_w.dtype:
+            zp = zp.to(scale_w.dtype)   # zero points are small integers: exact in any float type
     if bias is not None:
         bias = bias.reshape(-1).contiguous()
         assert bias.numel() == N
