@@ -45,37 +45,36 @@ struct A8W8Args {
 };
 
 
-// ------------------------------------------------------------------ pipelined main kernel
-// K % 256 == 0.  Slabs of 64 bytes of K; four static LDS stages form a ring, the copy of
-// slab j+3 is issued while slab j-1 is being finished, so a copy has three slabs of MFMA time
-// (about 1 us) to land.  One barrier per slab, placed at the start of the LAST k-step of the
-// previous slab: by then every fragment of that slab is in registers, which frees its stage
-// for the copy issued right after the barrier, and the barrier also publishes the next slab,
-// whose first fragments are read while the last MFMAs of the previous slab run.  Fragments
-// are double-buffered in registers; LDS reads and MFMAs are interleaved one to one.
-//
-// LDS rows are 64 bytes (4 chunks of 16); chunk c of row r is stored at slot c ^ ((r >> 1) & 3),
-// which spreads the 8 rows read together over all 32 banks.
-constexpr int BK4 = 64;
-
-template <int BM, int BN>
-struct Stage4 {
-    char bytes[(BM + BN) * BK4];
-};
+// ------------------------------------------------------------------ main MFMA kernel
+// K % 128 == 0, K >= 512.  K is walked in slabs of 128 bytes: every row piece a copy fetches
+// is one full 128-byte line, which is what the L2 -> LDS path needs to run at speed (64-byte
+// pieces reach little more than half the rate).  The LDS holds an asymmetric ring: three
+// stages for the a-rows (copied two slabs ahead) and two for the b-rows (one slab ahead);
+// 3*BM + 2*BN rows of 128 bytes = 144 KB for a 256x192 tile.  There is one barrier per slab, at
+// the start of its LAST k-step: by then every fragment of the slab is in registers, so both of
+// its stages are free and are re-armed right after the barrier, and the barrier publishes the
+// next slab, whose first fragments are read under the last MFMAs of the current one.
+// Fragments are double-buffered in registers; LDS reads and MFMAs alternate one to one.
+// Chunk c (16 bytes) of LDS row r is stored at slot c ^ ((r >> 1) & 7).  A 16-byte LDS read serves
+// 16 lanes (16 consecutive rows, same chunk) per cycle out of 64 banks = 256 bytes; two rows fill
+// that period, so rows of equal parity must land in 8 different slots.  (r & 7 instead gives
+// two-way conflicts: measured 8 instead of 4 cycles per read.)  The swizzle is applied on the
+// global side of the copy; the LDS side of a direct-to-LDS load is linear in the lane id.
 
 template <int BM, int BN, int MODE>
-__global__ __launch_bounds__(256) void gemm_a8w8_mfma4_kernel(const A8W8Args p) {
+__global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     constexpr int NWAVES = 4;
     constexpr int WTM = BM / 2, WTN = BN / 2;
     constexpr int FM = WTM / 32, FN = WTN / 32;
-    constexpr int ROWS = BM + BN;
-    constexpr int NLD = ROWS / (16 * NWAVES);   // a wave-load covers 16 rows of 64 bytes
-    static_assert(ROWS % (16 * NWAVES) == 0 && BM % (16 * NWAVES) == 0, "tile rows must split evenly");
+    constexpr int NLA = BM / (8 * NWAVES);   // a wave-load covers 8 rows of 128 bytes
+    constexpr int NLB = BN / (8 * NWAVES);
+    static_assert(BM % (8 * NWAVES) == 0 && BN % (8 * NWAVES) == 0, "tile rows must split evenly");
 
-    __shared__ __attribute__((aligned(1024))) Stage4<BM, BN> st0;
-    __shared__ __attribute__((aligned(1024))) Stage4<BM, BN> st1;
-    __shared__ __attribute__((aligned(1024))) Stage4<BM, BN> st2;
-    __shared__ __attribute__((aligned(1024))) Stage4<BM, BN> st3;
+    __shared__ __attribute__((aligned(1024))) char sa0[BM * BK];
+    __shared__ __attribute__((aligned(1024))) char sa1[BM * BK];
+    __shared__ __attribute__((aligned(1024))) char sa2[BM * BK];
+    __shared__ __attribute__((aligned(1024))) char sb0[BN * BK];
+    __shared__ __attribute__((aligned(1024))) char sb1[BN * BK];
     __shared__ __attribute__((aligned(16))) float sc_row[BM];   // alpha_row of the tile's rows, fp32
     __shared__ __attribute__((aligned(16))) float sc_col[BN];   // alpha_col of the tile's columns
 
@@ -92,9 +91,8 @@ __global__ __launch_bounds__(256) void gemm_a8w8_mfma4_kernel(const A8W8Args p) 
     const int wm = wave & 1;
     const int wn = wave >> 1;
 
-    // Scales of the tile go to LDS as fp32 before anything else is in flight (their loads are the
-    // oldest, so waiting for them does not wait for the copies issued below); the epilogue then
-    // needs no global loads at all.
+    // Scales of the tile go to LDS as fp32 before anything else is in flight; the epilogue then
+    // needs no global loads.
     if constexpr (MODE != OUT_I32) {
         for (int e = threadIdx.x; e < BM + BN; e += 256) {
             const bool is_row = e < BM;
@@ -104,36 +102,40 @@ __global__ __launch_bounds__(256) void gemm_a8w8_mfma4_kernel(const A8W8Args p) 
         }
     }
 
-    // copy plan: load j of this wave fills rows rg*16 .. rg*16+15, rg = j*NWAVES + wave; lane L
-    // writes slot (L & 3) of row rg*16 + (L >> 2), which holds logical chunk (L & 3) ^ ((row >> 1) & 3)
-    const int lrow = lane >> 2;
-    const int lchunk = (lane & 3) ^ ((lrow >> 1) & 3);
-    uint32_t goff[NLD];
+    // copy plan: load j of this wave fills rows (j*NWAVES + wave)*8 .. +7; lane L writes slot (L & 7)
+    // of row (L >> 3) of that group, which holds logical chunk (L & 7) ^ ((row >> 1) & 7)
+    const int lrow = lane >> 3;
+    const int lchunk = (lane & 7) ^ ((((wave & 1) << 2) + (lrow >> 1)) & 7);
+    uint32_t goa[NLA], gob[NLB];
 #pragma unroll
-    for (int j = 0; j < NLD; ++j) {
-        const int rr = (j * NWAVES + wave) * 16 + lrow;
-        if (rr < BM) goff[j] = (uint32_t)min(m0 + rr, p.M - 1) * (uint32_t)p.lda + lchunk * 16;
-        else goff[j] = (uint32_t)min(n0 + rr - BM, p.N - 1) * (uint32_t)p.ldb + lchunk * 16;
-    }
-    auto issue_loads = [&](char* stage_bytes, int kt) {
-        const char* a_slab = (const char*)p.a + (int64_t)kt * BK4;
-        const char* b_slab = (const char*)p.b + (int64_t)kt * BK4;
+    for (int j = 0; j < NLA; ++j)
+        goa[j] = (uint32_t)min(m0 + (j * NWAVES + wave) * 8 + lrow, p.M - 1) * (uint32_t)p.lda + lchunk * 16;
 #pragma unroll
-        for (int j = 0; j < NLD; ++j) {
-            char* dst = stage_bytes + (j * NWAVES + wave) * (16 * BK4);
-            const char* src = ((j * NWAVES) * 16 < BM ? a_slab : b_slab) + goff[j];
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)dst, 16, 0, 0);
-        }
+    for (int j = 0; j < NLB; ++j)
+        gob[j] = (uint32_t)min(n0 + (j * NWAVES + wave) * 8 + lrow, p.N - 1) * (uint32_t)p.ldb + lchunk * 16;
+    auto copy_a = [&](char* stage, int kt) {
+        const char* slab = (const char*)p.a + (int64_t)kt * BK;
+#pragma unroll
+        for (int j = 0; j < NLA; ++j)
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + goa[j]),
+                                             (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
+    };
+    auto copy_b = [&](char* stage, int kt) {
+        const char* slab = (const char*)p.b + (int64_t)kt * BK;
+#pragma unroll
+        for (int j = 0; j < NLB; ++j)
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
+                                             (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
 
-    // read plan: lane reads row (lane & 31) of a fragment, logical chunk 2*s + (lane >> 5)
+    // read plan: lane reads row (lane & 31) of a fragment, logical chunk 2*ks + (lane >> 5)
     const int frow = lane & 31;
     const int hsel = lane >> 5;
-    int rd_off[2];
+    int rd_off[4];
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) rd_off[s2] = frow * BK4 + (((2 * s2 + hsel) ^ ((frow >> 1) & 3)) * 16);
-    const int a_base = wm * WTM * BK4;
-    const int b_base = (BM + wn * WTN) * BK4;
+    for (int ks = 0; ks < 4; ++ks) rd_off[ks] = frow * BK + (((2 * ks + hsel) ^ ((frow >> 1) & 7)) * 16);
+    const int a_base = wm * WTM * BK;
+    const int b_base = wn * WTN * BK;
 
     v16i acc[FN][FM];
 #pragma unroll
@@ -144,88 +146,101 @@ __global__ __launch_bounds__(256) void gemm_a8w8_mfma4_kernel(const A8W8Args p) 
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     v4i wf[2][FN], af[2][FM];   // fragment double buffer, indexed by k-step parity
-    auto read_frags = [&](const char* stage_bytes, int s2) {
+    auto read_frags = [&](const char* sa, const char* sb, int ks) {
 #pragma unroll
-        for (int i = 0; i < FN; ++i) wf[s2][i] = *(const v4i*)(stage_bytes + b_base + i * 32 * BK4 + rd_off[s2]);
+        for (int i = 0; i < FN; ++i) wf[ks & 1][i] = *(const v4i*)(sb + b_base + i * 32 * BK + rd_off[ks]);
 #pragma unroll
-        for (int j = 0; j < FM; ++j) af[s2][j] = *(const v4i*)(stage_bytes + a_base + j * 32 * BK4 + rd_off[s2]);
+        for (int j = 0; j < FM; ++j) af[ks & 1][j] = *(const v4i*)(sa + a_base + j * 32 * BK + rd_off[ks]);
     };
-    auto mfmas = [&](int s2) {
+    auto mfmas = [&](int par) {
 #pragma unroll
         for (int i = 0; i < FN; ++i)
 #pragma unroll
             for (int j = 0; j < FM; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s2][i], af[s2][j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[par][i], af[par][j], acc[i][j], 0, 0, 0);
     };
-    // ask the scheduler for: MFMA, LDS read, MFMA, LDS read, ... then the remaining MFMAs
+    // ask the scheduler for: MFMA, 2 LDS reads, MFMA, 2 LDS reads, ... then the remaining MFMAs.
+    // The reads of the next k-step are all issued under the first few MFMAs, which leaves their
+    // latency the rest of the k-step (8 MFMAs = 256 cycles) to elapse.
     auto interleave = [&]() {
+        constexpr int NRD = FN + FM;
 #pragma unroll
-        for (int q = 0; q < FN + FM; ++q) {
+        for (int q = 0; q < NRD / 2; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        if constexpr (NRD % 2 == 1) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, FN * FM - (FN + FM), 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, FN * FM - (NRD + 1) / 2, 0);
     };
-
-    const int KT = p.K / BK4;   // multiple of 4, >= 8 (checked on the host)
-    // Wait until at most `newer` of this wave's copies are outstanding and all its LDS reads have
-    // returned, then cross the workgroup barrier.  A bare s_barrier is used: __syncthreads() would
-    // add a fence that waits for every outstanding copy and collapse the ring to depth one.
-    auto wait_barrier = [&](int newer) {
+    // Wait until at most `newer` of this wave's copies are outstanding and its LDS reads have
+    // returned, then cross the workgroup barrier.  A bare s_barrier: __syncthreads() would add a
+    // fence that waits for every outstanding copy and collapse the ring to depth one.
+    auto wait_barrier = [&](bool keep_a) {
         asm volatile("" ::: "memory");
-        if (newer == 2 * NLD) __builtin_amdgcn_s_waitcnt(0x0070 | ((2 * NLD) & 15) | (((2 * NLD) >> 4) << 14));
-        else if (newer == NLD) __builtin_amdgcn_s_waitcnt(0x0070 | (NLD & 15) | ((NLD >> 4) << 14));
+        if (keep_a) __builtin_amdgcn_s_waitcnt(0x0070 | (NLA & 15) | ((NLA >> 4) << 14));
         else __builtin_amdgcn_s_waitcnt(0x0070);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
-    // One slab = two k-steps.  Step 0 overlaps the fragment reads of step 1.  Step 1 (the last of
-    // the slab) first waits for the next slab and crosses the barrier, then reads the next slab's
-    // first fragments and re-arms the stage it has just finished, all under its own MFMAs.
-    //   newer  : copies that may stay outstanding at the barrier (-1: there is no next slab)
-    //   refill : slab index to copy into `cur`, or -1
-    auto slab = [&](char* cur, const char* nxt, int newer, int refill) {
-        read_frags(cur, 1);
-        mfmas(0);
-        interleave();
-        __builtin_amdgcn_sched_barrier(0);
-        if (newer >= 0) {
-            wait_barrier(newer);
-            read_frags(nxt, 0);
-            if (refill >= 0) issue_loads(cur, refill);
+
+    const int KT = p.K / BK;
+    // One slab = four k-steps.  `nsa`/`nsb` are the stages of the next slab (nullptr-free: the
+    // flags say whether there is one).  At the barrier the only copy that may stay in flight is
+    // the a-copy issued at the previous barrier (for the slab after next).
+    auto slab = [&](char* sa, char* sb, const char* nsa, const char* nsb, int j, bool steady) {
+#pragma unroll
+        for (int ks = 0; ks < 3; ++ks) {
+            read_frags(sa, sb, ks + 1);
+            mfmas(ks & 1);
+            interleave();
+            __builtin_amdgcn_sched_barrier(0);
         }
-        mfmas(1);
-        if (newer >= 0) interleave();
+        if (steady || j + 1 < KT) {
+            wait_barrier(steady || j + 2 < KT);
+            read_frags(nsa, nsb, 0);
+            if (steady || j + 2 < KT) copy_b(sb, j + 2);
+            if (steady || j + 3 < KT) copy_a(sa, j + 3);
+            mfmas(1);
+            interleave();
+        } else {
+            mfmas(1);
+        }
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    issue_loads(st0.bytes, 0);
-    issue_loads(st1.bytes, 1);
-    issue_loads(st2.bytes, 2);
-    issue_loads(st3.bytes, 3);
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0x0070 | ((3 * NLD) & 15) | (((3 * NLD) >> 4) << 14));   // slab 0 landed
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    read_frags(st0.bytes, 0);
-    int kt = 0;
-    for (; kt + 8 <= KT; kt += 4) {
-        slab(st0.bytes, st1.bytes, 2 * NLD, kt + 4);
-        slab(st1.bytes, st2.bytes, 2 * NLD, kt + 5);
-        slab(st2.bytes, st3.bytes, 2 * NLD, kt + 6);
-        slab(st3.bytes, st0.bytes, 2 * NLD, kt + 7);
+    copy_a(sa0, 0);
+    copy_b(sb0, 0);
+    copy_a(sa1, 1);
+    wait_barrier(true);
+    read_frags(sa0, sb0, 0);
+    copy_b(sb1, 1);
+    copy_a(sa2, 2);
+    int j = 0;
+    for (; j + 9 <= KT; j += 6) {   // every slab of the round still has both refills ahead of it
+        slab(sa0, sb0, sa1, sb1, j, true);
+        slab(sa1, sb1, sa2, sb0, j + 1, true);
+        slab(sa2, sb0, sa0, sb1, j + 2, true);
+        slab(sa0, sb1, sa1, sb0, j + 3, true);
+        slab(sa1, sb0, sa2, sb1, j + 4, true);
+        slab(sa2, sb1, sa0, sb0, j + 5, true);
     }
-    // last four slabs: nothing left to copy, the outstanding count runs down
-    slab(st0.bytes, st1.bytes, 2 * NLD, -1);
-    slab(st1.bytes, st2.bytes, NLD, -1);
-    slab(st2.bytes, st3.bytes, 0, -1);
-    slab(st3.bytes, st3.bytes, -1, -1);
+    for (; j < KT; j += 6) {        // the last three to eight slabs, with the refills guarded
+        slab(sa0, sb0, sa1, sb1, j, false);
+        if (j + 1 < KT) slab(sa1, sb1, sa2, sb0, j + 1, false);
+        if (j + 2 < KT) slab(sa2, sb0, sa0, sb1, j + 2, false);
+        if (j + 3 < KT) slab(sa0, sb1, sa1, sb0, j + 3, false);
+        if (j + 4 < KT) slab(sa1, sb0, sa2, sb1, j + 4, false);
+        if (j + 5 < KT) slab(sa2, sb1, sa0, sb0, j + 5, false);
+    }
 
     // ---- epilogue ----
     // acc[i][j][r]: n = wn0 + i*32 + 8*(r/4) + 4*(lane>>5) + (r&3),  m = wm0 + j*32 + (lane&31).
     // A lane owns 4 consecutive n of ONE row, so storing straight from registers would touch 32
     // rows per instruction with 16 bytes each.  Instead every wave transposes its sub-tile through
-    // LDS (the ring stage with its own index, free now) 64 rows at a time and writes whole rows:
+    // LDS (one ring stage per wave, free now) 64 rows at a time and writes whole rows:
     // 16 bytes per lane, consecutive lanes on consecutive addresses.
     const int wm0 = m0 + wm * WTM;
     const int wn0 = n0 + wn * WTN;
@@ -255,8 +270,8 @@ __global__ __launch_bounds__(256) void gemm_a8w8_mfma4_kernel(const A8W8Args p) 
     } else {
         constexpr int TSTRIDE = WTN * 2 + 16;      // bytes per staged row; the pad staggers the banks
         constexpr int PR = WTN * 2 / 16;           // 16-byte pieces per row
-        static_assert(64 * TSTRIDE <= (int)sizeof(Stage4<BM, BN>), "transpose buffer must fit a stage");
-        char* tbuf = wave == 0 ? st0.bytes : wave == 1 ? st1.bytes : wave == 2 ? st2.bytes : st3.bytes;
+        static_assert(64 * TSTRIDE <= BN * BK, "transpose buffer must fit a stage");
+        char* tbuf = wave == 0 ? sa0 : wave == 1 ? sa1 : wave == 2 ? sa2 : sb0;
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0x0070);   // all copies and LDS reads of this wave are done
         __builtin_amdgcn_s_barrier();         // ... and everybody else's: the stages are free
@@ -372,7 +387,7 @@ struct TileChoice { int bm, bn; };
 // Pick the tile whose last, partly filled round of workgroups costs least on 256 CUs.
 static TileChoice choose_tile(int64_t M, int64_t N) {
     static const struct { int bm, bn; double eff; } cand[] = {
-        {256, 256, 1.00}, {256, 192, 0.97}, {256, 128, 0.88}, {128, 128, 0.70}};
+        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.65}};
     double best = 1e300;
     TileChoice c{128, 128};
     for (const auto& t : cand) {
@@ -390,13 +405,13 @@ static void launch_mfma(A8W8Args& p, hipStream_t st) {
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
-    gemm_a8w8_mfma4_kernel<BM, BN, MODE><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p);
+    gemm_a8w8_ring_kernel<BM, BN, MODE><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p);
 }
 
 template <int MODE>
 static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
-    // the MFMA kernel walks K in four-slab rounds of 64 bytes and addresses rows with 32-bit offsets
-    const bool fast = p.K % 256 == 0 && p.K >= 512 && p.lda % 16 == 0 && p.ldb % 16 == 0 &&
+    // the MFMA kernel walks K in slabs of 128 bytes and addresses rows with 32-bit offsets
+    const bool fast = p.K % 128 == 0 && p.K >= 512 && p.lda % 16 == 0 && p.ldb % 16 == 0 &&
                       ((uintptr_t)p.a % 16) == 0 && ((uintptr_t)p.b % 16) == 0 &&
                       ((uintptr_t)p.out % 16) == 0 && (int64_t)p.M * p.lda < (1LL << 31) &&
                       (int64_t)p.N * p.ldb < (1LL << 31);
@@ -406,8 +421,7 @@ static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
     }
     TileChoice c = choose_tile(p.M, p.N);
     if (force_bm > 0) c = {force_bm, force_bn};
-    if (c.bm == 256 && c.bn == 256) launch_mfma<256, 256, MODE>(p, st);
-    else if (c.bm == 256 && c.bn == 192) launch_mfma<256, 192, MODE>(p, st);
+    if (c.bm == 256 && c.bn == 192) launch_mfma<256, 192, MODE>(p, st);
     else if (c.bm == 256 && c.bn == 128) launch_mfma<256, 128, MODE>(p, st);
     else launch_mfma<128, 128, MODE>(p, st);
 }
@@ -434,7 +448,7 @@ using namespace fnn;
 // Test hook: force a tile shape (bm, bn) for the next calls on any thread; (0, 0) = automatic.
 static int g_force_bm = 0, g_force_bn = 0;
 extern "C" int fnn_debug_force_a8w8_tile(int bm, int bn) {
-    const bool ok = (bm == 0 && bn == 0) || (bm == 256 && (bn == 256 || bn == 192 || bn == 128)) ||
+    const bool ok = (bm == 0 && bn == 0) || (bm == 256 && (bn == 192 || bn == 128)) ||
                     (bm == 128 && bn == 128);
     if (!ok) { set_error("fnn_debug_force_a8w8_tile: no such tile %dx%d", bm, bn); return FNN_ERR_ARG; }
     g_force_bm = bm;

@@ -125,8 +125,7 @@ int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const void* scale
 /*
  * Test hook, no counterpart in the reference: force the output tile (bm x bn) of the MFMA
  * A8W8 kernel for subsequent calls, so that every tile shape can be checked on small
- * problems; (0, 0) restores the automatic choice.  Valid tiles: 256x256, 256x192, 256x128,
- * 128x128.  Process-wide and not synchronised: for tests only.
+ * problems; (0, 0) restores the automatic choice.  Valid tiles: 256x192, 256x128, 128x128.  Process-wide and not synchronised: for tests only.
  */
 int fnn_debug_force_a8w8_tile(int bm, int bn);
 

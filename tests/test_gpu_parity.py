@@ -77,9 +77,9 @@ def _rand_i8(shape, seed, lo=-128, hi=128):
     return torch.randint(lo, hi, shape, generator=g, dtype=torch.int8)
 
 
-@pytest.mark.parametrize("tile", [(0, 0), (256, 256), (256, 192), (256, 128), (128, 128)])
-@pytest.mark.parametrize("mnk", [(128, 128, 128), (300, 200, 256), (512, 768, 1024), (16, 4096, 4096),
-                                 (257, 129, 384)])
+@pytest.mark.parametrize("tile", [(0, 0), (256, 192), (256, 128), (128, 128)])
+@pytest.mark.parametrize("mnk", [(128, 128, 128), (300, 200, 512), (512, 768, 1024), (16, 4096, 4096),
+                                 (257, 129, 640), (64, 320, 1152), (130, 100, 2048)])
 def test_a8w8_accumulators_bit_exact(hip_lib, tile, mnk):
     M, N, K = mnk
     a, b = _rand_i8((M, K), 1), _rand_i8((N, K), 2)
