@@ -37,10 +37,19 @@ __device__ __forceinline__ double block_sum(double v, double* red) {
     return r;
 }
 
-// q = round_half_even(round_DT(x / s)) with x/s an IEEE fp32 division.
-template <int DT> __device__ __forceinline__ int quant_in_dtype(float x, float s) {
-    float t = x / s;
-    float th = bits_to_f32<DT>(f32_to_bits<DT>(t));
+// Correctly rounded fp32 quotient x / s from r = RN(1/s) (one IEEE division per row):
+// q0 = RN(x*r) is within 2 ulp, e = x - s*q0 is exact in an fma, and RN(q0 + e*r) is the rounded
+// quotient (Markstein).  Three instructions instead of the ~10 of a full division sequence.
+__device__ __forceinline__ float div_by(float x, float s, float r) {
+    const float q0 = x * r;
+    const float e = __builtin_fmaf(-q0, s, x);
+    return __builtin_fmaf(e, r, q0);
+}
+
+// q = round_half_even(round_DT(x / s)) with x/s a correctly rounded fp32 division.
+template <int DT> __device__ __forceinline__ int quant_in_dtype(float x, float s, float r) {
+    const float t = div_by(x, s, r);
+    const float th = bits_to_f32<DT>(f32_to_bits<DT>(t));
     return (int)rintf(th);
 }
 
@@ -74,6 +83,7 @@ __global__ __launch_bounds__(kRowThreads) void dynamic_quant_vec_kernel(
     const uint32_t sbits = f32_to_bits<DT>(mx / 127.0f);
     const float s = bits_to_f32<DT>(sbits);
     if (threadIdx.x == 0) scale[row] = (uint16_t)(DT == FNN_F16 ? sbits : f32_to_f16_bits(s));
+    const float rcp = 1.0f / s;
     v2u* qr = (v2u*)(q + row * ldq);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -82,8 +92,8 @@ __global__ __launch_bounds__(kRowThreads) void dynamic_quant_vec_kernel(
             int o[8];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                o[2 * j] = s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(v[i][j] & 0xFFFFu), s);
-                o[2 * j + 1] = s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(v[i][j] >> 16), s);
+                o[2 * j] = s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(v[i][j] & 0xFFFFu), s, rcp);
+                o[2 * j + 1] = s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(v[i][j] >> 16), s, rcp);
             }
             qr[idx] = v2u{pack4(o[0], o[1], o[2], o[3]), pack4(o[4], o[5], o[6], o[7])};
         }
@@ -103,16 +113,35 @@ __global__ __launch_bounds__(kRowThreads) void dynamic_quant_any_kernel(
     const uint32_t sbits = f32_to_bits<DT>(mx / 127.0f);
     const float s = bits_to_f32<DT>(sbits);
     if (threadIdx.x == 0) scale[row] = (uint16_t)(DT == FNN_F16 ? sbits : f32_to_f16_bits(s));
+    const float rcp = 1.0f / s;
     int8_t* qr = q + row * ldq;
     for (int k = threadIdx.x; k < K; k += kRowThreads)
-        qr[k] = (int8_t)(s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(xr[k]), s));
+        qr[k] = (int8_t)(s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(xr[k]), s, rcp));
 }
 
 // ---------------------------------------------------------------- rmsnorm + quant
-__device__ __forceinline__ int quant_clamped(float n, float s) {
-    float r = rintf(n / s);
+__device__ __forceinline__ int quant_clamped(float n, float s, float rcp) {
+    float r = rintf(div_by(n, s, rcp));
     r = fminf(fmaxf(r, -128.f), 127.f);
     return s == 0.f ? 0 : (int)r;
+}
+
+// 8 consecutive gamma values as fp32 (vector loads; the type branch is uniform)
+__device__ __forceinline__ void load_gamma8(const void* gamma, int gamma_dtype, int64_t first, float g[8]) {
+    if (gamma_dtype == FNN_F32) {
+        const v4f a = *(const v4f*)((const float*)gamma + first);
+        const v4f b = *(const v4f*)((const float*)gamma + first + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { g[j] = a[j]; g[4 + j] = b[j]; }
+    } else {
+        const v4u a = *(const v4u*)((const uint16_t*)gamma + first);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = a[j] & 0xFFFFu, hi = a[j] >> 16;
+            g[2 * j] = gamma_dtype == FNN_F16 ? f16_bits_to_f32(lo) : bf16_bits_to_f32(lo);
+            g[2 * j + 1] = gamma_dtype == FNN_F16 ? f16_bits_to_f32(hi) : bf16_bits_to_f32(hi);
+        }
+    }
 }
 
 template <int DT, int NV>
@@ -146,10 +175,11 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_vec_kernel(
     for (int i = 0; i < NV; ++i) {
         const int idx = threadIdx.x + i * kRowThreads;
         if (idx < nvec) {
+            float g[8];
+            load_gamma8(gamma, gamma_dtype, (int64_t)idx * 8, g);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float g = load_as_f32(gamma, (int64_t)idx * 8 + j, gamma_dtype);
-                n[i][j] = (n[i][j] * rs) * g;
+                n[i][j] = (n[i][j] * rs) * g[j];
                 mx = fmaxf(mx, fabsf(n[i][j]));
             }
         }
@@ -157,6 +187,7 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_vec_kernel(
     mx = block_max(mx, red);
     const float s = mx / 127.0f;
     if (threadIdx.x == 0) scale[row] = (uint16_t)f32_to_bits<DT>(s);
+    const float rcp = 1.0f / s;
     v2u* qr = (v2u*)(q + row * ldq);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -164,7 +195,7 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_vec_kernel(
         if (idx < nvec) {
             int o[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) o[j] = quant_clamped(n[i][j], s);
+            for (int j = 0; j < 8; ++j) o[j] = quant_clamped(n[i][j], s, rcp);
             qr[idx] = v2u{pack4(o[0], o[1], o[2], o[3]), pack4(o[4], o[5], o[6], o[7])};
         }
     }
@@ -194,10 +225,11 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_any_kernel(
     mx = block_max(mx, red);
     const float s = mx / 127.0f;
     if (threadIdx.x == 0) scale[row] = (uint16_t)f32_to_bits<DT>(s);
+    const float rcp = 1.0f / s;
     int8_t* qr = q + row * ldq;
     for (int k = threadIdx.x; k < K; k += kRowThreads) {
         const float nv = (bits_to_f32<DT>(xr[k]) * rs) * load_as_f32(gamma, k, gamma_dtype);
-        qr[k] = (int8_t)quant_clamped(nv, s);
+        qr[k] = (int8_t)quant_clamped(nv, s, rcp);
     }
 }
 
@@ -226,7 +258,7 @@ template <int DT>
 static void launch_rq(int8_t* q, uint16_t* scale, const uint16_t* x, const void* gamma, int gdt,
                       float eps, int64_t M, int K, int64_t ldx, int64_t ldq, hipStream_t st) {
     const dim3 grid((unsigned)M), block(kRowThreads);
-    if (vec_ok(x, q, K, ldx, ldq)) {
+    if (vec_ok(x, q, K, ldx, ldq) && ((uintptr_t)gamma % 16) == 0) {
         const int nv = (K / 8 + kRowThreads - 1) / kRowThreads;
         if (nv <= 1) rmsnorm_dquant_vec_kernel<DT, 1><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
         else if (nv <= 2) rmsnorm_dquant_vec_kernel<DT, 2><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
