@@ -49,7 +49,7 @@ struct A8W8Args {
 // K % 128 == 0, K >= 512.  K is walked in slabs of 128 bytes: every row piece a copy fetches
 // is one full 128-byte line, which is what the L2 -> LDS path needs to run at speed (64-byte
 // pieces reach little more than half the rate).  The LDS holds an asymmetric ring: three
-// stages for the a-rows (copied two slabs ahead) and two for the b-rows (one slab ahead);
+// stages for the a-rows (copied two slabs ahead, a third per k-step) and two for the b-rows (one slab ahead);
 // 3*BM + 2*BN rows of 128 bytes = 144 KB for a 256x192 tile.  There is one barrier per slab, at
 // the start of its LAST k-step: by then every fragment of the slab is in registers, so both of
 // its stages are free and are re-armed right after the barrier, and the barrier publishes the
@@ -113,12 +113,20 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
 #pragma unroll
     for (int j = 0; j < NLB; ++j)
         gob[j] = (uint32_t)min(n0 + (j * NWAVES + wave) * 8 + lrow, p.N - 1) * (uint32_t)p.ldb + lchunk * 16;
-    auto copy_a = [&](char* stage, int kt) {
+    // the a-copy of a slab is issued in three parts, one per k-step, so that the copy unit is fed
+    // evenly instead of receiving a burst that blocks the wave's issue (and its MFMAs) behind it
+    auto copy_a_part = [&](char* stage, int kt, int part) {
         const char* slab = (const char*)p.a + (int64_t)kt * BK;
 #pragma unroll
         for (int j = 0; j < NLA; ++j)
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + goa[j]),
-                                             (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
+            if (j * 3 / NLA == part)
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + goa[j]),
+                                                 (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
+    };
+    auto copy_a = [&](char* stage, int kt) {
+        copy_a_part(stage, kt, 0);
+        copy_a_part(stage, kt, 1);
+        copy_a_part(stage, kt, 2);
     };
     auto copy_b = [&](char* stage, int kt) {
         const char* slab = (const char*)p.b + (int64_t)kt * BK;
@@ -187,13 +195,17 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     };
 
     const int KT = p.K / BK;
-    // One slab = four k-steps.  `nsa`/`nsb` are the stages of the next slab (nullptr-free: the
-    // flags say whether there is one).  At the barrier the only copy that may stay in flight is
-    // the a-copy issued at the previous barrier (for the slab after next).
-    auto slab = [&](char* sa, char* sb, const char* nsa, const char* nsb, int j, bool steady) {
+    // One slab = four k-steps; slab j lives in (sa, sb), slab j+1 in (nsa, nsb), and `fa` is the
+    // a-stage freed at the previous barrier (it held slab j-1), into which the a-rows of slab j+2 are
+    // copied during k-steps 0..2.  At the barrier of the last k-step the b-stage of slab j is free
+    // and receives the b-rows of slab j+2.  Copy order per slab: a(j+2) parts, then b(j+2); at the
+    // barrier for slab j+1 the only copies that may still be in flight are those a(j+2) parts.
+    // (Also tried: b-copies in parts as well - slower, their lead time becomes too short.)
+    auto slab = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fa, int j, bool steady) {
 #pragma unroll
         for (int ks = 0; ks < 3; ++ks) {
             read_frags(sa, sb, ks + 1);
+            if (steady || j + 2 < KT) copy_a_part(fa, j + 2, ks);
             mfmas(ks & 1);
             interleave();
             __builtin_amdgcn_sched_barrier(0);
@@ -202,7 +214,6 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             wait_barrier(steady || j + 2 < KT);
             read_frags(nsa, nsb, 0);
             if (steady || j + 2 < KT) copy_b(sb, j + 2);
-            if (steady || j + 3 < KT) copy_a(sa, j + 3);
             mfmas(1);
             interleave();
         } else {
@@ -217,23 +228,22 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     wait_barrier(true);
     read_frags(sa0, sb0, 0);
     copy_b(sb1, 1);
-    copy_a(sa2, 2);
     int j = 0;
-    for (; j + 9 <= KT; j += 6) {   // every slab of the round still has both refills ahead of it
-        slab(sa0, sb0, sa1, sb1, j, true);
-        slab(sa1, sb1, sa2, sb0, j + 1, true);
-        slab(sa2, sb0, sa0, sb1, j + 2, true);
-        slab(sa0, sb1, sa1, sb0, j + 3, true);
-        slab(sa1, sb0, sa2, sb1, j + 4, true);
-        slab(sa2, sb1, sa0, sb0, j + 5, true);
+    for (; j + 8 <= KT; j += 6) {   // every slab of the round still has both refills ahead of it
+        slab(sa0, sb0, sa1, sb1, sa2, j, true);
+        slab(sa1, sb1, sa2, sb0, sa0, j + 1, true);
+        slab(sa2, sb0, sa0, sb1, sa1, j + 2, true);
+        slab(sa0, sb1, sa1, sb0, sa2, j + 3, true);
+        slab(sa1, sb0, sa2, sb1, sa0, j + 4, true);
+        slab(sa2, sb1, sa0, sb0, sa1, j + 5, true);
     }
-    for (; j < KT; j += 6) {        // the last three to eight slabs, with the refills guarded
-        slab(sa0, sb0, sa1, sb1, j, false);
-        if (j + 1 < KT) slab(sa1, sb1, sa2, sb0, j + 1, false);
-        if (j + 2 < KT) slab(sa2, sb0, sa0, sb1, j + 2, false);
-        if (j + 3 < KT) slab(sa0, sb1, sa1, sb0, j + 3, false);
-        if (j + 4 < KT) slab(sa1, sb0, sa2, sb1, j + 4, false);
-        if (j + 5 < KT) slab(sa2, sb1, sa0, sb0, j + 5, false);
+    for (; j < KT; j += 6) {        // the last two to seven slabs, with the refills guarded
+        slab(sa0, sb0, sa1, sb1, sa2, j, false);
+        if (j + 1 < KT) slab(sa1, sb1, sa2, sb0, sa0, j + 1, false);
+        if (j + 2 < KT) slab(sa2, sb0, sa0, sb1, sa1, j + 2, false);
+        if (j + 3 < KT) slab(sa0, sb1, sa1, sb0, sa2, j + 3, false);
+        if (j + 4 < KT) slab(sa1, sb0, sa2, sb1, sa0, j + 4, false);
+        if (j + 5 < KT) slab(sa2, sb1, sa0, sb0, sa1, j + 5, false);
     }
 
     // ---- epilogue ----
