@@ -804,12 +804,18 @@ __global__ __launch_bounds__(kGemvMaxWaves * 64) void gemm_wo_gemv_kernel(const 
         sv[u] = *(const v4u*)((const uint16_t*)p.scale + off);
         zv[u] = *(const v4u*)(zp_tab + off);
     }
-    v4u av[4][AB];
+    constexpr int MROWS = G128 ? (MP < 4 ? MP : 4) : 4;   // activation rows staged (M <= MROWS)
+    v4u av[MROWS][AB];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
+    for (int m = 0; m < MROWS; ++m) {
         const v4u* src = (const v4u*)((const uint16_t*)p.act + (int64_t)min(m, p.M - 1) * p.lda);
 #pragma unroll
-        for (int u = 0; u < AB; ++u) av[m][u] = src[min(u * nt + (int)threadIdx.x, chunks - 1)];
+        for (int u = 0; u < AB; ++u) {
+            // batches beyond the row length are skipped (uniform), not clamped: a clamped batch would
+            // still cost the copy unit a full instruction per wave
+            if (u * nt < chunks) av[m][u] = src[min(u * nt + (int)threadIdx.x, chunks - 1)];
+            else av[m][u] = v4u{0, 0, 0, 0};
+        }
     }
     v4u wq[UN];
 #pragma unroll
@@ -839,7 +845,7 @@ __global__ __launch_bounds__(kGemvMaxWaves * 64) void gemm_wo_gemv_kernel(const 
         }
     }
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
+    for (int m = 0; m < MROWS; ++m) {
         v4u* dst = (v4u*)(a_lds + m * a_stride);
 #pragma unroll
         for (int u = 0; u < AB; ++u) {
