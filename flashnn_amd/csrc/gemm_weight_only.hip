@@ -26,97 +26,10 @@
 // flashnn/triton_kernels/gemm_a16w4.py:163-182 (nibble order), :296-297 (scale rows).
 #include "fnn_common.h"
 
+#include "wo_common.h"
+
 namespace fnn {
 
-struct WoArgs {
-    const void* act;
-    const int8_t* qw;
-    const void* scale;
-    const void* zp;
-    const void* bias;
-    void* out;
-    int M, N, K;          // N = output channels
-    int64_t lda, ldw, ldc;
-    int group;            // 0 = per channel
-    int out_dtype, scale_dtype, zp_dtype, bias_dtype;
-    int m_base;           // first activation row handled by this launch
-};
-
-constexpr int kWoWaves = 8;
-constexpr int kPF = 8;    // weight loads in flight per lane
-constexpr int kPFA = 2;   // activation steps in flight per lane
-
-template <int ADT> struct MfmaT;
-template <> struct MfmaT<FNN_F16> {
-    typedef v8h vec;
-    static constexpr uint32_t one2 = 0x3C003C00u;
-    __device__ static __forceinline__ v4f mma(v4u a, v4u b, v4f c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a),
-                                                      __builtin_bit_cast(v8h, b), c, 0, 0, 0);
-    }
-};
-template <> struct MfmaT<FNN_BF16> {
-    typedef v8bf vec;
-    static constexpr uint32_t one2 = 0x3F803F80u;
-    __device__ static __forceinline__ v4f mma(v4u a, v4u b, v4f c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a),
-                                                       __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
-    }
-};
-
-// 16 int8 (k .. k+15 of one row) -> two MFMA operands in natural k order.
-// Values come out as c + (v + 128) with c = 1024 (fp16) or 0 (bf16).
-template <int ADT>
-__device__ __forceinline__ void convert_w8(const v4u w, v4u& s0, v4u& s1) {
-    uint32_t o[8];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const uint32_t x = w[q] ^ 0x80808080u;
-        if constexpr (ADT == FNN_F16) {
-            o[2 * q] = __builtin_amdgcn_perm(x, 0x64646464u, 0x00050004u);
-            o[2 * q + 1] = __builtin_amdgcn_perm(x, 0x64646464u, 0x00070006u);
-        } else {
-            const uint32_t f0 = __float_as_uint((float)(x & 0xFFu));
-            const uint32_t f1 = __float_as_uint((float)((x >> 8) & 0xFFu));
-            const uint32_t f2 = __float_as_uint((float)((x >> 16) & 0xFFu));
-            const uint32_t f3 = __float_as_uint((float)(x >> 24));
-            o[2 * q] = __builtin_amdgcn_perm(f1, f0, 0x07060302u);
-            o[2 * q + 1] = __builtin_amdgcn_perm(f3, f2, 0x07060302u);
-        }
-    }
-    s0 = v4u{o[0], o[1], o[2], o[3]};
-    s1 = v4u{o[4], o[5], o[6], o[7]};
-}
-
-// 16 bytes = 16 k of two channels (low nibble: even channel).  Each operand holds k in the
-// order (0,2)(1,3)(4,6)(5,7); values are c + (v + 8), c = 1024 (fp16) / 128 (bf16).
-template <int ADT>
-__device__ __forceinline__ void convert_w4(const v4u w, v4u& e0, v4u& e1, v4u& o0, v4u& o1) {
-    // (x & 0x000F000F) ^ c with c = exponent bits | 0x0008 per half: the xor both flips the
-    // nibble's sign bit (two's complement -> offset by 8) and sets the exponent, because the two
-    // bit sets are disjoint.  One 3-input bit operation per pair of weights.
-    constexpr uint32_t msk = 0x000F000Fu;
-    constexpr uint32_t cst = (ADT == FNN_F16 ? 0x64006400u : 0x43004300u) ^ 0x00080008u;
-    uint32_t e[8], o[8];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const uint32_t x = w[q];
-        e[2 * q] = (x & msk) ^ cst;
-        e[2 * q + 1] = ((x >> 8) & msk) ^ cst;
-        o[2 * q] = ((x >> 4) & msk) ^ cst;
-        o[2 * q + 1] = ((x >> 12) & msk) ^ cst;
-    }
-    e0 = v4u{e[0], e[1], e[2], e[3]};
-    e1 = v4u{e[4], e[5], e[6], e[7]};
-    o0 = v4u{o[0], o[1], o[2], o[3]};
-    o1 = v4u{o[4], o[5], o[6], o[7]};
-}
-
-// reorder 8 consecutive 16-bit values to (0,2)(1,3)(4,6)(5,7)
-__device__ __forceinline__ v4u perm_act_w4(const v4u a) {
-    return v4u{__builtin_amdgcn_perm(a[1], a[0], 0x05040100u), __builtin_amdgcn_perm(a[1], a[0], 0x07060302u),
-               __builtin_amdgcn_perm(a[3], a[2], 0x05040100u), __builtin_amdgcn_perm(a[3], a[2], 0x07060302u)};
-}
 
 template <int WBITS, int ADT, int MB, bool GROUPED>
 __global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoArgs p) {
@@ -1112,6 +1025,7 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
         return;
     }
     if (launch_decode<WBITS, ADT>(p, st)) return;
+    if (launch_wo_panel(p, WBITS, ADT, st)) return;
     // up to 64 activation rows per pass over the weights
     for (int m0 = 0; m0 < p.M; m0 += 64) {
         p.m_base = m0;

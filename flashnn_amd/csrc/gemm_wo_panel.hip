@@ -1,0 +1,385 @@
+// Weight-only GEMM for 9 .. a few hundred activation rows ("panel" kernel, gfx950).
+//
+// The weights are still read exactly once per pass and go straight from global memory into the
+// MFMA "A" operand; what changes against the decode kernels is the activation side.  With 16..64
+// activation rows every weight tile needs M*K*2 bytes of activations, too much to pull through
+// the vector memory path once per 16 weight rows.  Here a workgroup owns 64 weight rows (four
+// waves, 16 rows each) and the four waves share each 128-k slab of the activation panel through
+// LDS:
+//   * 4*KS waves; wave (rt, ks) owns weight rows 16*rt .. +15 of the tile and the ks-th part of K;
+//   * activations: slabs of (16*MB rows) x 128 k are copied global -> LDS with 16-byte
+//     direct-to-LDS loads into a ring of 4 stages (3 slabs ahead).  The 16-byte chunks of a row
+//     are stored at slot (chunk ^ (row & 15)) so that the 16 lanes that read the same chunk of 16
+//     different rows hit 16 different bank groups;
+//   * weights: two 16-byte loads per lane and slab, kept 4 slabs ahead in registers; the refill
+//     of a register is issued after its last use, so the queue needs no copies;
+//   * group scales and zero points (group == 128): one 16-byte load each per lane and slab,
+//     4 slabs ahead, folded into the running output at the end of each slab:
+//         out += s * (acc - (c + zp) * sum_k a_k),
+//     c being the constant the exponent-trick conversion adds, sum_k a_k coming from an MFMA
+//     against ones;
+//   * all loads of an iteration are issued in a fixed order, so "slab j has landed" is one
+//     s_waitcnt vmcnt(X) with a compile-time X, followed by a bare s_barrier;
+//   * the K parts are added through LDS in a fixed order, then bias, rounding, 16-byte stores.
+//
+// Reference semantics: flashnn/quant_gemm.py:148-206.
+#include <type_traits>
+
+#include "wo_common.h"
+
+namespace fnn {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+// 16 bytes = 16 k of two channels -> operands in natural k order (one byte shuffle per dword
+// puts the nibbles of k and k+1 into the two halves of a dword).
+template <int ADT>
+__device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4u& o0, v4u& o1) {
+    constexpr uint32_t msk = 0x000F000Fu;
+    constexpr uint32_t cst = (ADT == FNN_F16 ? 0x64006400u : 0x43004300u) ^ 0x00080008u;
+    uint32_t e[8], o[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t y = __builtin_amdgcn_perm(w[q], w[q], 0x03010200u);   // bytes k0 k2 k1 k3
+        e[2 * q] = (y & msk) ^ cst;
+        e[2 * q + 1] = ((y >> 8) & msk) ^ cst;
+        o[2 * q] = ((y >> 4) & msk) ^ cst;
+        o[2 * q + 1] = ((y >> 12) & msk) ^ cst;
+    }
+    e0 = v4u{e[0], e[1], e[2], e[3]};
+    e1 = v4u{e[4], e[5], e[6], e[7]};
+    o0 = v4u{o[0], o[1], o[2], o[3]};
+    o1 = v4u{o[4], o[5], o[6], o[7]};
+}
+
+// G128: per-group tables with group size 128, entries of type SDT (fp16 or bf16), zero points in
+// the same type; otherwise per-channel scales of any type, applied once at the end.
+template <int WBITS, int ADT, bool G128, int SDT, int MB, int KS>
+__global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p, const int passes) {
+    typedef MfmaT<ADT> MT;
+    constexpr int NH = WBITS == 4 ? 2 : 1;      // channels per weight row
+    constexpr int NCL = 4 * NH;                 // consecutive channels per lane
+    constexpr float c_off = WBITS == 4 ? (ADT == FNN_F16 ? 1024.f + 8.f : 128.f + 8.f)
+                                       : (ADT == FNN_F16 ? 1024.f + 128.f : 128.f);
+    constexpr int SLAB = MB * 16 * 256;         // bytes of one activation slab: 16*MB rows x 128 k
+    constexpr int STG = KS * SLAB;
+    constexpr int RED = KS > 1 ? (KS - 1) * 4 * MB * NH * 4 * 64 * 4 : 16;
+    constexpr int STG0 = STG > RED ? STG : RED;
+    // one array per stage: the compiler then knows that reads of one stage cannot alias the
+    // copies in flight into another
+    __shared__ __attribute__((aligned(16))) char st0[STG0];
+    __shared__ __attribute__((aligned(16))) char st1[STG];
+    __shared__ __attribute__((aligned(16))) char st2[STG];
+    __shared__ __attribute__((aligned(16))) char st3[STG];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rt = wave & 3;
+    const int ks = wave >> 2;
+    const int li = lane & 15;
+    const int lg = lane >> 4;
+
+    // workgroups id, id+8, id+16 .. run on the same XCD: give them the same weight tile and
+    // consecutive passes so that the tile is fetched from HBM once and re-read from that L2
+    const int wrows = WBITS == 4 ? p.N / 2 : p.N;
+    const int tiles = wrows / 64;
+    const int y = blockIdx.x >> 3;
+    const int pass = y % passes;
+    const int tile = (y / passes) * 8 + (blockIdx.x & 7);
+    if (tile >= tiles) return;
+    const int m_base = p.m_base + pass * (MB * 16);
+    const int row0 = tile * 64 + rt * 16;
+
+    const int nsl = p.K / (128 * KS);           // slabs per K part (multiple of 4)
+    const int sl0 = ks * nsl;
+
+    const char* wptr = (const char*)p.qw + (int64_t)(row0 + li) * p.ldw + lg * 16 + (int64_t)sl0 * 128;
+    auto load_w = [&](int jj, int half) -> v4u {
+        const int j = min(jj, nsl - 1);
+        return *(const v4u*)(wptr + (int64_t)j * 128 + half * 64);
+    };
+
+    // ---- activation copies: thread t of the K part copies chunk (t & 15) ^ (t >> 4) of rows
+    // (t >> 4) + 16 i into slot (t & 15) of those rows
+    const int t = rt * 64 + lane;
+    const int tokq = t >> 4;
+    const int chunk = (t & 15) ^ tokq;
+    const char* act_part = (const char*)p.act + (int64_t)sl0 * 256 + chunk * 16;
+    int64_t goff[MB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+        goff[i] = (int64_t)min(m_base + i * 16 + tokq, p.M - 1) * p.lda * 2;
+    auto copy_act = [&](char* stage, int jj) {
+        const int j = min(jj, nsl - 1);
+        const char* src = act_part + (int64_t)j * 256;
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + goff[i]),
+                                             (lds_ptr_t)(stage + ks * SLAB + (i * 256 + rt * 64) * 16), 16, 0, 0);
+    };
+    // ---- activation fragment reads: lane (li, lg) reads chunks 8 s + 2 lg + h of row 16 mb + li
+    int rd[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) rd[s][h] = ks * SLAB + li * 256 + (((s * 8 + lg * 2 + h) ^ li) << 4);
+
+    // ---- group tables: NCL consecutive channels per lane
+    typedef typename std::conditional<NH == 2, v4u, v2u>::type tab_t;
+    const int n0 = NH * (row0 + 4 * lg);
+    const uint16_t* sptr = (const uint16_t*)p.scale + (int64_t)sl0 * p.N + n0;
+    const uint16_t* zptr = (p.zp ? (const uint16_t*)p.zp : (const uint16_t*)p.scale) + (int64_t)sl0 * p.N + n0;
+    const bool has_zp = p.zp != nullptr;
+    // without zero points the second table load reads the scales again and is multiplied away
+    const float zmul = has_zp ? 1.f : 0.f;
+    auto load_tab = [&](const uint16_t* base, int jj) -> tab_t {
+        const int j = min(jj, nsl - 1);
+        return *(const tab_t*)(base + (int64_t)j * p.N);
+    };
+
+    v4f outv[MB][NH], accg[MB][NH], asum[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        asum[mb] = v4f{0, 0, 0, 0};
+#pragma unroll
+        for (int h = 0; h < NH; ++h) { outv[mb][h] = v4f{0, 0, 0, 0}; accg[mb][h] = v4f{0, 0, 0, 0}; }
+    }
+    const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+
+    // loads issued per iteration, in this order: MB copies, 2 weight loads, 2 table loads
+    constexpr int C = MB + 2 + (G128 ? 2 : 0);
+    // the newest load slab j depends on is its last copy, issued three iterations earlier; after
+    // it came the rest of that iteration and two whole ones
+    constexpr int X = (C - MB) + 2 * C;
+    static_assert(X < 64, "vmcnt range");
+    auto wait_barrier = [&]() {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0070 | (X & 15) | ((X >> 4) << 14));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);   // nothing of the slab's work moves above the wait
+    };
+
+    v4u wq[4][2];
+    tab_t sq[4], zq[4];
+
+    auto fold = [&](const tab_t sv, const tab_t zv) {
+        float sc[NCL], zc[NCL];
+#pragma unroll
+        for (int c = 0; c < NCL; ++c) {
+            const uint32_t sb = (sv[c >> 1] >> (16 * (c & 1))) & 0xFFFFu;
+            const uint32_t zb = (zv[c >> 1] >> (16 * (c & 1))) & 0xFFFFu;
+            sc[c] = bits_to_f32<SDT>(sb);
+            zc[c] = c_off + zmul * bits_to_f32<SDT>(zb);
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int c = NH == 2 ? 2 * r + h : r;
+                    outv[mb][h][r] += sc[c] * (accg[mb][h][r] - zc[c] * asum[mb][r]);
+                    accg[mb][h][r] = 0.f;
+                }
+            asum[mb] = v4f{0, 0, 0, 0};
+        }
+    };
+
+    auto compute = [&](const char* stage, const v4u w0, const v4u w1) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const v4u w = s == 0 ? w0 : w1;
+            if constexpr (WBITS == 4) {
+                v4u e0, e1, o0, o1;
+                convert_w4_nat<ADT>(w, e0, e1, o0, o1);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const v4u b0 = *(const v4u*)(stage + rd[s][0] + mb * 4096);
+                    const v4u b1 = *(const v4u*)(stage + rd[s][1] + mb * 4096);
+                    accg[mb][0] = MT::mma(e0, b0, accg[mb][0]);
+                    accg[mb][1] = MT::mma(o0, b0, accg[mb][1]);
+                    asum[mb] = MT::mma(ones, b0, asum[mb]);
+                    accg[mb][0] = MT::mma(e1, b1, accg[mb][0]);
+                    accg[mb][1] = MT::mma(o1, b1, accg[mb][1]);
+                    asum[mb] = MT::mma(ones, b1, asum[mb]);
+                }
+            } else {
+                v4u s0, s1;
+                convert_w8<ADT>(w, s0, s1);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const v4u b0 = *(const v4u*)(stage + rd[s][0] + mb * 4096);
+                    const v4u b1 = *(const v4u*)(stage + rd[s][1] + mb * 4096);
+                    accg[mb][0] = MT::mma(s0, b0, accg[mb][0]);
+                    asum[mb] = MT::mma(ones, b0, asum[mb]);
+                    accg[mb][0] = MT::mma(s1, b1, accg[mb][0]);
+                    asum[mb] = MT::mma(ones, b1, asum[mb]);
+                }
+            }
+        }
+    };
+
+#define FNN_PANEL_ITER(Q, CUR, FREE, JJ)                                   \
+    do {                                                                   \
+        wait_barrier();                                                    \
+        copy_act(FREE, (JJ) + 3);                                          \
+        compute(CUR, wq[Q][0], wq[Q][1]);                                  \
+        if constexpr (G128) fold(sq[Q], zq[Q]);                            \
+        wq[Q][0] = load_w((JJ) + 4, 0);                                    \
+        wq[Q][1] = load_w((JJ) + 4, 1);                                    \
+        if constexpr (G128) {                                              \
+            sq[Q] = load_tab(sptr, (JJ) + 4);                              \
+            zq[Q] = load_tab(zptr, (JJ) + 4);                              \
+        }                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                 \
+    } while (0)
+
+    // ---- prologue: the same issue order as three iterations before the first one
+    wq[0][0] = load_w(0, 0);
+    wq[0][1] = load_w(0, 1);
+    if constexpr (G128) { sq[0] = load_tab(sptr, 0); zq[0] = load_tab(zptr, 0); }
+    __builtin_amdgcn_sched_barrier(0);
+    copy_act(st0, 0);
+    wq[1][0] = load_w(1, 0);
+    wq[1][1] = load_w(1, 1);
+    if constexpr (G128) { sq[1] = load_tab(sptr, 1); zq[1] = load_tab(zptr, 1); }
+    __builtin_amdgcn_sched_barrier(0);
+    copy_act(st1, 1);
+    wq[2][0] = load_w(2, 0);
+    wq[2][1] = load_w(2, 1);
+    if constexpr (G128) { sq[2] = load_tab(sptr, 2); zq[2] = load_tab(zptr, 2); }
+    __builtin_amdgcn_sched_barrier(0);
+    copy_act(st2, 2);
+    wq[3][0] = load_w(3, 0);
+    wq[3][1] = load_w(3, 1);
+    if constexpr (G128) { sq[3] = load_tab(sptr, 3); zq[3] = load_tab(zptr, 3); }
+    __builtin_amdgcn_sched_barrier(0);
+
+    for (int jj = 0; jj < nsl; jj += 4) {
+        FNN_PANEL_ITER(0, st0, st3, jj);
+        FNN_PANEL_ITER(1, st1, st0, jj + 1);
+        FNN_PANEL_ITER(2, st2, st1, jj + 2);
+        FNN_PANEL_ITER(3, st3, st2, jj + 3);
+    }
+#undef FNN_PANEL_ITER
+
+    // ---- per-channel scales: one fold at the end
+    if constexpr (!G128) {
+        float sc[NCL], zc[NCL];
+#pragma unroll
+        for (int c = 0; c < NCL; ++c) {
+            sc[c] = load_as_f32(p.scale, n0 + c, p.scale_dtype);
+            zc[c] = c_off + (has_zp ? load_as_f32(p.zp, n0 + c, p.zp_dtype) : 0.f);
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int c = NH == 2 ? 2 * r + h : r;
+                    outv[mb][h][r] = sc[c] * (accg[mb][h][r] - zc[c] * asum[mb][r]);
+                }
+    }
+
+    // ---- add the K parts in order (the stages are idle once every copy has landed)
+    if constexpr (KS > 1) {
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        float* red = (float*)st0;
+        if (ks > 0) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int h = 0; h < NH; ++h)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        red[(((((ks - 1) * 4 + rt) * MB + mb) * NH + h) * 4 + r) * 64 + lane] = outv[mb][h][r];
+        }
+        __syncthreads();
+        if (ks > 0) return;
+#pragma unroll
+        for (int k2 = 1; k2 < KS; ++k2)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int h = 0; h < NH; ++h)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        outv[mb][h][r] += red[(((((k2 - 1) * 4 + rt) * MB + mb) * NH + h) * 4 + r) * 64 + lane];
+    }
+
+    // ---- bias, rounding, store: lane (li, lg) holds channels n0 .. n0+NCL-1 of row 16 mb + li
+    float bias[NCL];
+#pragma unroll
+    for (int c = 0; c < NCL; ++c) bias[c] = p.bias ? load_as_f32(p.bias, n0 + c, p.bias_dtype) : 0.f;
+    const bool vec_out = (p.ldc * 2) % (NCL * 2) == 0 && ((uintptr_t)p.out % (NCL * 2)) == 0;
+    const bool out_f16 = p.out_dtype == FNN_F16;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = m_base + mb * 16 + li;
+        if (m >= p.M) continue;
+        uint32_t pk[NCL / 2];
+#pragma unroll
+        for (int c = 0; c < NCL; c += 2) {
+            const float v0 = (NH == 2 ? outv[mb][0][c >> 1] : outv[mb][0][c]) + bias[c];
+            const float v1 = (NH == 2 ? outv[mb][1][c >> 1] : outv[mb][0][c + 1]) + bias[c + 1];
+            const uint32_t b0 = out_f16 ? f32_to_f16_bits(v0) : f32_to_bf16_bits(v0);
+            const uint32_t b1 = out_f16 ? f32_to_f16_bits(v1) : f32_to_bf16_bits(v1);
+            pk[c >> 1] = (b0 & 0xFFFFu) | (b1 << 16);
+        }
+        uint16_t* dst = (uint16_t*)p.out + (int64_t)m * p.ldc + n0;
+        if (vec_out) {
+            if constexpr (NH == 2) *(v4u*)dst = v4u{pk[0], pk[1], pk[2], pk[3]};
+            else *(v2u*)dst = v2u{pk[0], pk[1]};
+        } else {
+#pragma unroll
+            for (int c = 0; c < NCL; ++c) dst[c] = (uint16_t)(pk[c >> 1] >> (16 * (c & 1)));
+        }
+    }
+}
+
+// Launches the panel kernel if the shape suits it; returns false otherwise.
+template <int WBITS, int ADT>
+static bool launch_panel_t(WoArgs& p, hipStream_t st) {
+    constexpr int NH = WBITS == 4 ? 2 : 1;
+    const int wrows = WBITS == 4 ? p.N / 2 : p.N;
+    if (wrows % 64 != 0 || p.K % 1024 != 0) return false;
+    if (p.group != 0 && p.group != 128) return false;
+    if (p.group == 128) {
+        const bool tables16 = is16(p.scale_dtype) && (!p.zp || p.zp_dtype == p.scale_dtype) &&
+                              p.N % (4 * NH) == 0 && ((uintptr_t)p.scale % (8 * NH)) == 0 &&
+                              (!p.zp || ((uintptr_t)p.zp % (8 * NH)) == 0);
+        if (!tables16) return false;
+    }
+    const int tiles = wrows / 64;
+    if (tiles < 128) return false;   // too few workgroups to fill the chip: the streaming kernel splits K further
+    const int mb = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
+    const int passes = (p.M + mb * 16 - 1) / (mb * 16);
+    const dim3 grid(((tiles + 7) / 8) * 8 * passes);
+    p.m_base = 0;
+#define FNN_PANEL(G, SDTV)                                                                               \
+    do {                                                                                                 \
+        if (mb == 1) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, 1, 2><<<grid, dim3(512), 0, st>>>(p, passes);      \
+        else if (mb == 2) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, 2, 2><<<grid, dim3(512), 0, st>>>(p, passes); \
+        else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, 4, 2><<<grid, dim3(512), 0, st>>>(p, passes);              \
+    } while (0)
+    if (p.group == 128) {
+        if (p.scale_dtype == FNN_F16) FNN_PANEL(true, FNN_F16);
+        else FNN_PANEL(true, FNN_BF16);
+    } else {
+        FNN_PANEL(false, FNN_F16);
+    }
+#undef FNN_PANEL
+    return true;
+}
+
+bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st) {
+    if (wbits == 4) return act_dtype == FNN_F16 ? launch_panel_t<4, FNN_F16>(p, st) : launch_panel_t<4, FNN_BF16>(p, st);
+    return act_dtype == FNN_F16 ? launch_panel_t<8, FNN_F16>(p, st) : launch_panel_t<8, FNN_BF16>(p, st);
+}
+
+}  // namespace fnn

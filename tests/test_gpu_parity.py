@@ -235,6 +235,36 @@ def test_weight_only_reference_test_shape():
                 _wo_check(*case, group, 8, torch.float16)
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("group", [0, 128])
+@pytest.mark.parametrize("M,K", [(9, 1024), (16, 2048), (33, 1024), (64, 2048), (100, 1024)])
+def test_weight_only_many_rows(bits, group, M, K):
+    """9 .. 100 activation rows over >= 8192 weight rows: the kernel that shares activation slabs
+    between four weight tiles (one, two and four 16-row blocks per pass, one and two passes)."""
+    N = 8192 * (2 if bits == 4 else 1)
+    act_ty = torch.float16 if M % 2 else torch.bfloat16
+    scale_ty = torch.bfloat16 if M == 33 else torch.float16
+    case = _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp=M != 16, with_bias=M in (9, 64), seed=M)
+    _wo_check(*case, group, bits, act_ty)
+
+
+def test_weight_only_many_rows_one_hot():
+    """Rows of the activation matrix that hold a single non-zero entry pick single weight columns:
+    checks the k order inside the slabs and the row -> output mapping exactly."""
+    M, N, K = 48, 16384, 2048
+    g = torch.Generator().manual_seed(77)
+    w = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(K // 128, N).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(-4, 4, (K // 128, N), generator=g).half()
+    ks = torch.randperm(K, generator=g)[:M]
+    act = torch.zeros(M, K, dtype=torch.float16)
+    act[torch.arange(M), ks] = 2.0
+    qw = torch.from_numpy(O.pack_int4(w.numpy()))
+    out = flashnn_amd.GemmWeightOnly(torch.float16)(act.to(DEV), qw.to(DEV), scale.to(DEV), None, zp.to(DEV))
+    want = 2.0 * (w[:, ks].float() - zp[ks // 128].float().t()) * scale[ks // 128].float().t()   # [N, M]
+    np.testing.assert_allclose(out.float().cpu().numpy(), want.t().half().float().numpy(), rtol=2.0 ** -10, atol=1e-6)
+
+
 @pytest.mark.parametrize("M", [1, 8, 32])
 @pytest.mark.parametrize("kn", workloads.A16W8_DECODE_SHAPES)
 def test_a16w8_decode_config(M, kn):
