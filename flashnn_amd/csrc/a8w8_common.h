@@ -1,0 +1,26 @@
+// Argument block and output modes shared by the A8W8 GEMM kernels.
+#pragma once
+
+#include "fnn_common.h"
+
+namespace fnn {
+
+enum { OUT_F16 = 0, OUT_BF16 = 1, OUT_I32 = 2 };
+
+struct A8W8Args {
+    const int8_t* a;
+    const int8_t* b;
+    void* out;
+    const void* arow;
+    const void* acol;
+    int M, N, K;
+    int64_t lda, ldb, ldc;
+    int out_dtype, arow_dtype, acol_dtype;
+    int tiles_m, tiles_n, tiles_per_xcd;
+};
+
+// gemm_a8w8_skinny.hip: up to 64 activation rows, the weights streamed once; false if the shape
+// does not suit it
+bool launch_a8w8_skinny(A8W8Args& p, int mode, hipStream_t st);
+
+}  // namespace fnn

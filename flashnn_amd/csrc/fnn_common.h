@@ -44,6 +44,13 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
     return c.u;
 }
 
+// Pins an fp32 value: the compiler otherwise fuses a multiplication with the conversion that
+// follows it into v_fma_mixlo_f16, which rounds once where the reference rounds twice.
+__device__ __forceinline__ float rounded_f32(float f) {
+    asm volatile("" : "+v"(f));
+    return f;
+}
+
 template <int DT> __device__ __forceinline__ float bits_to_f32(uint32_t h) {
     if constexpr (DT == FNN_F16) return f16_bits_to_f32(h);
     else return bf16_bits_to_f32(h);

@@ -21,7 +21,11 @@
 // Any other shape takes a small guarded LDS kernel built on v_dot4_i32_i8.
 //
 // Reference for the semantics: flashnn/triton_kernels/gemm_a8w8.py:74-179.
-#include "fnn_common.h"
+#include "a8w8_common.h"
+
+// The scaled output is two fp32 multiplications and one rounding to 16 bits, each rounded on its
+// own as in the reference's torch path.
+#pragma clang fp contract(off)
 
 namespace fnn {
 
@@ -30,19 +34,6 @@ constexpr int BK = 128;  // bytes of K per LDS slab row
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
-enum { OUT_F16 = 0, OUT_BF16 = 1, OUT_I32 = 2 };
-
-struct A8W8Args {
-    const int8_t* a;
-    const int8_t* b;
-    void* out;
-    const void* arow;
-    const void* acol;
-    int M, N, K;
-    int64_t lda, ldb, ldc;
-    int out_dtype, arow_dtype, acol_dtype;
-    int tiles_m, tiles_n, tiles_per_xcd;
-};
 
 
 // ------------------------------------------------------------------ main MFMA kernel
@@ -384,7 +375,7 @@ __global__ __launch_bounds__(256) void gemm_a8w8_any_kernel(const A8W8Args p) {
             if constexpr (MODE == OUT_I32) {
                 ((int32_t*)p.out)[(int64_t)m * p.ldc + n] = acc[i][j];
             } else {
-                const float v = ((float)acc[i][j] * ar) * load_as_f32(p.acol, n, p.acol_dtype);
+                const float v = rounded_f32(((float)acc[i][j] * ar) * load_as_f32(p.acol, n, p.acol_dtype));
                 store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
             }
         }
@@ -425,6 +416,8 @@ static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
                       ((uintptr_t)p.a % 16) == 0 && ((uintptr_t)p.b % 16) == 0 &&
                       ((uintptr_t)p.out % 16) == 0 && (int64_t)p.M * p.lda < (1LL << 31) &&
                       (int64_t)p.N * p.ldb < (1LL << 31);
+    // few activation rows: stream the weights once (unless a test forces a tile of the tiled kernel)
+    if (force_bm == 0 && p.M <= 64 && launch_a8w8_skinny(p, MODE, st)) return;
     if (!fast) {
         gemm_a8w8_any_kernel<MODE><<<dim3((p.N + 63) / 64, (p.M + 63) / 64), dim3(256), 0, st>>>(p);
         return;

@@ -11,8 +11,9 @@
 //     direct-to-LDS loads into a ring of 4 stages (3 slabs ahead).  The 16-byte chunks of a row
 //     are stored at slot (chunk ^ (row & 15)) so that the 16 lanes that read the same chunk of 16
 //     different rows hit 16 different bank groups;
-//   * weights: two 16-byte loads per lane and slab, kept 4 slabs ahead in registers; the refill
-//     of a register is issued after its last use, so the queue needs no copies;
+//   * weights: two 16-byte loads per lane and slab, kept 4 slabs ahead in registers and fetched
+//     as full 128-byte lines (8 rows per load); a wave-private LDS staging area reshapes them into
+//     the MFMA operand layout; the refill of a register is issued right after its last use;
 //   * group scales and zero points (group == 128): one 16-byte load each per lane and slab,
 //     4 slabs ahead, folded into the running output at the end of each slab:
 //         out += s * (acc - (c + zp) * sum_k a_k),
@@ -55,7 +56,8 @@ __device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4
 
 // G128: per-group tables with group size 128, entries of type SDT (fp16 or bf16), zero points in
 // the same type; otherwise per-channel scales of any type, applied once at the end.
-template <int WBITS, int ADT, bool G128, int SDT, int MB, int KS>
+// D: slabs of weights in flight per wave (4 or 8); the K part of a wave holds a multiple of D slabs.
+template <int WBITS, int ADT, bool G128, int SDT, int MB, int KS, int D>
 __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p, const int passes) {
     typedef MfmaT<ADT> MT;
     constexpr int NH = WBITS == 4 ? 2 : 1;      // channels per weight row
@@ -72,6 +74,7 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
     __shared__ __attribute__((aligned(16))) char st1[STG];
     __shared__ __attribute__((aligned(16))) char st2[STG];
     __shared__ __attribute__((aligned(16))) char st3[STG];
+    __shared__ __attribute__((aligned(16))) char wst[4 * KS * 2048];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -94,11 +97,24 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
     const int nsl = p.K / (128 * KS);           // slabs per K part (multiple of 4)
     const int sl0 = ks * nsl;
 
-    const char* wptr = (const char*)p.qw + (int64_t)(row0 + li) * p.ldw + lg * 16 + (int64_t)sl0 * 128;
+    // ---- weights: load h of a slab fetches rows 8h .. 8h+7 of the wave's tile, 8 lanes per row, one
+    // full 128-byte line per row (16 rows x 64 bytes per load, the MFMA operand's own shape, streams
+    // a quarter slower from HBM).  A wave-private 2 KB staging area in LDS turns the two loads
+    // into the operand layout: row i at i*128, its 16-byte chunk c at slot c ^ ((i >> 1) & 7).
+    const int wr8 = lane >> 3, wc8 = lane & 7;
+    const char* wptr = (const char*)p.qw + (int64_t)(row0 + wr8) * p.ldw + wc8 * 16 + (int64_t)sl0 * 128;
+    const int64_t w_half = 8 * p.ldw;
     auto load_w = [&](int jj, int half) -> v4u {
         const int j = min(jj, nsl - 1);
-        return *(const v4u*)(wptr + (int64_t)j * 128 + half * 64);
+        return *(const v4u*)(wptr + (int64_t)j * 128 + half * w_half);
     };
+    char* const wmine = wst + wave * 2048;
+    int wwr[2], wrd[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        wwr[h] = (8 * h + wr8) * 128 + ((wc8 ^ ((4 * h + (wr8 >> 1)) & 7)) << 4);
+        wrd[h] = li * 128 + (((4 * h + lg) ^ ((li >> 1) & 7)) << 4);
+    }
 
     // ---- activation copies: thread t of the K part copies chunk (t & 15) ^ (t >> 4) of rows
     // (t >> 4) + 16 i into slot (t & 15) of those rows
@@ -161,7 +177,7 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
         __builtin_amdgcn_sched_barrier(0);   // nothing of the slab's work moves above the wait
     };
 
-    v4u wq[4][2];
+    v4u wq[D][2];
     tab_t sq[4], zq[4];
 
     auto fold = [&](const tab_t sv, const tab_t zv) {
@@ -221,14 +237,17 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
         }
     };
 
-#define FNN_PANEL_ITER(Q, CUR, FREE, JJ)                                   \
+#define FNN_PANEL_ITER(Q, W, CUR, FREE, JJ)                                \
     do {                                                                   \
         wait_barrier();                                                    \
         copy_act(FREE, (JJ) + 3);                                          \
-        compute(CUR, wq[Q][0], wq[Q][1]);                                  \
+        *(v4u*)(wmine + wwr[0]) = wq[W][0];                                \
+        *(v4u*)(wmine + wwr[1]) = wq[W][1];                                \
+        wq[W][0] = load_w((JJ) + D, 0);                                    \
+        wq[W][1] = load_w((JJ) + D, 1);                                    \
+        __builtin_amdgcn_sched_barrier(0);                                 \
+        compute(CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1])); \
         if constexpr (G128) fold(sq[Q], zq[Q]);                            \
-        wq[Q][0] = load_w((JJ) + 4, 0);                                    \
-        wq[Q][1] = load_w((JJ) + 4, 1);                                    \
         if constexpr (G128) {                                              \
             sq[Q] = load_tab(sptr, (JJ) + 4);                              \
             zq[Q] = load_tab(zptr, (JJ) + 4);                              \
@@ -236,32 +255,42 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
         __builtin_amdgcn_sched_barrier(0);                                 \
     } while (0)
 
-    // ---- prologue: the same issue order as three iterations before the first one
-    wq[0][0] = load_w(0, 0);
-    wq[0][1] = load_w(0, 1);
+    // ---- prologue: the older weight slabs first, then the same issue order as the three
+    // iterations before the first one
+#pragma unroll
+    for (int d = 0; d <= D - 4; ++d) {
+        wq[d][0] = load_w(d, 0);
+        wq[d][1] = load_w(d, 1);
+    }
     if constexpr (G128) { sq[0] = load_tab(sptr, 0); zq[0] = load_tab(zptr, 0); }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st0, 0);
-    wq[1][0] = load_w(1, 0);
-    wq[1][1] = load_w(1, 1);
+    wq[D - 3][0] = load_w(D - 3, 0);
+    wq[D - 3][1] = load_w(D - 3, 1);
     if constexpr (G128) { sq[1] = load_tab(sptr, 1); zq[1] = load_tab(zptr, 1); }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st1, 1);
-    wq[2][0] = load_w(2, 0);
-    wq[2][1] = load_w(2, 1);
+    wq[D - 2][0] = load_w(D - 2, 0);
+    wq[D - 2][1] = load_w(D - 2, 1);
     if constexpr (G128) { sq[2] = load_tab(sptr, 2); zq[2] = load_tab(zptr, 2); }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st2, 2);
-    wq[3][0] = load_w(3, 0);
-    wq[3][1] = load_w(3, 1);
+    wq[D - 1][0] = load_w(D - 1, 0);
+    wq[D - 1][1] = load_w(D - 1, 1);
     if constexpr (G128) { sq[3] = load_tab(sptr, 3); zq[3] = load_tab(zptr, 3); }
     __builtin_amdgcn_sched_barrier(0);
 
-    for (int jj = 0; jj < nsl; jj += 4) {
-        FNN_PANEL_ITER(0, st0, st3, jj);
-        FNN_PANEL_ITER(1, st1, st0, jj + 1);
-        FNN_PANEL_ITER(2, st2, st1, jj + 2);
-        FNN_PANEL_ITER(3, st3, st2, jj + 3);
+    for (int jj = 0; jj < nsl; jj += D) {
+        FNN_PANEL_ITER(0, 0, st0, st3, jj);
+        FNN_PANEL_ITER(1, 1, st1, st0, jj + 1);
+        FNN_PANEL_ITER(2, 2, st2, st1, jj + 2);
+        FNN_PANEL_ITER(3, 3, st3, st2, jj + 3);
+        if constexpr (D == 8) {
+            FNN_PANEL_ITER(0, 4, st0, st3, jj + 4);
+            FNN_PANEL_ITER(1, 5, st1, st0, jj + 5);
+            FNN_PANEL_ITER(2, 6, st2, st1, jj + 6);
+            FNN_PANEL_ITER(3, 7, st3, st2, jj + 7);
+        }
     }
 #undef FNN_PANEL_ITER
 
@@ -360,12 +389,18 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     const int mb = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);
+    const bool deep = p.K % 2048 == 0;   // 8 weight slabs in flight per wave instead of 4
     p.m_base = 0;
-#define FNN_PANEL(G, SDTV)                                                                               \
+#define FNN_PANEL2(G, SDTV, MBV)                                                                         \
     do {                                                                                                 \
-        if (mb == 1) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, 1, 2><<<grid, dim3(512), 0, st>>>(p, passes);      \
-        else if (mb == 2) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, 2, 2><<<grid, dim3(512), 0, st>>>(p, passes); \
-        else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, 4, 2><<<grid, dim3(512), 0, st>>>(p, passes);              \
+        if (deep) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, 2, 8><<<grid, dim3(512), 0, st>>>(p, passes);   \
+        else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, 2, 4><<<grid, dim3(512), 0, st>>>(p, passes);        \
+    } while (0)
+#define FNN_PANEL(G, SDTV)                       \
+    do {                                         \
+        if (mb == 1) FNN_PANEL2(G, SDTV, 1);     \
+        else if (mb == 2) FNN_PANEL2(G, SDTV, 2);\
+        else FNN_PANEL2(G, SDTV, 4);             \
     } while (0)
     if (p.group == 128) {
         if (p.scale_dtype == FNN_F16) FNN_PANEL(true, FNN_F16);
@@ -374,6 +409,7 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
         FNN_PANEL(false, FNN_F16);
     }
 #undef FNN_PANEL
+#undef FNN_PANEL2
     return true;
 }
 

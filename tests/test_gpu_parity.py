@@ -99,6 +99,25 @@ def test_a8w8_guarded_kernel_bit_exact(mnk):
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
 
 
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("nk", [(1000, 64), (16, 448), (4100, 4096), (520, 8192)])
+def test_a8w8_few_rows_bit_exact(M, nk):
+    """Up to 64 activation rows take the weight-streaming kernel: accumulators and scaled outputs,
+    N not a multiple of the 16-row tile, fewer k-steps than waves."""
+    N, K = nk
+    a, b = _rand_i8((M, K), 10 + M), _rand_i8((N, K), 11)
+    acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+    want = O.gemm_a8w8_acc(a.numpy(), b.numpy())
+    assert np.array_equal(acc, want)
+    g = torch.Generator().manual_seed(12)
+    out_ty = torch.float16 if M % 2 else torch.bfloat16
+    ar = (torch.rand(M, 1, generator=g) * 0.05).to(out_ty)
+    ac = (torch.rand(1, N, generator=g) * 0.05).float()
+    out = flashnn_amd.GemmA8W8(out_ty)(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV))
+    assert np.array_equal(out.float().cpu().numpy(),
+                          O.gemm_a8w8_epilogue_fp32(want, O.to_np(ar), O.to_np(ac), _tag(out_ty)))
+
+
 def test_a8w8_saturation_and_identity():
     a = torch.full((256, 4096), -128, dtype=torch.int8)
     acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), a.to(DEV))
