@@ -1024,8 +1024,10 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
         gemm_wo_any_kernel<WBITS, ADT><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(p);
         return;
     }
+    // from 5 activation rows on, four weight tiles sharing the activations through LDS beat the
+    // decode kernels wherever there are enough weight rows to fill the chip that way
+    if (p.M > 4 && launch_wo_panel(p, WBITS, ADT, st)) return;
     if (launch_decode<WBITS, ADT>(p, st)) return;
-    if (launch_wo_panel(p, WBITS, ADT, st)) return;
     // up to 64 activation rows per pass over the weights
     for (int m0 = 0; m0 < p.M; m0 += 64) {
         p.m_base = m0;
