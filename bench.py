@@ -8,8 +8,9 @@ per-token x per-channel scale epilogue writing bf16 (the Llama-7B QKV prefill sh
 
 Also measured in the same run and reported in the same JSON line:
   roofline          the A8W8 GEMM kernel alone against the dense int8 MFMA peak
-  secondary[0]      A16W4 group-128 decode GEMV, M=1 K=8192 N=28672 bf16, against 8 TB/s HBM
-  secondary[1..]    the row kernels (dynamic quant, RMSNorm+quant) against HBM
+  secondary         the other configurations: the remaining prefill shapes, A16W4 group-128 at
+                    M = 1 .. 256 (M=1 is the decode GEMV of the second headline metric), A8W8 with
+                    few activation rows, A16W8 decode and the row kernels, each against its bound
   cpu_baseline      the reference's torch CPU path (oracle/torch_path.py) on the host cores
 
 Operand sets are rotated so that the working set exceeds the 256 MB Infinity Cache; kernel
@@ -167,7 +168,7 @@ def main():
         pk = [packed.to(dev).clone() for _ in range(nset4)]
         sc = [scale4.to(dev).clone() for _ in range(nset4)]
         zp = [zp4.to(dev).clone() for _ in range(nset4)]
-        for m4 in (1, 4, 16):
+        for m4 in (1, 4, 16, 64, 256):
             act = workloads.activations(m4, K4, torch.bfloat16, seed=3).to(dev)
             o4 = torch.empty(m4, N4, dtype=torch.bfloat16, device=dev)
             f = lambda i: launchers.hip_gemm_a16w4_forward(o4, act, pk[i % nset4], sc[i % nset4], None, zp[i % nset4])
@@ -178,12 +179,34 @@ def main():
             allbytes = wbytes + 2.0 * m4 * K4 + 2.0 * m4 * N4
             gbs = allbytes / (ms * 1e-3) / 1e9
             secondary.append({"workload": f"a16w4 g128 decode M={m4} K={K4} N={N4} bf16",
-                              "kernel": "gemm_wo_gemv_kernel" if m4 <= 4 else "gemm_wo_stream_kernel", "us_per_launch": round(ms * 1e3, 2),
+                              "kernel": "gemm_wo_gemv_kernel" if m4 <= 4 else "gemm_wo_panel_kernel", "us_per_launch": round(ms * 1e3, 2),
                               "weight_GBps": round(wbytes / (ms * 1e-3) / 1e9, 1),
                               "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
                                            "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
                                            "traffic": _traffic("gemm_wo_gemv_kernel") if m4 == 1 else None}})
         del pk, sc, zp
+        torch.cuda.empty_cache()
+
+    # ------------------------------------- few activation rows: RMSNorm+quant -> A8W8, K = N = 8192
+    if "a8w8" in legs:
+        k5 = n5 = 8192
+        w5 = [torch.randint(-127, 128, (n5, k5), dtype=torch.int8, device=dev) for _ in range(5)]
+        c5 = torch.rand(n5, device=dev) * 0.01
+        for m5 in (1, 32):
+            a5 = torch.randint(-127, 128, (m5, k5), dtype=torch.int8, device=dev)
+            s5 = torch.rand(m5, device=dev).bfloat16()
+            o5 = torch.empty(m5, n5, dtype=torch.bfloat16, device=dev)
+            f = lambda i: launchers.hip_gemm_a8w8_forward(o5, a5, w5[i % 5], s5, c5)
+            for i in range(10):
+                f(i)
+            ms = _events_ms(f, 100, torch)
+            b5 = float(n5) * k5 + m5 * k5 + 2.0 * m5 * n5 + 2.0 * m5 + 4.0 * n5
+            secondary.append({"workload": f"a8w8 few rows M={m5} K={k5} N={n5} bf16", "kernel": "gemm_a8w8_skinny_kernel",
+                              "us_per_launch": round(ms * 1e3, 2),
+                              "roofline": {"bound": "hbm", "achieved": round(b5 / (ms * 1e-3) / 1e9, 1),
+                                           "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                           "frac": round(b5 / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+        del w5
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------- A16W8 decode + row kernels
