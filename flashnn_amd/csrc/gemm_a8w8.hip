@@ -39,9 +39,10 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // ------------------------------------------------------------------ main MFMA kernel
 // K % 128 == 0, K >= 512.  K is walked in slabs of 128 bytes: every row piece a copy fetches
 // is one full 128-byte line, which is what the L2 -> LDS path needs to run at speed (64-byte
-// pieces reach little more than half the rate).  The LDS holds an asymmetric ring: three
-// stages for the a-rows (copied two slabs ahead, a third per k-step) and two for the b-rows (one slab ahead);
-// 3*BM + 2*BN rows of 128 bytes = 144 KB for a 256x192 tile.  There is one barrier per slab, at
+// pieces reach little more than half the rate).  The LDS holds a ring of three stages for the a-rows
+// (copied two slabs ahead, a third per k-step) and, for the 256x192 tile, two for the b-rows (one slab
+// ahead): 3*BM + 2*BN rows of 128 bytes = 144 KB.  The smaller tiles have room for a third b-stage
+// and copy the b-rows two slabs ahead as well (3 to 20 % faster).  There is one barrier per slab, at
 // the start of its LAST k-step: by then every fragment of the slab is in registers, so both of
 // its stages are free and are re-armed right after the barrier, and the barrier publishes the
 // next slab, whose first fragments are read under the last MFMAs of the current one.
@@ -66,6 +67,11 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     __shared__ __attribute__((aligned(1024))) char sa2[BM * BK];
     __shared__ __attribute__((aligned(1024))) char sb0[BN * BK];
     __shared__ __attribute__((aligned(1024))) char sb1[BN * BK];
+    // a third b-stage where the tile leaves room for it (3 * (BM + BN) rows <= 160 KB): the b-rows are
+    // then copied two slabs ahead like the a-rows; with two stages their copy has exactly one slab
+    // to land, which is about the loaded L2 latency
+    constexpr int NSB = 3 * (BM + BN) * BK + 4 * (BM + BN) + 1024 <= 160 * 1024 ? 3 : 2;
+    __shared__ __attribute__((aligned(1024))) char sb2[NSB == 3 ? BN * BK : 16];
     __shared__ __attribute__((aligned(16))) float sc_row[BM];   // alpha_row of the tile's rows, fp32
     __shared__ __attribute__((aligned(16))) float sc_col[BN];   // alpha_col of the tile's columns
 
@@ -125,6 +131,14 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         for (int j = 0; j < NLB; ++j)
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
                                              (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
+    };
+    auto copy_b_part = [&](char* stage, int kt, int part) {
+        const char* slab = (const char*)p.b + (int64_t)kt * BK;
+#pragma unroll
+        for (int j = 0; j < NLB; ++j)
+            if (j * 3 / NLB == part)
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
+                                                 (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
 
     // read plan: lane reads row (lane & 31) of a fragment, logical chunk 2*ks + (lane >> 5)
@@ -213,28 +227,81 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    copy_a(sa0, 0);
-    copy_b(sb0, 0);
-    copy_a(sa1, 1);
-    wait_barrier(true);
-    read_frags(sa0, sb0, 0);
-    copy_b(sb1, 1);
-    int j = 0;
-    for (; j + 8 <= KT; j += 6) {   // every slab of the round still has both refills ahead of it
-        slab(sa0, sb0, sa1, sb1, sa2, j, true);
-        slab(sa1, sb1, sa2, sb0, sa0, j + 1, true);
-        slab(sa2, sb0, sa0, sb1, sa1, j + 2, true);
-        slab(sa0, sb1, sa1, sb0, sa2, j + 3, true);
-        slab(sa1, sb0, sa2, sb1, sa0, j + 4, true);
-        slab(sa2, sb1, sa0, sb0, sa1, j + 5, true);
-    }
-    for (; j < KT; j += 6) {        // the last two to seven slabs, with the refills guarded
-        slab(sa0, sb0, sa1, sb1, sa2, j, false);
-        if (j + 1 < KT) slab(sa1, sb1, sa2, sb0, sa0, j + 1, false);
-        if (j + 2 < KT) slab(sa2, sb0, sa0, sb1, sa1, j + 2, false);
-        if (j + 3 < KT) slab(sa0, sb1, sa1, sb0, sa2, j + 3, false);
-        if (j + 4 < KT) slab(sa1, sb0, sa2, sb1, sa0, j + 4, false);
-        if (j + 5 < KT) slab(sa2, sb1, sa0, sb0, sa1, j + 5, false);
+    if constexpr (NSB == 2) {
+        copy_a(sa0, 0);
+        copy_b(sb0, 0);
+        copy_a(sa1, 1);
+        wait_barrier(true);
+        read_frags(sa0, sb0, 0);
+        copy_b(sb1, 1);
+        int j = 0;
+        for (; j + 8 <= KT; j += 6) {   // every slab of the round still has both refills ahead of it
+            slab(sa0, sb0, sa1, sb1, sa2, j, true);
+            slab(sa1, sb1, sa2, sb0, sa0, j + 1, true);
+            slab(sa2, sb0, sa0, sb1, sa1, j + 2, true);
+            slab(sa0, sb1, sa1, sb0, sa2, j + 3, true);
+            slab(sa1, sb0, sa2, sb1, sa0, j + 4, true);
+            slab(sa2, sb1, sa0, sb0, sa1, j + 5, true);
+        }
+        for (; j < KT; j += 6) {        // the last two to seven slabs, with the refills guarded
+            slab(sa0, sb0, sa1, sb1, sa2, j, false);
+            if (j + 1 < KT) slab(sa1, sb1, sa2, sb0, sa0, j + 1, false);
+            if (j + 2 < KT) slab(sa2, sb0, sa0, sb1, sa1, j + 2, false);
+            if (j + 3 < KT) slab(sa0, sb1, sa1, sb0, sa2, j + 3, false);
+            if (j + 4 < KT) slab(sa1, sb0, sa2, sb1, sa0, j + 4, false);
+            if (j + 5 < KT) slab(sa2, sb1, sa0, sb0, sa1, j + 5, false);
+        }
+    } else {
+        // three stages each: a(j+2) and b(j+2) are both copied in parts during k-steps 0..2 of slab j,
+        // into the stages freed at the previous barrier; at the barrier only they may be in flight
+        auto wait_barrier3 = [&](bool keep) {
+            constexpr int NK = NLA + NLB;
+            asm volatile("" ::: "memory");
+            if (keep) __builtin_amdgcn_s_waitcnt(0x0070 | (NK & 15) | ((NK >> 4) << 14));
+            else __builtin_amdgcn_s_waitcnt(0x0070);
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        };
+        auto slab3 = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fa, char* fb, int j,
+                         bool steady) {
+#pragma unroll
+            for (int ks = 0; ks < 3; ++ks) {
+                read_frags(sa, sb, ks + 1);
+                if (steady || j + 2 < KT) {
+                    copy_a_part(fa, j + 2, ks);
+                    copy_b_part(fb, j + 2, ks);
+                }
+                mfmas(ks & 1);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (steady || j + 1 < KT) {
+                wait_barrier3(steady || j + 2 < KT);
+                read_frags(nsa, nsb, 0);
+                mfmas(1);
+                interleave();
+            } else {
+                mfmas(1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        copy_a(sa0, 0);
+        copy_b(sb0, 0);
+        copy_a(sa1, 1);
+        copy_b(sb1, 1);
+        wait_barrier3(true);
+        read_frags(sa0, sb0, 0);
+        int j = 0;
+        for (; j + 5 <= KT; j += 3) {
+            slab3(sa0, sb0, sa1, sb1, sa2, sb2, j, true);
+            slab3(sa1, sb1, sa2, sb2, sa0, sb0, j + 1, true);
+            slab3(sa2, sb2, sa0, sb0, sa1, sb1, j + 2, true);
+        }
+        for (; j < KT; j += 3) {
+            slab3(sa0, sb0, sa1, sb1, sa2, sb2, j, false);
+            if (j + 1 < KT) slab3(sa1, sb1, sa2, sb2, sa0, sb0, j + 1, false);
+            if (j + 2 < KT) slab3(sa2, sb2, sa0, sb0, sa1, sb1, j + 2, false);
+        }
     }
 
     // ---- epilogue ----
@@ -388,7 +455,7 @@ struct TileChoice { int bm, bn; };
 // Pick the tile whose last, partly filled round of workgroups costs least on 256 CUs.
 static TileChoice choose_tile(int64_t M, int64_t N) {
     static const struct { int bm, bn; double eff; } cand[] = {
-        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.65}};
+        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.72}};   // throughput per tile area, measured at K = N = 8192 (at smaller shapes the smaller tiles come closer)
     double best = 1e300;
     TileChoice c{128, 128};
     for (const auto& t : cand) {
