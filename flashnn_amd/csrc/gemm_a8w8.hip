@@ -21,6 +21,8 @@
 // Any other shape takes a small guarded LDS kernel built on v_dot4_i32_i8.
 //
 // Reference for the semantics: flashnn/triton_kernels/gemm_a8w8.py:74-179.
+#include <type_traits>
+
 #include "a8w8_common.h"
 
 // The scaled output is two fp32 multiplications and one rounding to 16 bits, each rounded on its
@@ -64,14 +66,17 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
 
     __shared__ __attribute__((aligned(1024))) char sa0[BM * BK];
     __shared__ __attribute__((aligned(1024))) char sa1[BM * BK];
-    __shared__ __attribute__((aligned(1024))) char sa2[BM * BK];
+    // tiles too large for three stages of both operands give the third stage to the b-rows (the
+    // weights, streamed from HBM) and copy the a-rows (L2 hits after their first use) one slab ahead
+    constexpr bool BDEEP = 3 * (BM + BN) * BK + 4 * (BM + BN) + 1024 > 160 * 1024;
+    __shared__ __attribute__((aligned(1024))) char sa2[BDEEP ? 16 : BM * BK];
     __shared__ __attribute__((aligned(1024))) char sb0[BN * BK];
     __shared__ __attribute__((aligned(1024))) char sb1[BN * BK];
     // a third b-stage where the tile leaves room for it (3 * (BM + BN) rows <= 160 KB): the b-rows are
     // then copied two slabs ahead like the a-rows; with two stages their copy has exactly one slab
     // to land, which is about the loaded L2 latency
     constexpr int NSB = 3 * (BM + BN) * BK + 4 * (BM + BN) + 1024 <= 160 * 1024 ? 3 : 2;
-    __shared__ __attribute__((aligned(1024))) char sb2[NSB == 3 ? BN * BK : 16];
+    __shared__ __attribute__((aligned(1024))) char sb2[NSB == 3 || BDEEP ? BN * BK : 16];
     __shared__ __attribute__((aligned(16))) float sc_row[BM];   // alpha_row of the tile's rows, fp32
     __shared__ __attribute__((aligned(16))) float sc_col[BN];   // alpha_col of the tile's columns
 
@@ -191,77 +196,69 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     // Wait until at most `newer` of this wave's copies are outstanding and its LDS reads have
     // returned, then cross the workgroup barrier.  A bare s_barrier: __syncthreads() would add a
     // fence that waits for every outstanding copy and collapse the ring to depth one.
-    auto wait_barrier = [&](bool keep_a) {
+    auto wait_barrier_n = [&](int newer_is_kept, auto nkeep) {
+        constexpr int NK = decltype(nkeep)::value;
         asm volatile("" ::: "memory");
-        if (keep_a) __builtin_amdgcn_s_waitcnt(0x0070 | (NLA & 15) | ((NLA >> 4) << 14));
+        if (newer_is_kept) __builtin_amdgcn_s_waitcnt(0x0070 | (NK & 15) | ((NK >> 4) << 14));
         else __builtin_amdgcn_s_waitcnt(0x0070);
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
 
     const int KT = p.K / BK;
-    // One slab = four k-steps; slab j lives in (sa, sb), slab j+1 in (nsa, nsb), and `fa` is the
-    // a-stage freed at the previous barrier (it held slab j-1), into which the a-rows of slab j+2 are
-    // copied during k-steps 0..2.  At the barrier of the last k-step the b-stage of slab j is free
-    // and receives the b-rows of slab j+2.  Copy order per slab: a(j+2) parts, then b(j+2); at the
-    // barrier for slab j+1 the only copies that may still be in flight are those a(j+2) parts.
-    // (Also tried: b-copies in parts as well - slower, their lead time becomes too short.)
-    auto slab = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fa, int j, bool steady) {
+    // One slab = four k-steps; slab j lives in (sa, sb), slab j+1 in (nsa, nsb).  Copies of slab j+2
+    // are issued in three parts during k-steps 0..2 into the stage freed at the previous barrier
+    // (issued in one burst they block the wave's MFMAs behind them).  The barrier at the start of the
+    // last k-step publishes slab j+1, whose first fragments are read under the last MFMAs of slab j.
+    if constexpr (BDEEP) {
+        auto wait_barrierB = [&](bool keep) { wait_barrier_n(keep, std::integral_constant<int, NLB>{}); };
+        auto slabB = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fb, int j, bool steady) {
 #pragma unroll
-        for (int ks = 0; ks < 3; ++ks) {
-            read_frags(sa, sb, ks + 1);
-            if (steady || j + 2 < KT) copy_a_part(fa, j + 2, ks);
-            mfmas(ks & 1);
-            interleave();
+            for (int ks = 0; ks < 3; ++ks) {
+                read_frags(sa, sb, ks + 1);
+                if (steady || j + 2 < KT) copy_b_part(fb, j + 2, ks);
+                mfmas(ks & 1);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (steady || j + 1 < KT) {
+                wait_barrierB(steady || j + 2 < KT);
+                read_frags(nsa, nsb, 0);
+                if (steady || j + 2 < KT) copy_a(sa, j + 2);
+                mfmas(1);
+                interleave();
+            } else {
+                mfmas(1);
+            }
             __builtin_amdgcn_sched_barrier(0);
-        }
-        if (steady || j + 1 < KT) {
-            wait_barrier(steady || j + 2 < KT);
-            read_frags(nsa, nsb, 0);
-            if (steady || j + 2 < KT) copy_b(sb, j + 2);
-            mfmas(1);
-            interleave();
-        } else {
-            mfmas(1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    if constexpr (NSB == 2) {
-        copy_a(sa0, 0);
+        };
         copy_b(sb0, 0);
-        copy_a(sa1, 1);
-        wait_barrier(true);
-        read_frags(sa0, sb0, 0);
+        copy_a(sa0, 0);
         copy_b(sb1, 1);
+        wait_barrierB(true);
+        read_frags(sa0, sb0, 0);
+        copy_a(sa1, 1);
         int j = 0;
-        for (; j + 8 <= KT; j += 6) {   // every slab of the round still has both refills ahead of it
-            slab(sa0, sb0, sa1, sb1, sa2, j, true);
-            slab(sa1, sb1, sa2, sb0, sa0, j + 1, true);
-            slab(sa2, sb0, sa0, sb1, sa1, j + 2, true);
-            slab(sa0, sb1, sa1, sb0, sa2, j + 3, true);
-            slab(sa1, sb0, sa2, sb1, sa0, j + 4, true);
-            slab(sa2, sb1, sa0, sb0, sa1, j + 5, true);
+        for (; j + 8 <= KT; j += 6) {
+            slabB(sa0, sb0, sa1, sb1, sb2, j, true);
+            slabB(sa1, sb1, sa0, sb2, sb0, j + 1, true);
+            slabB(sa0, sb2, sa1, sb0, sb1, j + 2, true);
+            slabB(sa1, sb0, sa0, sb1, sb2, j + 3, true);
+            slabB(sa0, sb1, sa1, sb2, sb0, j + 4, true);
+            slabB(sa1, sb2, sa0, sb0, sb1, j + 5, true);
         }
-        for (; j < KT; j += 6) {        // the last two to seven slabs, with the refills guarded
-            slab(sa0, sb0, sa1, sb1, sa2, j, false);
-            if (j + 1 < KT) slab(sa1, sb1, sa2, sb0, sa0, j + 1, false);
-            if (j + 2 < KT) slab(sa2, sb0, sa0, sb1, sa1, j + 2, false);
-            if (j + 3 < KT) slab(sa0, sb1, sa1, sb0, sa2, j + 3, false);
-            if (j + 4 < KT) slab(sa1, sb0, sa2, sb1, sa0, j + 4, false);
-            if (j + 5 < KT) slab(sa2, sb1, sa0, sb0, sa1, j + 5, false);
+        for (; j < KT; j += 6) {
+            slabB(sa0, sb0, sa1, sb1, sb2, j, false);
+            if (j + 1 < KT) slabB(sa1, sb1, sa0, sb2, sb0, j + 1, false);
+            if (j + 2 < KT) slabB(sa0, sb2, sa1, sb0, sb1, j + 2, false);
+            if (j + 3 < KT) slabB(sa1, sb0, sa0, sb1, sb2, j + 3, false);
+            if (j + 4 < KT) slabB(sa0, sb1, sa1, sb2, sb0, j + 4, false);
+            if (j + 5 < KT) slabB(sa1, sb2, sa0, sb0, sb1, j + 5, false);
         }
     } else {
         // three stages each: a(j+2) and b(j+2) are both copied in parts during k-steps 0..2 of slab j,
         // into the stages freed at the previous barrier; at the barrier only they may be in flight
-        auto wait_barrier3 = [&](bool keep) {
-            constexpr int NK = NLA + NLB;
-            asm volatile("" ::: "memory");
-            if (keep) __builtin_amdgcn_s_waitcnt(0x0070 | (NK & 15) | ((NK >> 4) << 14));
-            else __builtin_amdgcn_s_waitcnt(0x0070);
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-        };
+        auto wait_barrier3 = [&](bool keep) { wait_barrier_n(keep, std::integral_constant<int, NLA + NLB>{}); };
         auto slab3 = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fa, char* fb, int j,
                          bool steady) {
 #pragma unroll
@@ -339,7 +336,7 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         constexpr int TSTRIDE = WTN * 2 + 16;      // bytes per staged row; the pad staggers the banks
         constexpr int PR = WTN * 2 / 16;           // 16-byte pieces per row
         static_assert(64 * TSTRIDE <= BN * BK, "transpose buffer must fit a stage");
-        char* tbuf = wave == 0 ? sa0 : wave == 1 ? sa1 : wave == 2 ? sa2 : sb0;
+        char* tbuf = wave == 0 ? sa0 : wave == 1 ? sa1 : wave == 2 ? (BDEEP ? sb1 : sa2) : sb0;
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0x0070);   // all copies and LDS reads of this wave are done
         __builtin_amdgcn_s_barrier();         // ... and everybody else's: the stages are free
