@@ -56,11 +56,16 @@ __device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4
 
 // G128: per-group tables with group size 128, entries of type SDT (fp16 or bf16), zero points in
 // the same type; otherwise per-channel scales of any type, applied once at the end.
-// D: slabs of weights in flight per wave; the K part of a wave holds a multiple of D slabs.  (8 loads
-// per lane in flight stream faster than 16: measured 19.8 against 21.7 us for 117 MB in a load-only
-// model.)  NTL: non-temporal weight loads, for a single pass over the weights.
-template <int WBITS, int ADT, bool G128, int SDT, int MB, int KS, int D, bool NTL>
-__global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p, const int passes) {
+// RT: 16-row weight tiles per workgroup (4, 2 or 1); the 8 waves are RT tiles x KS = 8 / RT parts of K.
+// Fewer rows per workgroup make more workgroups for matrices with few rows, at the price of each
+// activation slab being shared by fewer waves.  K parts may differ by one slab; all waves run the
+// same number of iterations (the barriers are shared) and skip the work of slabs they do not have.
+// D: slabs of weights in flight per wave (8 loads per lane in flight stream faster than 16: measured
+// 19.8 against 21.7 us for 117 MB in a load-only model).  NTL: non-temporal weight loads, for a
+// single pass over the weights.
+template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL>
+__global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, const int passes) {
+    constexpr int KS = 8 / RT;
     typedef MfmaT<ADT> MT;
     constexpr int NH = WBITS == 4 ? 2 : 1;      // channels per weight row
     constexpr int NCL = 4 * NH;                 // consecutive channels per lane
@@ -68,7 +73,7 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
                                        : (ADT == FNN_F16 ? 1024.f + 128.f : 128.f);
     constexpr int SLAB = MB * 16 * 256;         // bytes of one activation slab: 16*MB rows x 128 k
     constexpr int STG = KS * SLAB;
-    constexpr int RED = KS > 1 ? (KS - 1) * 4 * MB * NH * 4 * 64 * 4 : 16;
+    constexpr int RED = (KS - 1) * RT * MB * NH * 4 * 64 * 4;
     constexpr int STG0 = STG > RED ? STG : RED;
     // one array per stage: the compiler then knows that reads of one stage cannot alias the
     // copies in flight into another
@@ -76,28 +81,30 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
     __shared__ __attribute__((aligned(16))) char st1[STG];
     __shared__ __attribute__((aligned(16))) char st2[STG];
     __shared__ __attribute__((aligned(16))) char st3[STG];
-    __shared__ __attribute__((aligned(16))) char wst[4 * KS * 2048];
+    __shared__ __attribute__((aligned(16))) char wst[8 * 2048];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int rt = wave & 3;
-    const int ks = wave >> 2;
+    const int rt = wave % RT;
+    const int ks = wave / RT;
     const int li = lane & 15;
     const int lg = lane >> 4;
 
     // workgroups id, id+8, id+16 .. run on the same XCD: give them the same weight tile and
     // consecutive passes so that the tile is fetched from HBM once and re-read from that L2
     const int wrows = WBITS == 4 ? p.N / 2 : p.N;
-    const int tiles = wrows / 64;
+    const int tiles = wrows / (16 * RT);
     const int y = blockIdx.x >> 3;
     const int pass = y % passes;
     const int tile = (y / passes) * 8 + (blockIdx.x & 7);
     if (tile >= tiles) return;
     const int m_base = p.m_base + pass * (MB * 16);
-    const int row0 = tile * 64 + rt * 16;
+    const int row0 = (tile * RT + rt) * 16;
 
-    const int nsl = p.K / (128 * KS);           // slabs per K part (multiple of 4)
-    const int sl0 = ks * nsl;
+    const int KT = p.K / 128;
+    const int sl0 = KT * ks / KS;               // this wave's slabs: sl0 .. sl0 + nsl - 1
+    const int nsl = KT * (ks + 1) / KS - sl0;
+    const int n_iter = ((KT + KS - 1) / KS + D - 1) / D * D;   // iterations of every wave
 
     // ---- weights: load h of a slab fetches rows 8h .. 8h+7 of the wave's tile, 8 lanes per row, one
     // full 128-byte line per row (16 rows x 64 bytes per load, the MFMA operand's own shape, streams
@@ -121,21 +128,25 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
 
     // ---- activation copies: thread t of the K part copies chunk (t & 15) ^ (t >> 4) of rows
     // (t >> 4) + 16 i into slot (t & 15) of those rows
+    // (the RT waves of a K part make 64 RT lanes; copy i of a wave covers rows 4 RT i + (t >> 4))
+    constexpr int NCP = MB * 4 / RT;            // copies per wave and slab
     const int t = rt * 64 + lane;
     const int tokq = t >> 4;
-    const int chunk = (t & 15) ^ tokq;
-    const char* act_part = (const char*)p.act + (int64_t)sl0 * 256 + chunk * 16;
-    int64_t goff[MB];
+    const char* act_part = (const char*)p.act + (int64_t)sl0 * 256;
+    int64_t goff[NCP];
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
-        goff[i] = (int64_t)min(m_base + i * 16 + tokq, p.M - 1) * p.lda * 2;
+    for (int i = 0; i < NCP; ++i) {
+        const int tok = i * (4 * RT) + tokq;
+        const int chunk = (t & 15) ^ (tok & 15);
+        goff[i] = (int64_t)min(m_base + tok, p.M - 1) * p.lda * 2 + chunk * 16;
+    }
     auto copy_act = [&](char* stage, int jj) {
         const int j = min(jj, nsl - 1);
         const char* src = act_part + (int64_t)j * 256;
 #pragma unroll
-        for (int i = 0; i < MB; ++i)
+        for (int i = 0; i < NCP; ++i)
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + goff[i]),
-                                             (lds_ptr_t)(stage + ks * SLAB + (i * 256 + rt * 64) * 16), 16, 0, 0);
+                                             (lds_ptr_t)(stage + ks * SLAB + (i * RT * 64 + rt * 64) * 16), 16, 0, 0);
     };
     // ---- activation fragment reads: lane (li, lg) reads chunks 8 s + 2 lg + h of row 16 mb + li
     int rd[2][2];
@@ -166,11 +177,11 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
     }
     const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
 
-    // loads issued per iteration, in this order: MB copies, 2 weight loads, 2 table loads
-    constexpr int C = MB + 2 + (G128 ? 2 : 0);
+    // loads issued per iteration, in this order: NCP copies, 2 weight loads, 2 table loads
+    constexpr int C = NCP + 2 + (G128 ? 2 : 0);
     // the newest load slab j depends on is its last copy, issued three iterations earlier; after
     // it came the rest of that iteration and two whole ones
-    constexpr int X = (C - MB) + 2 * C;
+    constexpr int X = (C - NCP) + 2 * C;
     static_assert(X < 64, "vmcnt range");
     auto wait_barrier = [&]() {
         asm volatile("" ::: "memory");
@@ -244,13 +255,18 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
     do {                                                                   \
         wait_barrier();                                                    \
         copy_act(FREE, (JJ) + 3);                                          \
-        *(v4u*)(wmine + wwr[0]) = wq[W][0];                                \
-        *(v4u*)(wmine + wwr[1]) = wq[W][1];                                \
+        const bool mine_ = (JJ) < nsl;   /* wave-uniform */                \
+        if (mine_) {                                                       \
+            *(v4u*)(wmine + wwr[0]) = wq[W][0];                            \
+            *(v4u*)(wmine + wwr[1]) = wq[W][1];                            \
+        }                                                                  \
         wq[W][0] = load_w((JJ) + D, 0);                                    \
         wq[W][1] = load_w((JJ) + D, 1);                                    \
         __builtin_amdgcn_sched_barrier(0);                                 \
-        compute(CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1])); \
-        if constexpr (G128) fold(sq[Q], zq[Q]);                            \
+        if (mine_) {                                                       \
+            compute(CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1])); \
+            if constexpr (G128) fold(sq[Q], zq[Q]);                        \
+        }                                                                  \
         if constexpr (G128) {                                              \
             sq[Q] = load_tab(sptr, (JJ) + 4);                              \
             zq[Q] = load_tab(zptr, (JJ) + 4);                              \
@@ -284,7 +300,7 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
     __builtin_amdgcn_sched_barrier(0);
 
     static_assert(D == 4, "the unrolled loop below walks four weight slots");
-    for (int jj = 0; jj < nsl; jj += D) {
+    for (int jj = 0; jj < n_iter; jj += D) {
         FNN_PANEL_ITER(0, 0, st0, st3, jj);
         FNN_PANEL_ITER(1, 1, st1, st0, jj + 1);
         FNN_PANEL_ITER(2, 2, st2, st1, jj + 2);
@@ -324,7 +340,7 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
                 for (int h = 0; h < NH; ++h)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        red[(((((ks - 1) * 4 + rt) * MB + mb) * NH + h) * 4 + r) * 64 + lane] = outv[mb][h][r];
+                        red[(((((ks - 1) * RT + rt) * MB + mb) * NH + h) * 4 + r) * 64 + lane] = outv[mb][h][r];
         }
         __syncthreads();
         if (ks > 0) return;
@@ -336,7 +352,7 @@ __global__ __launch_bounds__(256 * KS) void gemm_wo_panel_kernel(const WoArgs p,
                 for (int h = 0; h < NH; ++h)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        outv[mb][h][r] += red[(((((k2 - 1) * 4 + rt) * MB + mb) * NH + h) * 4 + r) * 64 + lane];
+                        outv[mb][h][r] += red[(((((k2 - 1) * RT + rt) * MB + mb) * NH + h) * 4 + r) * 64 + lane];
     }
 
     // ---- bias, rounding, store: lane (li, lg) holds channels n0 .. n0+NCL-1 of row 16 mb + li
@@ -374,7 +390,7 @@ template <int WBITS, int ADT>
 static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     constexpr int NH = WBITS == 4 ? 2 : 1;
     const int wrows = WBITS == 4 ? p.N / 2 : p.N;
-    if (wrows % 64 != 0 || p.K % 1024 != 0) return false;
+    if (wrows % 16 != 0 || p.K % 128 != 0 || p.K < 8 * 128) return false;
     if (p.group != 0 && p.group != 128) return false;
     if (p.group == 128) {
         const bool tables16 = is16(p.scale_dtype) && (!p.zp || p.zp_dtype == p.scale_dtype) &&
@@ -382,22 +398,41 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
                               (!p.zp || ((uintptr_t)p.zp % (8 * NH)) == 0);
         if (!tables16) return false;
     }
-    const int tiles = wrows / 64;
-    if (tiles < 128) return false;   // too few workgroups to fill the chip: the streaming kernel splits K further
-    const int mb = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
+    // rows per workgroup: 64, 32 or 16.  Fewer rows make more workgroups (a better fill of the 256
+    // CUs, counted in whole rounds) but share each activation slab between fewer waves and allow
+    // fewer activation rows per pass, hence the bonus for the larger ones.
+    int rt = 0;
+    double best = 0.0;
+    for (int cand = 4; cand >= 1; cand >>= 1) {
+        if (wrows % (16 * cand) != 0) continue;
+        const int t = wrows / (16 * cand);
+        const double fill = (double)t / (((t + 255) / 256) * 256);
+        const double score = fill * (cand == 4 ? 1.0 : cand == 2 ? 0.9 : 0.6);
+        if (score > best) { best = score; rt = cand; }
+    }
+    const int mb_max = rt;   // 16-row activation blocks per pass
+    const int mb = p.M <= 16 ? 1 : p.M <= 32 ? (mb_max >= 2 ? 2 : 1) : (mb_max >= 4 ? 4 : mb_max);
+    const int tiles = wrows / (16 * rt);
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);
     p.m_base = 0;
-#define FNN_PANEL2(G, SDTV, MBV)                                                                         \
+#define FNN_PANEL2(G, SDTV, MBV, RTV)                                                                    \
     do {                                                                                                 \
-        if (passes == 1) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, 2, 4, true><<<grid, dim3(512), 0, st>>>(p, passes); \
-        else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, 2, 4, false><<<grid, dim3(512), 0, st>>>(p, passes);         \
+        if (passes == 1) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, true><<<grid, dim3(512), 0, st>>>(p, passes); \
+        else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, false><<<grid, dim3(512), 0, st>>>(p, passes);         \
     } while (0)
-#define FNN_PANEL(G, SDTV)                       \
-    do {                                         \
-        if (mb == 1) FNN_PANEL2(G, SDTV, 1);     \
-        else if (mb == 2) FNN_PANEL2(G, SDTV, 2);\
-        else FNN_PANEL2(G, SDTV, 4);             \
+#define FNN_PANEL(G, SDTV)                                   \
+    do {                                                     \
+        if (rt == 4) {                                       \
+            if (mb == 1) FNN_PANEL2(G, SDTV, 1, 4);          \
+            else if (mb == 2) FNN_PANEL2(G, SDTV, 2, 4);     \
+            else FNN_PANEL2(G, SDTV, 4, 4);                  \
+        } else if (rt == 2) {                                \
+            if (mb == 1) FNN_PANEL2(G, SDTV, 1, 2);          \
+            else FNN_PANEL2(G, SDTV, 2, 2);                  \
+        } else {                                             \
+            FNN_PANEL2(G, SDTV, 1, 1);                       \
+        }                                                    \
     } while (0)
     if (p.group == 128) {
         if (p.scale_dtype == FNN_F16) FNN_PANEL(true, FNN_F16);

@@ -267,6 +267,18 @@ def test_weight_only_many_rows(bits, group, M, K):
     _wo_check(*case, group, bits, act_ty)
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("group", [0, 128])
+@pytest.mark.parametrize("M,N8,K", [(5, 1024, 1152), (20, 2048, 1024), (40, 1040, 2304), (33, 6400, 1280)])
+def test_weight_only_many_rows_small_matrices(bits, group, M, N8, K):
+    """Few weight rows: 16- and 32-row workgroups, K parts that differ by one slab (K = 9, 18 and 10
+    slabs of 128 over 8 or 4 parts), several passes over the activation rows."""
+    N = N8 * (2 if bits == 4 else 1)
+    act_ty = torch.float16 if M % 2 else torch.bfloat16
+    case = _wo_inputs(M, N, K, group, bits, act_ty, torch.float16, with_zp=M != 20, with_bias=M == 5, seed=100 + M)
+    _wo_check(*case, group, bits, act_ty)
+
+
 def test_weight_only_many_rows_one_hot():
     """Rows of the activation matrix that hold a single non-zero entry pick single weight columns:
     checks the k order inside the slabs and the row -> output mapping exactly."""
