@@ -64,11 +64,16 @@ def dtype_code(dt):
 
 
 def current_stream(device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    """Raw hipStream_t of torch's current stream on `device` (an int; 0 is the null stream)."""
+    idx = device.index
+    if idx is None:
+        idx = torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(idx)
 
 
 def ptr(t):
-    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+    """Device address as an int (None -> NULL); ctypes converts it for a void* parameter."""
+    return t.data_ptr() if t is not None else None
 
 
 def check(rc):

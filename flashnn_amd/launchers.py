@@ -46,7 +46,8 @@ def hip_rmsnorm_dquant_forward(x, weight, eps):
 
 
 def _flat_scale(t, n, what):
-    t = torch.squeeze(t)
+    if t.dim() != 1:
+        t = torch.squeeze(t)
     if t.dim() == 0:
         t = t.reshape(1)
     assert t.dim() == 1 and t.numel() == n, f"{what} must have {n} entries"
@@ -101,27 +102,36 @@ def _weight_only(fn_name, out, act, quant_w, scale_w, bias, zero_points, n_out):
     assert act.shape[1] == quant_w.shape[1], "Matrix B must be transposed"
     _lib.require_gpu(out, act, quant_w, scale_w, bias, zero_points)
     lib = _lib.load()
-    scale_w = scale_w.squeeze()
     M, K = act.shape
     N = n_out
     assert out.shape == (M, N) and out.stride(1) == 1
+    # the common layouts ([N] or [K/g, N], contiguous) pass through without creating views
+    if not (scale_w.dim() == 1 or (scale_w.dim() == 2 and scale_w.shape[0] > 1 and scale_w.shape[1] == N)):
+        scale_w = scale_w.squeeze()
     if scale_w.dim() <= 1:
         group = 0
-        scale_w = scale_w.reshape(-1)
+        if scale_w.dim() == 0:
+            scale_w = scale_w.reshape(-1)
         assert scale_w.numel() == N
     else:
         assert scale_w.dim() == 2 and scale_w.shape[1] == N
         group = int(K / scale_w.shape[0])
         assert group > 0, "k_per_scale should greater than 0"
         assert group * scale_w.shape[0] == K, "K must be a multiple of the scale rows"
-    scale_w = scale_w.contiguous()
+    if not scale_w.is_contiguous():
+        scale_w = scale_w.contiguous()
     zp = None
     if zero_points is not None:
-        zp = zero_points.squeeze().reshape(scale_w.shape).contiguous()
+        zp = zero_points
+        if zp.shape != scale_w.shape:
+            zp = zp.squeeze().reshape(scale_w.shape)
+        if not zp.is_contiguous():
+            zp = zp.contiguous()
         if zp.dtype != scale_w.dtype:
             zp = zp.to(scale_w.dtype)   # zero points are small integers: exact in any float type
     if bias is not None:
-        bias = bias.reshape(-1).contiguous()
+        if bias.dim() != 1 or not bias.is_contiguous():
+            bias = bias.reshape(-1).contiguous()
         assert bias.numel() == N
     fn = getattr(lib, fn_name)
     _lib.check(fn(_lib.ptr(out), _lib.ptr(act), _lib.ptr(quant_w), _lib.ptr(scale_w), _lib.ptr(bias),
