@@ -937,8 +937,9 @@ static void launch_stream(WoArgs& p, hipStream_t st) {
     else gemm_wo_stream_kernel<WBITS, ADT, MB, false><<<grid, block, 0, st>>>(p);
 }
 
+// gemv_only: take the one-wave-per-tile kernel or nothing
 template <int WBITS, int ADT>
-static bool launch_decode(WoArgs& p, hipStream_t st) {
+static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
     constexpr int NH = WBITS == 4 ? 2 : 1;
     if (p.M > 8 || p.K % 128 != 0) return false;
     if (p.group > 0 && (p.group % 128 != 0)) return false;
@@ -986,6 +987,7 @@ static bool launch_decode(WoArgs& p, hipStream_t st) {
             return true;
         }
     }
+    if (gemv_only) return false;
     if (tables16 && act_lds && (p.group == 0 || p.group == 128)) {
         const int steps = p.K / 128;
         const bool full16 = steps % (kDecWaves * 16) == 0, full8 = steps % (kDecWaves * 8) == 0;
@@ -1024,10 +1026,13 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
         gemm_wo_any_kernel<WBITS, ADT><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(p);
         return;
     }
-    // from 5 activation rows on, four weight tiles sharing the activations through LDS beat the
-    // decode kernels wherever there are enough weight rows to fill the chip that way
-    if (p.M > 4 && launch_wo_panel(p, WBITS, ADT, st)) return;
-    if (launch_decode<WBITS, ADT>(p, st)) return;
+    // Measured order of preference: the one-wave-per-tile kernel for up to 4 rows over int4 weights
+    // with many tiles (and for a single row over int8 weights); from 2 rows on the panel kernel,
+    // whose waves share the activations through LDS; the other decode kernels for a single row and
+    // for the shapes the panel kernel does not take.
+    if (p.M <= 4 && (WBITS == 4 || p.M == 1) && launch_decode<WBITS, ADT>(p, st, true)) return;
+    if (p.M >= 2 && launch_wo_panel(p, WBITS, ADT, st)) return;
+    if (launch_decode<WBITS, ADT>(p, st, false)) return;
     // up to 64 activation rows per pass over the weights
     for (int m0 = 0; m0 < p.M; m0 += 64) {
         p.m_base = m0;

@@ -217,37 +217,45 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         }
     };
 
+    // All activation fragments of the slab are requested first, the weights are converted while
+    // those reads are in flight, and the MFMAs then run back to back behind a single wait.
     auto compute = [&](const char* stage, const v4u w0, const v4u w1) {
+        v4u bf[2][MB][2];
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const v4u w = s == 0 ? w0 : w1;
-            if constexpr (WBITS == 4) {
-                v4u e0, e1, o0, o1;
-                convert_w4_nat<ADT>(w, e0, e1, o0, o1);
+        for (int s = 0; s < 2; ++s)
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    const v4u b0 = *(const v4u*)(stage + rd[s][0] + mb * 4096);
-                    const v4u b1 = *(const v4u*)(stage + rd[s][1] + mb * 4096);
-                    accg[mb][0] = MT::mma(e0, b0, accg[mb][0]);
-                    accg[mb][1] = MT::mma(o0, b0, accg[mb][1]);
-                    asum[mb] = MT::mma(ones, b0, asum[mb]);
-                    accg[mb][0] = MT::mma(e1, b1, accg[mb][0]);
-                    accg[mb][1] = MT::mma(o1, b1, accg[mb][1]);
-                    asum[mb] = MT::mma(ones, b1, asum[mb]);
-                }
-            } else {
-                v4u s0, s1;
-                convert_w8<ADT>(w, s0, s1);
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    const v4u b0 = *(const v4u*)(stage + rd[s][0] + mb * 4096);
-                    const v4u b1 = *(const v4u*)(stage + rd[s][1] + mb * 4096);
-                    accg[mb][0] = MT::mma(s0, b0, accg[mb][0]);
-                    asum[mb] = MT::mma(ones, b0, asum[mb]);
-                    accg[mb][0] = MT::mma(s1, b1, accg[mb][0]);
-                    asum[mb] = MT::mma(ones, b1, asum[mb]);
-                }
+            for (int mb = 0; mb < MB; ++mb) {
+                bf[s][mb][0] = *(const v4u*)(stage + rd[s][0] + mb * 4096);
+                bf[s][mb][1] = *(const v4u*)(stage + rd[s][1] + mb * 4096);
             }
+        if constexpr (WBITS == 4) {
+            v4u e[2][2], o[2][2];
+            convert_w4_nat<ADT>(w0, e[0][0], e[0][1], o[0][0], o[0][1]);
+            convert_w4_nat<ADT>(w1, e[1][0], e[1][1], o[1][0], o[1][1]);
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    accg[mb][0] = MT::mma(e[s][0], bf[s][mb][0], accg[mb][0]);
+                    accg[mb][1] = MT::mma(o[s][0], bf[s][mb][0], accg[mb][1]);
+                    asum[mb] = MT::mma(ones, bf[s][mb][0], asum[mb]);
+                    accg[mb][0] = MT::mma(e[s][1], bf[s][mb][1], accg[mb][0]);
+                    accg[mb][1] = MT::mma(o[s][1], bf[s][mb][1], accg[mb][1]);
+                    asum[mb] = MT::mma(ones, bf[s][mb][1], asum[mb]);
+                }
+        } else {
+            v4u c[2][2];
+            convert_w8<ADT>(w0, c[0][0], c[0][1]);
+            convert_w8<ADT>(w1, c[1][0], c[1][1]);
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    accg[mb][0] = MT::mma(c[s][0], bf[s][mb][0], accg[mb][0]);
+                    asum[mb] = MT::mma(ones, bf[s][mb][0], asum[mb]);
+                    accg[mb][0] = MT::mma(c[s][1], bf[s][mb][1], accg[mb][0]);
+                    asum[mb] = MT::mma(ones, bf[s][mb][1], asum[mb]);
+                }
         }
     };
 
