@@ -100,7 +100,9 @@ def test_a8w8_guarded_kernel_bit_exact(mnk):
 
 
 @pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 48, 64])
-@pytest.mark.parametrize("nk", [(1000, 64), (16, 448), (4100, 4096), (520, 8192)])
+@pytest.mark.parametrize("nk", [(1000, 64), (16, 448), (4100, 4096), (520, 8192),
+                                # shared activation slabs: 16-, 32- and 64-row workgroups, uneven K parts
+                                (4096, 4096), (8192, 1152), (16384, 1024), (2048, 11008)])
 def test_a8w8_few_rows_bit_exact(M, nk):
     """Up to 64 activation rows take the weight-streaming kernel: accumulators and scaled outputs,
     N not a multiple of the 16-row tile, fewer k-steps than waves."""
