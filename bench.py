@@ -201,7 +201,8 @@ def main():
                 f(i)
             ms = _events_ms(f, 100, torch)
             b5 = float(n5) * k5 + m5 * k5 + 2.0 * m5 * n5 + 2.0 * m5 + 4.0 * n5
-            secondary.append({"workload": f"a8w8 few rows M={m5} K={k5} N={n5} bf16", "kernel": "gemm_a8w8_skinny_kernel",
+            secondary.append({"workload": f"a8w8 few rows M={m5} K={k5} N={n5} bf16",
+                              "kernel": "gemm_a8w8_skinny_kernel" if m5 == 1 else "gemm_a8w8_panel_kernel",
                               "us_per_launch": round(ms * 1e3, 2),
                               "roofline": {"bound": "hbm", "achieved": round(b5 / (ms * 1e-3) / 1e9, 1),
                                            "peak": PEAK_HBM_GBS, "unit": "GB/s",
