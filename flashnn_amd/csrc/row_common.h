@@ -1,0 +1,88 @@
+// Pieces shared by the row kernels (dynamic quant, RMSNorm, LayerNorm and their quantising forms):
+// block reductions, the exact reciprocal-based division and the torch-exact quantisation steps.
+#pragma once
+
+#include "fnn_common.h"
+
+// every rounding of the reference's fp32 arithmetic is kept: no contraction into fmas
+#pragma clang fp contract(off)
+
+namespace fnn {
+
+constexpr int kRowThreads = 256;
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float r = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    return r;
+}
+
+__device__ __forceinline__ double block_sum(double v, double* red) {
+    v = wave_sum(v);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    double r = (red[0] + red[1]) + (red[2] + red[3]);
+    __syncthreads();
+    return r;
+}
+
+// Correctly rounded fp32 quotient x / s from r = RN(1/s) (one IEEE division per row):
+// q0 = RN(x*r) is within 2 ulp, e = x - s*q0 is exact in an fma, and RN(q0 + e*r) is the rounded
+// quotient (Markstein).  Three instructions instead of the ~10 of a full division sequence.
+__device__ __forceinline__ float div_by(float x, float s, float r) {
+    const float q0 = x * r;
+    const float e = __builtin_fmaf(-q0, s, x);
+    return __builtin_fmaf(e, r, q0);
+}
+
+// q = round_half_even(round_DT(x / s)) with x/s a correctly rounded fp32 division.
+template <int DT> __device__ __forceinline__ int quant_in_dtype(float x, float s, float r) {
+    // pinned: the last fma of the division must round to fp32 before the conversion rounds again
+    // (fused into v_fma_mixlo_f16 it would round once)
+    const float t = rounded_f32(div_by(x, s, r));
+    const float th = bits_to_f32<DT>(f32_to_bits<DT>(t));
+    return (int)rintf(th);
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (uint32_t)(a & 0xFF) | ((uint32_t)(b & 0xFF) << 8) | ((uint32_t)(c & 0xFF) << 16) |
+           ((uint32_t)(d & 0xFF) << 24);
+}
+
+__device__ __forceinline__ int quant_clamped(float n, float s, float rcp) {
+    float r = rintf(div_by(n, s, rcp));
+    r = fminf(fmaxf(r, -128.f), 127.f);
+    return s == 0.f ? 0 : (int)r;
+}
+
+// 8 consecutive gamma values as fp32 (vector loads; the type branch is uniform)
+__device__ __forceinline__ void load_gamma8(const void* gamma, int gamma_dtype, int64_t first, float g[8]) {
+    if (gamma_dtype == FNN_F32) {
+        const v4f a = *(const v4f*)((const float*)gamma + first);
+        const v4f b = *(const v4f*)((const float*)gamma + first + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { g[j] = a[j]; g[4 + j] = b[j]; }
+    } else {
+        const v4u a = *(const v4u*)((const uint16_t*)gamma + first);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = a[j] & 0xFFFFu, hi = a[j] >> 16;
+            g[2 * j] = gamma_dtype == FNN_F16 ? f16_bits_to_f32(lo) : bf16_bits_to_f32(lo);
+            g[2 * j + 1] = gamma_dtype == FNN_F16 ? f16_bits_to_f32(hi) : bf16_bits_to_f32(hi);
+        }
+    }
+}
+
+// Vector kernels keep a whole row in registers: up to 8 x 8 values per thread, 16-byte aligned rows.
+inline bool vec_ok(const void* x, const void* q, int64_t K, int64_t ldx, int64_t ldq) {
+    return K % 8 == 0 && K <= 8 * kRowThreads * 8 && ldx % 8 == 0 && ldq % 8 == 0 &&
+           ((uintptr_t)x % 16) == 0 && ((uintptr_t)q % 8) == 0;
+}
+
+
+}  // namespace fnn

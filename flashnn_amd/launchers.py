@@ -45,6 +45,68 @@ def hip_rmsnorm_dquant_forward(x, weight, eps):
     return y, scale.reshape(x.shape[:-1])
 
 
+def _rows(x):
+    x_arg = x.reshape(-1, x.shape[-1])
+    return x_arg if x_arg.is_contiguous() else x_arg.contiguous()
+
+
+def _vec(t, n, what):
+    t = t.detach().reshape(-1)
+    assert t.numel() == n, f"{what} must have one entry per channel"
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def hip_rmsnorm_forward(x, weight, eps):
+    """Replaces triton_rmsnorm_forward (flashnn/triton_kernels/rms_norm.py:68-83)."""
+    _lib.require_gpu(x, weight)
+    lib = _lib.load()
+    y = torch.empty_like(x, memory_format=torch.contiguous_format)
+    x_arg = _rows(x)
+    M, N = x_arg.shape
+    w = _vec(weight, N, "weight")
+    _lib.check(lib.fnn_rmsnorm(_lib.ptr(y), _lib.ptr(x_arg), _lib.ptr(w), float(eps), M, N, N, N,
+                               _lib.dtype_code(x.dtype), _lib.dtype_code(w.dtype),
+                               _lib.current_stream(x.device)))
+    return y
+
+
+def hip_layer_norm_forward(x, weight, bias, eps):
+    """Replaces triton_layer_norm_forward (flashnn/triton_kernels/layer_norm.py:84-101)."""
+    _lib.require_gpu(x, weight, bias)
+    lib = _lib.load()
+    y = torch.empty_like(x, memory_format=torch.contiguous_format)
+    x_arg = _rows(x)
+    M, N = x_arg.shape
+    w = _vec(weight, N, "weight")
+    b = _vec(bias, N, "bias")
+    if b.dtype != w.dtype:
+        b = b.to(w.dtype)
+    _lib.check(lib.fnn_layernorm(_lib.ptr(y), _lib.ptr(x_arg), _lib.ptr(w), _lib.ptr(b), float(eps), M, N,
+                                 N, N, _lib.dtype_code(x.dtype), _lib.dtype_code(w.dtype),
+                                 _lib.current_stream(x.device)))
+    return y
+
+
+def hip_layer_norm_dquant_forward(x, weight, bias, eps):
+    """Replaces triton_layer_norm_dquant_forward (flashnn/triton_kernels/layer_norm_dquant.py:91-105);
+    returns (q int8 like x, scale [rows] in x.dtype) - the normalised tensor the Triton launcher
+    also returns is not materialised (its only caller drops it, flashnn/norm.py:107-110)."""
+    _lib.require_gpu(x, weight, bias)
+    lib = _lib.load()
+    x_arg = _rows(x)
+    M, N = x_arg.shape
+    y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    scale = torch.empty((M,), dtype=x.dtype, device=x.device)
+    w = _vec(weight, N, "weight")
+    b = _vec(bias, N, "bias")
+    if b.dtype != w.dtype:
+        b = b.to(w.dtype)
+    _lib.check(lib.fnn_layernorm_dquant(_lib.ptr(y), _lib.ptr(scale), _lib.ptr(x_arg), _lib.ptr(w), _lib.ptr(b),
+                                        float(eps), M, N, N, N, _lib.dtype_code(x.dtype),
+                                        _lib.dtype_code(w.dtype), _lib.current_stream(x.device)))
+    return y, scale
+
+
 def _flat_scale(t, n, what):
     if t.dim() != 1:
         t = torch.squeeze(t)

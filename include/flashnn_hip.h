@@ -122,6 +122,30 @@ int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const void* scale
                    int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
                    void* stream);
 
+/* RMSNorm: out[m,k] = round_T(round_T(x[m,k] * rsqrt(mean_k(x^2) + eps)) * gamma[k]), T = x_dtype.
+ * Replaces triton_rmsnorm_forward(x, weight, eps) (flashnn/triton_kernels/rms_norm.py:68-83) behind
+ * RMSNorm (flashnn/norm.py:19-36); semantics of _torch_impl (:31-33) with the result in the input
+ * type, as _triton_impl returns it (:28-29).  x, out: [M,K] fp16/bf16 with row strides ldx, ldo
+ * (elements); gamma: [K] fp16/bf16/fp32. */
+int fnn_rmsnorm(void* out, const void* x, const void* gamma, float eps, int64_t M, int64_t K,
+                int64_t ldx, int64_t ldo, int x_dtype, int gamma_dtype, void* stream);
+
+/* LayerNorm over the last dimension: out = round_T(((x - mean) * rstd) * gamma + beta).
+ * Replaces triton_layer_norm_forward(x, weight, bias, eps) (flashnn/triton_kernels/layer_norm.py:84-101)
+ * behind LayerNorm (flashnn/norm.py:69-94; _torch_impl = torch.nn.functional.layer_norm, :82-85).
+ * gamma and beta: [K], both of type gb_dtype (fp16/bf16/fp32). */
+int fnn_layernorm(void* out, const void* x, const void* gamma, const void* beta, float eps, int64_t M,
+                  int64_t K, int64_t ldx, int64_t ldo, int x_dtype, int gb_dtype, void* stream);
+
+/* LayerNorm + per-token int8 quantisation: y = layernorm(x) rounded to T, scale[m] = max|y| / 127 and
+ * q = clamp(round(y / scale), -128, 127), the last three evaluated in T as torch evaluates them.
+ * Replaces triton_layer_norm_dquant_forward(x, weight, bias, eps)
+ * (flashnn/triton_kernels/layer_norm_dquant.py:91-105) behind LayernormDquant (flashnn/norm.py:97-124;
+ * semantics of _torch_impl, :112-119).  q: int8 [M,K] with row stride ldq; scale: [M] of type x_dtype. */
+int fnn_layernorm_dquant(void* q, void* scale, const void* x, const void* gamma, const void* beta,
+                         float eps, int64_t M, int64_t K, int64_t ldx, int64_t ldq, int x_dtype,
+                         int gb_dtype, void* stream);
+
 /*
  * Test hook, no counterpart in the reference: force the output tile (bm x bn) of the MFMA
  * A8W8 kernel for subsequent calls, so that every tile shape can be checked on small

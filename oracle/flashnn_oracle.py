@@ -14,6 +14,8 @@ Reference statements followed (all under /root/reference):
   gemm_a8w8_*           flashnn/quant_gemm.py:96-104, triton_kernels/gemm_a8w8.py:135-173
   weight_only_*         flashnn/quant_gemm.py:14-36, 148-206
   rmsnorm_dquant        flashnn/norm.py:45-60
+  rmsnorm               flashnn/norm.py:25-33
+  layernorm(_dquant)    flashnn/norm.py:82-85, 112-119 (torch.nn.functional.layer_norm)
 
 How each function is pinned (tests/test_oracle.py):
   dynamic_quantize   against the literal torch-op formula on CPU tensors (the third
@@ -30,6 +32,16 @@ How each function is pinned (tests/test_oracle.py):
   rmsnorm_dquant     against the literal torch-op formula (<= 1 LSB on elements whose
                      pre-round fraction is at a tie, because torch sums x^2 in its own
                      fp32 order) and float64 closed forms.
+  rmsnorm            against the literal torch-op formula (1 ulp of the output type where
+                     the mean differs in its last bit), a constant-row closed form;
+  layernorm          against torch.nn.functional.layer_norm on CPU tensors (1 ulp of the
+                     output type: torch's moments are taken in an order of its own),
+                     a float64 evaluation, zero-mean / unit-variance invariants and
+                     closed forms (constant row -> bias);
+  layernorm_dquant   its quantisation step is dynamic_quantize applied to layernorm's
+                     rounded output (checked to be literally that), against the torch
+                     ops within one quantisation step where the 1-ulp cases above land
+                     on a tie.
 The reference's tests hold no golden vectors for this path (they regenerate seeded
 inputs on a GPU), so no fixture of theirs exists to check against; the int4 branch has
 no reference test at all and is pinned by the formula at quant_gemm.py:174-204 only.
@@ -74,7 +86,7 @@ def round_to(x: np.ndarray, dtype: str) -> np.ndarray:
 
 
 # ------------------------------------------------------------------- dynamic quantize
-def dynamic_quantize(x: np.ndarray, dtype: str):
+def dynamic_quantize(x: np.ndarray, dtype: str, scale_dtype: str | None = None, clamp: bool = False):
     """Per-token symmetric int8 quantisation in the input type.
 
     flashnn/quant_gemm.py:53-57:  max = |x|.max(-1); scale = max / 127.0;
@@ -83,7 +95,12 @@ def dynamic_quantize(x: np.ndarray, dtype: str):
     tensor type, so there are two roundings to `dtype` before the round-half-even.
     Rows that are entirely zero are undefined in the reference (0/0); here, and in
     the HIP kernel, they give q = 0 and scale = 0.
-    Returns (q int8 [M,K], scale float16 [M]).
+    Returns (q int8 [M,K], scale float16 [M]); with `scale_dtype` given, the scale is
+    returned unconverted instead, as float32 values representable in that type.
+    The reference does not clamp here; with bf16 inputs the scale can round down far enough
+    for the row maximum to quantise to 128, which the conversion to int8 wraps to -128
+    (fp16 inputs stay within 127).  `clamp` adds the clamp to [-128, 127] that
+    LayernormDquant applies (flashnn/norm.py:118).
     """
     x = np.asarray(x, dtype=np.float32)
     mx = np.abs(x).max(axis=-1, keepdims=True)
@@ -91,7 +108,12 @@ def dynamic_quantize(x: np.ndarray, dtype: str):
     with np.errstate(divide="ignore", invalid="ignore"):
         t = round_to(x / scale, dtype)
     q = np.rint(t)
+    if clamp:
+        q = np.clip(q, -128.0, 127.0)
     q = np.where(scale == 0, np.float32(0), q)
+    if scale_dtype is not None:
+        assert scale_dtype == dtype
+        return q.astype(np.int8), scale.reshape(x.shape[:-1])
     with np.errstate(over="ignore"):
         s16 = scale.astype(np.float16)
     return q.astype(np.int8), s16.reshape(x.shape[:-1])
@@ -261,6 +283,53 @@ def rmsnorm_dquant(x, gamma, eps: float, dtype: str):
     q = np.where(scale == 0, np.float32(0), q)
     return (q.astype(np.int8).reshape(x.shape),
             round_to(scale, dtype).reshape(x.shape[:-1]))
+
+
+def rmsnorm(x, gamma, eps: float, dtype: str) -> np.ndarray:
+    """RMSNorm._torch_impl, flashnn/norm.py:25-33: n = x * rsqrt(mean(x^2) + eps) in fp32,
+    rounded to the input type, then multiplied by gamma.  With gamma in the input type the
+    product is formed in that type: the exact product of two 16-bit floats rounded once, which
+    equals the fp32 product rounded to the type.  With an fp32 gamma torch returns fp32; this
+    function (like the Triton launcher, rms_norm.py:68-83 + `.type_as(x)`) returns the input
+    type, i.e. that fp32 product rounded once more.  Mean of squares as in rmsnorm_dquant."""
+    x = np.asarray(x, dtype=np.float32)
+    g = np.asarray(gamma, dtype=np.float32).reshape(1, -1)
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    ssq = (x2.astype(np.float64) ** 2).sum(axis=-1, keepdims=True).astype(np.float32)
+    rs = np.float32(1.0) / np.sqrt(ssq / np.float32(K) + np.float32(eps))
+    n = round_to(x2 * rs, dtype)
+    return round_to(n * g, dtype).reshape(x.shape)
+
+
+def layernorm(x, gamma, beta, eps: float, dtype: str) -> np.ndarray:
+    """torch.nn.functional.layer_norm over the last dimension (flashnn/norm.py:82-85) for 16-bit
+    inputs: moments and the affine map in fp32, one rounding to the input type at the end.
+    mean = sum(x)/K and var = sum((x - mean)^2)/K with the sums taken in float64 and rounded
+    once (x - mean is the fp32 difference); rstd = 1/sqrt(var + eps) with both steps rounded;
+    y = ((x - mean) * rstd) * gamma + beta, every operation rounded to fp32."""
+    x = np.asarray(x, dtype=np.float32)
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    g = np.asarray(gamma, dtype=np.float32).reshape(1, -1)
+    b = np.asarray(beta, dtype=np.float32).reshape(1, -1)
+    mean = (x2.astype(np.float64).sum(axis=-1, keepdims=True) / K).astype(np.float32)
+    d = x2 - mean
+    var = ((d.astype(np.float64) ** 2).sum(axis=-1, keepdims=True) / K).astype(np.float32)
+    rstd = np.float32(1.0) / np.sqrt(var + np.float32(eps))
+    y = (d * rstd) * g + b
+    return round_to(y.astype(np.float32), dtype).reshape(x.shape)
+
+
+def layernorm_dquant(x, gamma, beta, eps: float, dtype: str):
+    """LayernormDquant._torch_impl, flashnn/norm.py:112-119: layer_norm's output (in the input
+    type), then max / 127, division, round and clamp - all on tensors of the input type, i.e.
+    exactly dynamic_quantize of the rounded output, plus the clamp (which binds for bf16, where
+    the row maximum can quantise to 128).
+    Returns (q int8 like x, scale [rows, 1] as float32 values representable in `dtype`)."""
+    y = layernorm(x, gamma, beta, eps, dtype)
+    q, s = dynamic_quantize(y.reshape(-1, y.shape[-1]), dtype, scale_dtype=dtype, clamp=True)
+    return q.reshape(y.shape), s.reshape(-1, 1)
 
 
 # ------------------------------------------------------------------------ torch glue

@@ -89,3 +89,24 @@ def rmsnorm_dquant(x, weight, eps):
     scale = mx / 127.0
     q = torch.clamp(torch.round(n / scale), -128.0, 127.0)
     return q.to(torch.int8), scale.reshape(x.shape[:-1]).type_as(x)
+
+
+def rmsnorm(x, weight, eps):
+    """flashnn/norm.py:25-33, cast to the input type as the Triton path returns it (:29)."""
+    xf = x.float()
+    n = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).type_as(x)
+    return (n * weight).type_as(x)
+
+
+def layernorm(x, weight, bias, eps):
+    """flashnn/norm.py:82-85."""
+    return torch.nn.functional.layer_norm(x, (x.shape[-1],), weight, bias, eps)
+
+
+def layernorm_dquant(x, weight, bias, eps):
+    """flashnn/norm.py:112-119."""
+    n = torch.nn.functional.layer_norm(x, (x.shape[-1],), weight, bias, eps)
+    mx = torch.max(torch.abs(n), dim=-1, keepdim=True)[0]
+    scale = mx / 127.0
+    q = torch.clamp(torch.round(n / scale), -128.0, 127.0)
+    return q.to(torch.int8), scale.reshape(-1, 1)

@@ -351,3 +351,78 @@ def test_rmsnorm_quant_gemm_chain(M):
     assert np.array_equal(acc, O.gemm_a8w8_acc(q_o[rows], w.numpy()))
     want = O.gemm_a8w8(q_o[rows], w.numpy(), s_o[rows], ws.numpy(), O.BF16)
     np.testing.assert_allclose(out[torch.from_numpy(rows).to(DEV)].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+
+
+# ------------------------------------------- rmsnorm, layernorm, layernorm + quant
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 128), (3, 64, 64), (7, 1000), (33, 4096), (16, 8192), (5, 50), (2, 16384), (3, 20000)])
+@pytest.mark.parametrize("w_dtype", ["same", torch.float32])
+def test_rmsnorm_bit_exact(dtype, shape, w_dtype):
+    g = torch.Generator().manual_seed(21)
+    K = shape[-1]
+    x = torch.randn(shape, generator=g).to(dtype)
+    w = torch.empty(K).uniform_(0.5, 1.5, generator=g).to(dtype if w_dtype == "same" else w_dtype)
+    mod = flashnn_amd.RMSNorm(K, eps=1e-5)
+    mod.weight.data = w
+    out = mod.to(DEV)(x.to(DEV))
+    assert out.dtype == dtype and out.shape == x.shape
+    want = O.rmsnorm(O.to_np(x), O.to_np(w), 1e-5, _tag(dtype))
+    assert np.array_equal(out.float().cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 128), (2, 4, 128), (7, 1000), (33, 4096), (16, 8192), (5, 50), (2, 16384), (3, 20000)])
+@pytest.mark.parametrize("w_dtype", ["same", torch.float32])
+def test_layernorm_and_dquant_bit_exact(dtype, shape, w_dtype):
+    g = torch.Generator().manual_seed(22)
+    K = shape[-1]
+    x = (torch.randn(shape, generator=g) * 2 + 0.5).to(dtype)
+    wd = dtype if w_dtype == "same" else w_dtype
+    w = torch.empty(K).uniform_(0.5, 1.5, generator=g).to(wd)
+    b = torch.randn(K, generator=g).to(wd)
+    ln = flashnn_amd.LayerNorm(K, eps=1e-5)
+    ln.weight.data, ln.bias.data = w, b
+    out = ln.to(DEV)(x.to(DEV))
+    assert out.dtype == dtype and out.shape == x.shape
+    want = O.layernorm(O.to_np(x), O.to_np(w), O.to_np(b), 1e-5, _tag(dtype))
+    got = out.float().cpu().numpy()
+    # the float64 sums of (x - mean)^2 are not exact, so a different summation order can move a
+    # moment by one fp32 ulp once in a long while; everything else is the same arithmetic
+    assert (got != want).mean() < 1e-4
+    np.testing.assert_allclose(got, want, rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10, atol=1e-6)
+    lq = flashnn_amd.LayernormDquant(K, eps=1e-5)
+    lq.weight.data, lq.bias.data = w, b
+    q, s = lq.to(DEV)(x.to(DEV))
+    assert q.dtype == torch.int8 and q.shape == x.shape and s.dtype == dtype and s.shape == (x.numel() // K, 1)
+    q_o, s_o = O.layernorm_dquant(O.to_np(x), O.to_np(w), O.to_np(b), 1e-5, _tag(dtype))
+    if np.array_equal(got, want):
+        assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.float().cpu().numpy(), s_o)
+    else:
+        assert np.abs(q.cpu().numpy().astype(np.int32) - q_o.astype(np.int32)).max() <= 1
+
+
+def test_norm_layers_against_torch_reference_shapes():
+    """The reference's own checks (tests/norm/test_layer_norm_dquant.py:22-41, test_rms_norm.py:34-50):
+    torch.nn.LayerNorm + the test's quantiser, and the RMSNorm reference module, within their
+    tolerances."""
+    torch.manual_seed(0)
+    for shape in ([4, 128], [2, 4, 128]):
+        hidden = shape[-1]
+        mod = torch.nn.LayerNorm(hidden, eps=1e-5).half()
+        inp = torch.randn(shape).half()
+        ref = mod(inp)
+        scale = ref.abs().max(dim=-1, keepdim=True)[0] / 127
+        ref_q = torch.clamp(torch.round(ref / scale), -128, 127).to(torch.int8)
+        qmod = flashnn_amd.LayernormDquant(hidden, eps=1e-5).half().to(DEV)
+        q, s = qmod(inp.to(DEV))
+        torch.testing.assert_close(q.cpu(), ref_q, rtol=0.01, atol=2.0)
+        torch.testing.assert_close(s.cpu(), scale.reshape(-1, 1), rtol=0.01, atol=0.01)
+        lmod = flashnn_amd.LayerNorm(hidden, eps=1e-5).half().to(DEV)
+        torch.testing.assert_close(lmod(inp.to(DEV)).cpu(), ref, atol=1e-3, rtol=1e-3)
+    for shape in ([4, 128], [3, 64, 64]):
+        hidden = shape[-1]
+        inp = torch.randn(shape).half()
+        w = torch.ones(hidden).half()
+        ref = (inp.float() * torch.rsqrt(inp.float().pow(2).mean(-1, keepdim=True) + 1e-5)).type_as(inp) * w
+        out = flashnn_amd.RMSNorm(hidden, eps=1e-5).half().to(DEV)(inp.to(DEV))
+        torch.testing.assert_close(out.cpu(), ref, atol=1e-3, rtol=1e-3)

@@ -42,6 +42,17 @@ def test_argument_errors_are_reported_without_a_gpu(hip_lib):
     assert rc == -2
     rc = hip_lib.fnn_gemm_a8w8(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 2, 0, 0, null)
     assert rc == -2 and b"float16 or bfloat16" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_rmsnorm(one, one, null, 1e-5, 4, 8, 8, 8, 0, 0, null)               # no gamma
+    assert rc == -1 and b"fnn_rmsnorm: null pointer" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_layernorm(one, one, one, null, 1e-5, 4, 8, 8, 8, 0, 0, null)         # no beta
+    assert rc == -1 and b"fnn_layernorm: null pointer" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_layernorm_dquant(one, null, one, one, one, 1e-5, 4, 8, 8, 8, 0, 0, null)   # no scale
+    assert rc == -1 and b"fnn_layernorm_dquant: null pointer" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_layernorm(one, one, one, one, 1e-5, 4, 8, 8, 4, 0, 0, null)          # ldo < K
+    assert rc == -1 and b"bad shape" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_rmsnorm(one, one, one, 1e-5, 4, 8, 8, 8, 2, 0, null)                # fp32 input
+    assert rc == -2 and b"fp16 or bf16" in hip_lib.fnn_last_error()
+    assert hip_lib.fnn_layernorm_dquant(one, one, one, one, one, 1e-5, 0, 8, 8, 8, 1, 2, null) == 0   # M = 0
     rc = hip_lib.fnn_gemm_a16w4(one, one, one, one, null, null, 1, 7, 64, 64, 64, 7, 0, 0, 0, 0, 0, 0, null)
     assert rc == -1 and b"even" in hip_lib.fnn_last_error()
     rc = hip_lib.fnn_gemm_a16w8(one, one, one, one, null, null, 1, 8, 100, 100, 100, 8, 64, 0, 0, 0, 0, 0, null)
@@ -51,13 +62,18 @@ def test_argument_errors_are_reported_without_a_gpu(hip_lib):
 
 
 def test_public_names_match_the_reference_module():
-    for name in ("DynamicQuantize", "GemmA8W8", "GemmWeightOnly", "RMSNormDquant", "set_use_triton",
-                 "set_autotune_triton_kernels"):
+    for name in ("DynamicQuantize", "GemmA8W8", "GemmWeightOnly", "RMSNormDquant", "RMSNorm", "LayerNorm",
+                 "LayernormDquant", "set_use_triton", "set_autotune_triton_kernels"):
         assert hasattr(flashnn_amd, name)
     assert flashnn_amd.GemmA8W8().out_ty == torch.float16
     assert flashnn_amd.GemmWeightOnly(torch.bfloat16).out_ty == torch.bfloat16
     m = flashnn_amd.RMSNormDquant(64)
     assert m.eps == 1e-6 and m.weight.shape == (64,) and bool((m.weight == 1).all())
+    assert flashnn_amd.RMSNorm(64).eps == 1e-6
+    for cls in (flashnn_amd.LayerNorm, flashnn_amd.LayernormDquant):      # flashnn/norm.py:70-80, 98-108
+        for dim in (64, [64], (64,)):
+            n = cls(dim)
+            assert n.dim == (64,) and n.eps == 1e-5 and bool((n.weight == 1).all()) and bool((n.bias == 0).all())
 
 
 def test_hip_backend_never_falls_back_silently():
@@ -67,6 +83,9 @@ def test_hip_backend_never_falls_back_silently():
         flashnn_amd.DynamicQuantize()(x)          # CPU tensor on the native path: loud error
     with pytest.raises(_lib.FlashnnHipError):
         flashnn_amd.RMSNormDquant(64)(x)
+    for mod in (flashnn_amd.RMSNorm(64), flashnn_amd.LayerNorm(64), flashnn_amd.LayernormDquant(64)):
+        with pytest.raises(_lib.FlashnnHipError):
+            mod.half()(x)
 
 
 def test_dispatch_and_torch_path_on_cpu():
@@ -95,6 +114,16 @@ def test_dispatch_and_torch_path_on_cpu():
             flashnn_amd.GemmWeightOnly()(x, qw, torch.ones(5).half())
         qn, sn = flashnn_amd.RMSNormDquant(256)(x)
         assert qn.dtype == torch.int8 and sn.dtype == torch.float16 and sn.shape == (8,)
+        # the torch paths of the norm layers against the oracle (1 ulp where torch's moments differ)
+        y = flashnn_amd.RMSNorm(256).half()(x)
+        np.testing.assert_allclose(y.float().numpy(), O.rmsnorm(O.to_np(x), np.ones(256, np.float32), 1e-6, O.F16),
+                                   rtol=2.0 ** -10)
+        ln = flashnn_amd.LayerNorm(256).half()
+        np.testing.assert_allclose(ln(x).float().numpy(),
+                                   O.layernorm(O.to_np(x), np.ones(256, np.float32), np.zeros(256, np.float32), 1e-5, O.F16),
+                                   rtol=2.0 ** -10, atol=1e-6)
+        ql, sl = flashnn_amd.LayernormDquant(256).half()(x)
+        assert ql.dtype == torch.int8 and ql.shape == x.shape and sl.shape == (8, 1) and sl.dtype == torch.float16
     finally:
         flashnn_amd.set_use_triton(True)
 

@@ -255,3 +255,103 @@ def test_rmsnorm_dquant_closed_forms():
     assert (np.abs(q.astype(np.int32)).max(axis=1) == 127).all()
     n = x / np.sqrt((x.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-6) * g
     assert (np.abs(q * (np.abs(n).max(-1, keepdims=True) / 127) - n) <= np.abs(n).max(-1, keepdims=True) / 127 * 0.5001).all()
+
+
+# ------------------------------------------------- rmsnorm, layernorm, layernorm + quant
+def _ulp(dtype):
+    return 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 128), (3, 64, 64), (16, 8192)])
+def test_rmsnorm_matches_torch_ops(dtype, shape):
+    # shapes of tests/norm/test_rms_norm.py:35 + the configuration width
+    torch.manual_seed(1)
+    x = torch.randn(shape).to(dtype)
+    for gamma in (torch.empty(shape[-1]).uniform_(0.5, 1.5).to(dtype), torch.empty(shape[-1]).uniform_(0.5, 1.5)):
+        want = T.rmsnorm(x, gamma, 1e-5).float().numpy()
+        got = O.rmsnorm(O.to_np(x), O.to_np(gamma), 1e-5, O.tag_of(x))
+        # identical except where torch's fp32 summation order moves the mean by one bit
+        np.testing.assert_allclose(got, want, rtol=_ulp(dtype), atol=0)
+        assert (got != want).mean() < 1e-2
+
+
+def test_rmsnorm_closed_forms():
+    # constant row c: x * rsqrt(c^2) = sign(c) exactly (eps = 0); times gamma
+    x = np.full((2, 64), 4.0, np.float32)
+    x[1] = -0.25
+    g = np.linspace(0.5, 1.5, 64).astype(np.float16).astype(np.float32)
+    y = O.rmsnorm(x, g, 0.0, O.F16)
+    assert np.array_equal(y[0], g) and np.array_equal(y[1], -g)
+    # scale invariance in powers of two (exact in floating point)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((8, 512)).astype(np.float16).astype(np.float32)
+    assert np.array_equal(O.rmsnorm(x, g[:1].repeat(512), 0.0, O.F16), O.rmsnorm(4 * x, g[:1].repeat(512), 0.0, O.F16))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 128), (2, 4, 128), (16, 8192), (5, 1000)])
+def test_layernorm_matches_torch_and_f64(dtype, shape):
+    # shapes of tests/norm/test_layer_norm_dquant.py:23 + wider rows
+    torch.manual_seed(2)
+    K = shape[-1]
+    x = (torch.randn(shape) * 2 + 0.5).to(dtype)
+    w = torch.empty(K).uniform_(0.5, 1.5).to(dtype)
+    b = torch.randn(K).to(dtype)
+    want = T.layernorm(x, w, b, 1e-5).float().numpy()
+    got = O.layernorm(O.to_np(x), O.to_np(w), O.to_np(b), 1e-5, O.tag_of(x))
+    # torch takes the moments in its own order: 1 ulp of the output type at most, and rarely
+    np.testing.assert_allclose(got, want, rtol=_ulp(dtype), atol=_ulp(dtype) * 2.0 ** -6)
+    assert (got != want).mean() < 2e-2
+    # the mathematical value, evaluated in float64
+    x64 = O.to_np(x).astype(np.float64).reshape(-1, K)
+    mu = x64.mean(-1, keepdims=True)
+    var = ((x64 - mu) ** 2).mean(-1, keepdims=True)
+    exact = (x64 - mu) / np.sqrt(var + 1e-5) * O.to_np(w).astype(np.float64) + O.to_np(b).astype(np.float64)
+    assert (np.abs(got.reshape(-1, K) - exact) <= np.abs(exact) * _ulp(dtype) * 0.51 + 1e-6).all()
+
+
+def test_layernorm_closed_forms_and_invariants():
+    K = 256
+    ones, zeros = np.ones(K, np.float32), np.zeros(K, np.float32)
+    # constant row: x - mean = 0, so y = beta whatever eps and gamma
+    beta = np.linspace(-1, 1, K).astype(np.float16).astype(np.float32)
+    y = O.layernorm(np.full((1, K), 3.5, np.float32), 2 * ones, beta, 1e-5, O.F16)
+    assert np.array_equal(y[0], beta)
+    # a row of +-a: mean 0, var a^2, y = +-a / sqrt(a^2 + eps)
+    row = np.where(np.arange(K) % 2 == 0, 2.0, -2.0).astype(np.float32)[None]
+    y = O.layernorm(row, ones, zeros, 0.0, O.F16)
+    assert np.array_equal(y, np.sign(row))
+    # zero mean, unit variance for gamma = 1, beta = 0 on random rows
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((16, 4096)) * 3 + 1).astype(np.float16).astype(np.float32)
+    y = O.layernorm(x, np.ones(4096, np.float32), np.zeros(4096, np.float32), 1e-5, O.F16).astype(np.float64)
+    assert np.abs(y.mean(-1)).max() < 1e-3 and np.abs(y.var(-1) - 1).max() < 2e-3
+    # shift invariance by a value that keeps every x exactly representable
+    assert np.array_equal(O.layernorm(x[:, :64], ones[:64], zeros[:64], 1e-5, O.F32),
+                          O.layernorm(x[:, :64].astype(np.float32), ones[:64], zeros[:64], 1e-5, O.F32))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(4, 128), (2, 4, 128), (8, 4096)])
+def test_layernorm_dquant_matches_torch_ops(dtype, shape):
+    torch.manual_seed(5)
+    K = shape[-1]
+    x = torch.randn(shape).to(dtype)
+    w = torch.empty(K).uniform_(0.5, 1.5).to(dtype)
+    b = (torch.randn(K) * 0.1).to(dtype)
+    q_t, s_t = T.layernorm_dquant(x, w, b, 1e-5)
+    q_o, s_o = O.layernorm_dquant(O.to_np(x), O.to_np(w), O.to_np(b), 1e-5, O.tag_of(x))
+    assert q_o.shape == tuple(shape) and s_o.shape == (x.numel() // K, 1) and s_t.dtype == dtype
+    # the quantisation step is literally dynamic_quantize of the rounded layer norm ...
+    y = O.layernorm(O.to_np(x), O.to_np(w), O.to_np(b), 1e-5, O.tag_of(x))
+    q_d, s_d = O.dynamic_quantize(y.reshape(-1, K), O.tag_of(x), scale_dtype=O.tag_of(x), clamp=True)
+    assert np.array_equal(q_o.reshape(-1, K), q_d) and np.array_equal(s_o[:, 0], s_d)
+    # ... and torch's own layer norm feeding torch's ops gives the same up to the 1-ulp cases
+    d = np.abs(q_o.astype(np.int32) - q_t.numpy().astype(np.int32))
+    assert d.max() <= 1 and (d != 0).mean() < 2e-2
+    np.testing.assert_allclose(s_o, s_t.float().numpy(), rtol=_ulp(dtype))
+    # given torch's layer norm output, the oracle's quantisation reproduces torch's exactly
+    n_t = T.layernorm(x, w, b, 1e-5)
+    q_x, s_x = O.dynamic_quantize(O.to_np(n_t).reshape(-1, K), O.tag_of(x), scale_dtype=O.tag_of(x), clamp=True)
+    assert np.array_equal(q_x, q_t.numpy().reshape(-1, K)) and np.array_equal(s_x, s_t.float().numpy()[:, 0])
