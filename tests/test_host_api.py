@@ -116,10 +116,10 @@ def test_dispatch_and_torch_path_on_cpu():
         assert qn.dtype == torch.int8 and sn.dtype == torch.float16 and sn.shape == (8,)
         # the torch paths of the norm layers against the oracle (1 ulp where torch's moments differ)
         y = flashnn_amd.RMSNorm(256).half()(x)
-        np.testing.assert_allclose(y.float().numpy(), O.rmsnorm(O.to_np(x), np.ones(256, np.float32), 1e-6, O.F16),
+        np.testing.assert_allclose(y.detach().float().numpy(), O.rmsnorm(O.to_np(x), np.ones(256, np.float32), 1e-6, O.F16),
                                    rtol=2.0 ** -10)
         ln = flashnn_amd.LayerNorm(256).half()
-        np.testing.assert_allclose(ln(x).float().numpy(),
+        np.testing.assert_allclose(ln(x).detach().float().numpy(),
                                    O.layernorm(O.to_np(x), np.ones(256, np.float32), np.zeros(256, np.float32), 1e-5, O.F16),
                                    rtol=2.0 ** -10, atol=1e-6)
         ql, sl = flashnn_amd.LayernormDquant(256).half()(x)
