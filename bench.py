@@ -243,6 +243,21 @@ def main():
                           "roofline": {"bound": "hbm", "achieved": round(rb / (ms * 1e-3) / 1e9, 1),
                                        "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                        "frac": round(rb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+        # the layers one step before the path, same matrix
+        for name, mod, kern, wr in (("rmsnorm", flashnn_amd.RMSNorm(Kr), "norm_vec_kernel", 2.0),
+                                    ("layernorm", flashnn_amd.LayerNorm(Kr), "norm_vec_kernel", 2.0),
+                                    ("layernorm_dquant", flashnn_amd.LayernormDquant(Kr), "norm_vec_kernel", 1.0)):
+            mod = mod.to(torch.bfloat16).to(dev)
+            f = lambda i: mod(hs[i % 3])
+            for i in range(5):
+                f(i)
+            ms = _events_ms(f, 50, torch)
+            nb = (2.0 + wr) * Mr * Kr
+            secondary.append({"workload": f"{name} bf16 M={Mr} K={Kr}", "kernel": kern,
+                              "us_per_launch": round(ms * 1e3, 2),
+                              "roofline": {"bound": "hbm", "achieved": round(nb / (ms * 1e-3) / 1e9, 1),
+                                           "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                           "frac": round(nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
         del hs
         torch.cuda.empty_cache()
 

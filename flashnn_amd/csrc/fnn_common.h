@@ -25,11 +25,10 @@ typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 // ---- 16-bit float <-> fp32 on raw bit patterns -------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-// round-to-nearest-even; inputs here are finite
+// round-to-nearest-even through the hardware conversion (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return u >> 16;
+    const v2bf t = __builtin_convertvector(v2f{f, f}, v2bf);
+    return __builtin_bit_cast(uint32_t, t) & 0xFFFFu;
 }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {

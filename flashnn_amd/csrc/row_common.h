@@ -31,6 +31,18 @@ __device__ __forceinline__ double block_sum(double v, double* red) {
     return r;
 }
 
+// two sums at once (one pair of barriers)
+__device__ __forceinline__ void block_sum2(double& a, double& b, double* red) {
+    a = wave_sum(a);
+    b = wave_sum(b);
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { red[w] = a; red[4 + w] = b; }
+    __syncthreads();
+    a = (red[0] + red[1]) + (red[2] + red[3]);
+    b = (red[4] + red[5]) + (red[6] + red[7]);
+    __syncthreads();
+}
+
 // Correctly rounded fp32 quotient x / s from r = RN(1/s) (one IEEE division per row):
 // q0 = RN(x*r) is within 2 ulp, e = x - s*q0 is exact in an fma, and RN(q0 + e*r) is the rounded
 // quotient (Markstein).  Three instructions instead of the ~10 of a full division sequence.

@@ -9,9 +9,11 @@
 //   layernorm + quant  the rounded y, then scale = max|y| / 127 and q = clamp(round(y / scale)), both
 //                      evaluated in the input type as torch evaluates them (flashnn/norm.py:112-119)
 //
-// Sums are taken in fp64 over exactly representable terms (x, x^2 and the fp32 differences squared)
-// and rounded once, so the kernels are bit-identical to a float64 restatement; torch's own fp32
-// summation order can differ from that in the last bit of a moment.
+// Sums are taken in fp64 over exactly representable terms (x and x^2 of 16-bit inputs: 22-bit
+// products, so a row whose magnitudes span less than 2^15 sums without any rounding); their order
+// then does not matter and the kernels are bit-identical to a float64 restatement
+// (var = sum(x^2)/K - (sum(x)/K)^2 in fp64, rounded once); torch's own fp32 moments can differ from
+// that in their last bit.
 #include "row_common.h"
 
 namespace fnn {
@@ -39,13 +41,13 @@ template <int DT> __device__ __forceinline__ float round_dt(float v) {
 
 template <int DT, int NV, int OP>
 __global__ __launch_bounds__(kRowThreads) void norm_vec_kernel(const NormArgs p) {
-    __shared__ double redd[4];
+    __shared__ double redd[8];
     __shared__ float red[4];
     const int64_t row = blockIdx.x;
     const v4u* xr = (const v4u*)(p.x + row * p.ldx);
     const int nvec = p.K >> 3;
     float n[NV][8];
-    double acc = 0.0;
+    double acc = 0.0, acc1 = 0.0;   // sum of squares; sum
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int idx = threadIdx.x + i * kRowThreads;
@@ -56,25 +58,25 @@ __global__ __launch_bounds__(kRowThreads) void norm_vec_kernel(const NormArgs p)
             n[i][2 * j + 1] = bits_to_f32<DT>(v[j] >> 16);
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc += OP == OP_RMS ? (double)(n[i][j] * n[i][j]) : (double)n[i][j];
+        for (int j = 0; j < 8; ++j) {
+            const double xd = (double)n[i][j];
+            acc = __builtin_fma(xd, xd, acc);     // the product is exact; one fp64 conversion serves both sums
+            if constexpr (OP != OP_RMS) acc1 += xd;
+        }
     }
     float mul;   // the row's multiplier: 1/rms or rstd
     if constexpr (OP == OP_RMS) {
         const float sum = (float)block_sum(acc, redd);
         mul = 1.0f / sqrtf(sum / (float)p.K + p.eps);
     } else {
-        const float mean = (float)(block_sum(acc, redd) / (double)p.K);
-        double vs = 0.0;
+        block_sum2(acc, acc1, redd);
+        const double m64 = acc1 / (double)p.K;
+        const float mean = (float)m64;
+        const float var = (float)fmax(acc / (double)p.K - m64 * m64, 0.0);
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int idx = threadIdx.x + i * kRowThreads;
+        for (int i = 0; i < NV; ++i)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                n[i][j] = n[i][j] - mean;
-                if (idx < nvec) vs += (double)n[i][j] * (double)n[i][j];
-            }
-        }
-        const float var = (float)(block_sum(vs, redd) / (double)p.K);
+            for (int j = 0; j < 8; ++j) n[i][j] = n[i][j] - mean;
         mul = 1.0f / sqrtf(var + p.eps);
     }
     float mx = 0.f;
@@ -124,27 +126,25 @@ __global__ __launch_bounds__(kRowThreads) void norm_vec_kernel(const NormArgs p)
 // Any K and alignment: the row is re-read for every pass.
 template <int DT, int OP>
 __global__ __launch_bounds__(kRowThreads) void norm_any_kernel(const NormArgs p) {
-    __shared__ double redd[4];
+    __shared__ double redd[8];
     __shared__ float red[4];
     const int64_t row = blockIdx.x;
     const uint16_t* xr = p.x + row * p.ldx;
-    double acc = 0.0;
+    double acc = 0.0, acc1 = 0.0;
     for (int k = threadIdx.x; k < p.K; k += kRowThreads) {
         const float v = bits_to_f32<DT>(xr[k]);
-        acc += OP == OP_RMS ? (double)(v * v) : (double)v;
+        acc += (double)(v * v);
+        acc1 += (double)v;
     }
     float mean = 0.f, mul;
     if constexpr (OP == OP_RMS) {
         const float sum = (float)block_sum(acc, redd);
         mul = 1.0f / sqrtf(sum / (float)p.K + p.eps);
     } else {
-        mean = (float)(block_sum(acc, redd) / (double)p.K);
-        double vs = 0.0;
-        for (int k = threadIdx.x; k < p.K; k += kRowThreads) {
-            const float d = bits_to_f32<DT>(xr[k]) - mean;
-            vs += (double)d * (double)d;
-        }
-        const float var = (float)(block_sum(vs, redd) / (double)p.K);
+        block_sum2(acc, acc1, redd);
+        const double m64 = acc1 / (double)p.K;
+        mean = (float)m64;
+        const float var = (float)fmax(acc / (double)p.K - m64 * m64, 0.0);
         mul = 1.0f / sqrtf(var + p.eps);
     }
     auto value = [&](int k) -> float {

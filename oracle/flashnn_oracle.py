@@ -305,17 +305,20 @@ def rmsnorm(x, gamma, eps: float, dtype: str) -> np.ndarray:
 def layernorm(x, gamma, beta, eps: float, dtype: str) -> np.ndarray:
     """torch.nn.functional.layer_norm over the last dimension (flashnn/norm.py:82-85) for 16-bit
     inputs: moments and the affine map in fp32, one rounding to the input type at the end.
-    mean = sum(x)/K and var = sum((x - mean)^2)/K with the sums taken in float64 and rounded
-    once (x - mean is the fp32 difference); rstd = 1/sqrt(var + eps) with both steps rounded;
-    y = ((x - mean) * rstd) * gamma + beta, every operation rounded to fp32."""
+    mean = sum(x)/K and var = sum(x^2)/K - (sum(x)/K)^2 evaluated in float64 (both sums are exact
+    there for 16-bit inputs, so their order does not matter) and rounded once to fp32;
+    rstd = 1/sqrt(var + eps) with both steps rounded; y = ((x - mean) * rstd) * gamma + beta, every
+    operation rounded to fp32."""
     x = np.asarray(x, dtype=np.float32)
     K = x.shape[-1]
     x2 = x.reshape(-1, K)
     g = np.asarray(gamma, dtype=np.float32).reshape(1, -1)
     b = np.asarray(beta, dtype=np.float32).reshape(1, -1)
-    mean = (x2.astype(np.float64).sum(axis=-1, keepdims=True) / K).astype(np.float32)
+    x64 = x2.astype(np.float64)
+    m64 = x64.sum(axis=-1, keepdims=True) / K
+    mean = m64.astype(np.float32)
+    var = np.maximum((x64 * x64).sum(axis=-1, keepdims=True) / K - m64 * m64, 0.0).astype(np.float32)
     d = x2 - mean
-    var = ((d.astype(np.float64) ** 2).sum(axis=-1, keepdims=True) / K).astype(np.float32)
     rstd = np.float32(1.0) / np.sqrt(var + np.float32(eps))
     y = (d * rstd) * g + b
     return round_to(y.astype(np.float32), dtype).reshape(x.shape)

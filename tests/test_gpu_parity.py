@@ -386,19 +386,13 @@ def test_layernorm_and_dquant_bit_exact(dtype, shape, w_dtype):
     assert out.dtype == dtype and out.shape == x.shape
     want = O.layernorm(O.to_np(x), O.to_np(w), O.to_np(b), 1e-5, _tag(dtype))
     got = out.float().cpu().numpy()
-    # the float64 sums of (x - mean)^2 are not exact, so a different summation order can move a
-    # moment by one fp32 ulp once in a long while; everything else is the same arithmetic
-    assert (got != want).mean() < 1e-4
-    np.testing.assert_allclose(got, want, rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10, atol=1e-6)
+    assert np.array_equal(got, want)     # both moments are exact sums in fp64: same bits
     lq = flashnn_amd.LayernormDquant(K, eps=1e-5)
     lq.weight.data, lq.bias.data = w, b
     q, s = lq.to(DEV)(x.to(DEV))
     assert q.dtype == torch.int8 and q.shape == x.shape and s.dtype == dtype and s.shape == (x.numel() // K, 1)
     q_o, s_o = O.layernorm_dquant(O.to_np(x), O.to_np(w), O.to_np(b), 1e-5, _tag(dtype))
-    if np.array_equal(got, want):
-        assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.float().cpu().numpy(), s_o)
-    else:
-        assert np.abs(q.cpu().numpy().astype(np.int32) - q_o.astype(np.int32)).max() <= 1
+    assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.float().cpu().numpy(), s_o)
 
 
 def test_norm_layers_against_torch_reference_shapes():
