@@ -117,18 +117,20 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         gob[j] = (uint32_t)min(n0 + (j * NWAVES + wave) * 8 + lrow, p.N - 1) * (uint32_t)p.ldb + lchunk * 16;
     // the a-copy of a slab is issued in three parts, one per k-step, so that the copy unit is fed
     // evenly instead of receiving a burst that blocks the wave's issue (and its MFMAs) behind it
-    auto copy_a_part = [&](char* stage, int kt, int part) {
-        const char* slab = (const char*)p.a + (int64_t)kt * BK;
+    // `fix` moves a lane's 16 bytes back to the start of its row piece: the lanes of the last,
+    // partial slab whose chunk lies beyond K fetch bytes that exist (and are never used)
+    auto copy_a_part = [&](char* stage, int kt, int part, int fix = 0) {
+        const char* slab = (const char*)p.a + (int64_t)kt * BK + fix;
 #pragma unroll
         for (int j = 0; j < NLA; ++j)
             if (j * 3 / NLA == part)
                 __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + goa[j]),
                                                  (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
-    auto copy_a = [&](char* stage, int kt) {
-        copy_a_part(stage, kt, 0);
-        copy_a_part(stage, kt, 1);
-        copy_a_part(stage, kt, 2);
+    auto copy_a = [&](char* stage, int kt, int fix = 0) {
+        copy_a_part(stage, kt, 0, fix);
+        copy_a_part(stage, kt, 1, fix);
+        copy_a_part(stage, kt, 2, fix);
     };
     auto copy_b = [&](char* stage, int kt) {
         const char* slab = (const char*)p.b + (int64_t)kt * BK;
@@ -137,8 +139,8 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
                                              (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
-    auto copy_b_part = [&](char* stage, int kt, int part) {
-        const char* slab = (const char*)p.b + (int64_t)kt * BK;
+    auto copy_b_part = [&](char* stage, int kt, int part, int fix = 0) {
+        const char* slab = (const char*)p.b + (int64_t)kt * BK + fix;
 #pragma unroll
         for (int j = 0; j < NLB; ++j)
             if (j * 3 / NLB == part)
@@ -205,7 +207,21 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         asm volatile("" ::: "memory");
     };
 
-    const int KT = p.K / BK;
+    // K = 128 * (KT - 1) + 32 * last_steps: the last slab may hold fewer than four k-steps
+    const int KT = (p.K + BK - 1) / BK;
+    const int last_steps = (p.K - (KT - 1) * BK) / 32;
+    const int tail_fix = lchunk * 16 >= last_steps * 32 ? -(lchunk * 16) : 0;
+    // the slabs 0 .. KT-2 run through the ring; the last one has no successor to prefetch and is
+    // worked off after the loops, from whichever stages it landed in
+    auto last_slab = [&](const char* sa, const char* sb) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            if (ks < last_steps) {
+                if (ks + 1 < last_steps) read_frags(sa, sb, ks + 1);
+                mfmas(ks & 1);
+            }
+        }
+    };
     // One slab = four k-steps; slab j lives in (sa, sb), slab j+1 in (nsa, nsb).  Copies of slab j+2
     // are issued in three parts during k-steps 0..2 into the stage freed at the previous barrier
     // (issued in one burst they block the wave's MFMAs behind them).  The barrier at the start of the
@@ -213,23 +229,21 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     if constexpr (BDEEP) {
         auto wait_barrierB = [&](bool keep) { wait_barrier_n(keep, std::integral_constant<int, NLB>{}); };
         auto slabB = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fb, int j, bool steady) {
+            const bool more = steady || j + 2 < KT;
+            const int fix = !steady && j + 2 == KT - 1 ? tail_fix : 0;
 #pragma unroll
             for (int ks = 0; ks < 3; ++ks) {
                 read_frags(sa, sb, ks + 1);
-                if (steady || j + 2 < KT) copy_b_part(fb, j + 2, ks);
+                if (more) copy_b_part(fb, j + 2, ks, fix);
                 mfmas(ks & 1);
                 interleave();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (steady || j + 1 < KT) {
-                wait_barrierB(steady || j + 2 < KT);
-                read_frags(nsa, nsb, 0);
-                if (steady || j + 2 < KT) copy_a(sa, j + 2);
-                mfmas(1);
-                interleave();
-            } else {
-                mfmas(1);
-            }
+            wait_barrierB(more);
+            read_frags(nsa, nsb, 0);
+            if (more) copy_a(sa, j + 2, fix);
+            mfmas(1);
+            interleave();
             __builtin_amdgcn_sched_barrier(0);
         };
         copy_b(sb0, 0);
@@ -239,7 +253,8 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         read_frags(sa0, sb0, 0);
         copy_a(sa1, 1);
         int j = 0;
-        for (; j + 8 <= KT; j += 6) {
+        // (the steady loop stops one slab earlier when the last slab is partial: its copies need the fix)
+        for (; j + 8 + (last_steps < 4) <= KT; j += 6) {
             slabB(sa0, sb0, sa1, sb1, sb2, j, true);
             slabB(sa1, sb1, sa0, sb2, sb0, j + 1, true);
             slabB(sa0, sb2, sa1, sb0, sb1, j + 2, true);
@@ -247,39 +262,39 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             slabB(sa0, sb1, sa1, sb2, sb0, j + 4, true);
             slabB(sa1, sb2, sa0, sb0, sb1, j + 5, true);
         }
-        for (; j < KT; j += 6) {
+        for (; j < KT - 1; j += 6) {
             slabB(sa0, sb0, sa1, sb1, sb2, j, false);
-            if (j + 1 < KT) slabB(sa1, sb1, sa0, sb2, sb0, j + 1, false);
-            if (j + 2 < KT) slabB(sa0, sb2, sa1, sb0, sb1, j + 2, false);
-            if (j + 3 < KT) slabB(sa1, sb0, sa0, sb1, sb2, j + 3, false);
-            if (j + 4 < KT) slabB(sa0, sb1, sa1, sb2, sb0, j + 4, false);
-            if (j + 5 < KT) slabB(sa1, sb2, sa0, sb0, sb1, j + 5, false);
+            if (j + 2 < KT) slabB(sa1, sb1, sa0, sb2, sb0, j + 1, false);
+            if (j + 3 < KT) slabB(sa0, sb2, sa1, sb0, sb1, j + 2, false);
+            if (j + 4 < KT) slabB(sa1, sb0, sa0, sb1, sb2, j + 3, false);
+            if (j + 5 < KT) slabB(sa0, sb1, sa1, sb2, sb0, j + 4, false);
+            if (j + 6 < KT) slabB(sa1, sb2, sa0, sb0, sb1, j + 5, false);
         }
+        const int lb = (KT - 1) % 3;
+        last_slab((KT - 1) & 1 ? sa1 : sa0, lb == 0 ? sb0 : lb == 1 ? sb1 : sb2);
     } else {
         // three stages each: a(j+2) and b(j+2) are both copied in parts during k-steps 0..2 of slab j,
         // into the stages freed at the previous barrier; at the barrier only they may be in flight
         auto wait_barrier3 = [&](bool keep) { wait_barrier_n(keep, std::integral_constant<int, NLA + NLB>{}); };
         auto slab3 = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fa, char* fb, int j,
                          bool steady) {
+            const bool more = steady || j + 2 < KT;
+            const int fix = !steady && j + 2 == KT - 1 ? tail_fix : 0;
 #pragma unroll
             for (int ks = 0; ks < 3; ++ks) {
                 read_frags(sa, sb, ks + 1);
-                if (steady || j + 2 < KT) {
-                    copy_a_part(fa, j + 2, ks);
-                    copy_b_part(fb, j + 2, ks);
+                if (more) {
+                    copy_a_part(fa, j + 2, ks, fix);
+                    copy_b_part(fb, j + 2, ks, fix);
                 }
                 mfmas(ks & 1);
                 interleave();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (steady || j + 1 < KT) {
-                wait_barrier3(steady || j + 2 < KT);
-                read_frags(nsa, nsb, 0);
-                mfmas(1);
-                interleave();
-            } else {
-                mfmas(1);
-            }
+            wait_barrier3(more);
+            read_frags(nsa, nsb, 0);
+            mfmas(1);
+            interleave();
             __builtin_amdgcn_sched_barrier(0);
         };
         copy_a(sa0, 0);
@@ -289,16 +304,18 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         wait_barrier3(true);
         read_frags(sa0, sb0, 0);
         int j = 0;
-        for (; j + 5 <= KT; j += 3) {
+        for (; j + 5 + (last_steps < 4) <= KT; j += 3) {
             slab3(sa0, sb0, sa1, sb1, sa2, sb2, j, true);
             slab3(sa1, sb1, sa2, sb2, sa0, sb0, j + 1, true);
             slab3(sa2, sb2, sa0, sb0, sa1, sb1, j + 2, true);
         }
-        for (; j < KT; j += 3) {
+        for (; j < KT - 1; j += 3) {
             slab3(sa0, sb0, sa1, sb1, sa2, sb2, j, false);
-            if (j + 1 < KT) slab3(sa1, sb1, sa2, sb2, sa0, sb0, j + 1, false);
-            if (j + 2 < KT) slab3(sa2, sb2, sa0, sb0, sa1, sb1, j + 2, false);
+            if (j + 2 < KT) slab3(sa1, sb1, sa2, sb2, sa0, sb0, j + 1, false);
+            if (j + 3 < KT) slab3(sa2, sb2, sa0, sb0, sa1, sb1, j + 2, false);
         }
+        const int ls = (KT - 1) % 3;
+        last_slab(ls == 0 ? sa0 : ls == 1 ? sa1 : sa2, ls == 0 ? sb0 : ls == 1 ? sb1 : sb2);
     }
 
     // ---- epilogue ----
@@ -476,7 +493,7 @@ static void launch_mfma(A8W8Args& p, hipStream_t st) {
 template <int MODE>
 static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
     // the MFMA kernel walks K in slabs of 128 bytes and addresses rows with 32-bit offsets
-    const bool fast = p.K % 128 == 0 && p.K >= 512 && p.lda % 16 == 0 && p.ldb % 16 == 0 &&
+    const bool fast = p.K % 32 == 0 && p.K >= 512 && p.lda % 16 == 0 && p.ldb % 16 == 0 &&
                       ((uintptr_t)p.a % 16) == 0 && ((uintptr_t)p.b % 16) == 0 &&
                       ((uintptr_t)p.out % 16) == 0 && (int64_t)p.M * p.lda < (1LL << 31) &&
                       (int64_t)p.N * p.ldb < (1LL << 31);

@@ -90,11 +90,25 @@ __device__ __forceinline__ void load_gamma8(const void* gamma, int gamma_dtype, 
     }
 }
 
-// Vector kernels keep a whole row in registers: up to 8 x 8 values per thread, 16-byte aligned rows.
+// Vector kernels keep a whole row in registers: up to kRowMaxNV x 8 values per thread (rows of up
+// to 40960 values), 16-byte aligned rows.
+constexpr int kRowMaxNV = 20;
 inline bool vec_ok(const void* x, const void* q, int64_t K, int64_t ldx, int64_t ldq) {
-    return K % 8 == 0 && K <= 8 * kRowThreads * 8 && ldx % 8 == 0 && ldq % 8 == 0 &&
+    return K % 8 == 0 && K <= 8 * kRowThreads * kRowMaxNV && ldx % 8 == 0 && ldq % 8 == 0 &&
            ((uintptr_t)x % 16) == 0 && ((uintptr_t)q % 8) == 0;
 }
+
+// Launches KERNEL<..., NV, ...> with the smallest NV of the list that holds `nv` vectors per thread.
+#define FNN_ROW_DISPATCH_NV(nv, LAUNCH)                   \
+    do {                                                  \
+        if ((nv) <= 1) { LAUNCH(1); }                     \
+        else if ((nv) <= 2) { LAUNCH(2); }                \
+        else if ((nv) <= 4) { LAUNCH(4); }                \
+        else if ((nv) <= 8) { LAUNCH(8); }                \
+        else if ((nv) <= 12) { LAUNCH(12); }              \
+        else if ((nv) <= 16) { LAUNCH(16); }              \
+        else { LAUNCH(20); }                              \
+    } while (0)
 
 
 }  // namespace fnn

@@ -174,16 +174,15 @@ template <int DT, int OP>
 static void launch_norm(const NormArgs& p, int64_t M, hipStream_t st) {
     const dim3 grid((unsigned)M), block(kRowThreads);
     const int esz = OP == OP_LNQ ? 1 : 2;
-    const bool vec = p.K % 8 == 0 && p.K <= 8 * kRowThreads * 8 && p.ldx % 8 == 0 &&
+    const bool vec = p.K % 8 == 0 && p.K <= 8 * kRowThreads * kRowMaxNV && p.ldx % 8 == 0 &&
                      (p.ldo * esz) % (OP == OP_LNQ ? 8 : 16) == 0 && ((uintptr_t)p.x % 16) == 0 &&
                      ((uintptr_t)p.out % (OP == OP_LNQ ? 8 : 16)) == 0 && ((uintptr_t)p.gamma % 16) == 0 &&
                      (OP == OP_RMS || ((uintptr_t)p.beta % 16) == 0);
     if (vec) {
         const int nv = (p.K / 8 + kRowThreads - 1) / kRowThreads;
-        if (nv <= 1) norm_vec_kernel<DT, 1, OP><<<grid, block, 0, st>>>(p);
-        else if (nv <= 2) norm_vec_kernel<DT, 2, OP><<<grid, block, 0, st>>>(p);
-        else if (nv <= 4) norm_vec_kernel<DT, 4, OP><<<grid, block, 0, st>>>(p);
-        else norm_vec_kernel<DT, 8, OP><<<grid, block, 0, st>>>(p);
+#define FNN_NORM(NV) norm_vec_kernel<DT, NV, OP><<<grid, block, 0, st>>>(p)
+        FNN_ROW_DISPATCH_NV(nv, FNN_NORM);
+#undef FNN_NORM
     } else {
         norm_any_kernel<DT, OP><<<grid, block, 0, st>>>(p);
     }

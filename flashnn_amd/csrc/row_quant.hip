@@ -3,7 +3,7 @@
 // One 256-thread workgroup owns one row.  The row is read from HBM once (16-byte loads)
 // and kept in VGPRs across the reduction(s), so the HBM traffic is the algorithmic
 // 2*K bytes in + K bytes out per row.  Rows that cannot use 16-byte accesses (K not a
-// multiple of 8, unaligned base/stride, or K > 16384) take a strided path that re-reads
+// multiple of 8, unaligned base/stride, or K > 40960) take a strided path that re-reads
 // the row from L2.
 //
 // Arithmetic follows the reference's torch path exactly:
@@ -173,10 +173,9 @@ static void launch_dq(int8_t* q, uint16_t* scale, const uint16_t* x, int64_t M, 
     const dim3 grid((unsigned)M), block(kRowThreads);
     if (vec_ok(x, q, K, ldx, ldq)) {
         const int nv = (K / 8 + kRowThreads - 1) / kRowThreads;
-        if (nv <= 1) dynamic_quant_vec_kernel<DT, 1><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
-        else if (nv <= 2) dynamic_quant_vec_kernel<DT, 2><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
-        else if (nv <= 4) dynamic_quant_vec_kernel<DT, 4><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
-        else dynamic_quant_vec_kernel<DT, 8><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
+#define FNN_DQ(NV) dynamic_quant_vec_kernel<DT, NV><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq)
+        FNN_ROW_DISPATCH_NV(nv, FNN_DQ);
+#undef FNN_DQ
     } else {
         dynamic_quant_any_kernel<DT><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
     }
@@ -188,10 +187,10 @@ static void launch_rq(int8_t* q, uint16_t* scale, const uint16_t* x, const void*
     const dim3 grid((unsigned)M), block(kRowThreads);
     if (vec_ok(x, q, K, ldx, ldq) && ((uintptr_t)gamma % 16) == 0) {
         const int nv = (K / 8 + kRowThreads - 1) / kRowThreads;
-        if (nv <= 1) rmsnorm_dquant_vec_kernel<DT, 1><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
-        else if (nv <= 2) rmsnorm_dquant_vec_kernel<DT, 2><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
-        else if (nv <= 4) rmsnorm_dquant_vec_kernel<DT, 4><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
-        else rmsnorm_dquant_vec_kernel<DT, 8><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
+#define FNN_RQ(NV) \
+    rmsnorm_dquant_vec_kernel<DT, NV><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq)
+        FNN_ROW_DISPATCH_NV(nv, FNN_RQ);
+#undef FNN_RQ
     } else {
         rmsnorm_dquant_any_kernel<DT><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
     }

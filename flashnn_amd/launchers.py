@@ -108,6 +108,8 @@ def hip_layer_norm_dquant_forward(x, weight, bias, eps):
 
 
 def _flat_scale(t, n, what):
+    if t.numel() == n and t.is_contiguous():
+        return t            # [n], [n, 1] and [1, n] share one memory layout: no view needed
     if t.dim() != 1:
         t = torch.squeeze(t)
     if t.dim() == 0:

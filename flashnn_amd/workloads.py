@@ -59,3 +59,23 @@ A8W8_PREFILL_SHAPES = {"qkv": (4096, 12288), "o": (4096, 4096), "gate_up": (4096
                        "down": (11008, 4096)}
 A16W8_DECODE_SHAPES = [(4096, 4096), (4096, 11008), (11008, 4096)]
 A16W4_SHAPE = (8192, 28672)
+
+
+def sharded_model_gemm_shapes():
+    """(N, K) of the four linear layers of the sharded decoder models the reference's A8W8 sweep
+    walks (benchmark/benchmark_gemm_a8w8_amd.py:19-34): FFN up, FFN gate+down input, attention
+    output and QKV projection, for (hidden, intermediate, shards, heads, kv_heads)."""
+    shapes = []
+    for hidden, inter, tp, heads, kv_heads in [(13312, 71168, 8, 104, 8), (13312, 71168, 4, 104, 4),
+                                               (8192, 29568, 4, 64, 8), (8192, 29568, 2, 64, 8),
+                                               (3584, 18944, 1, 28, 4)]:
+        gqa = heads // kv_heads
+        shapes += [(hidden, inter // tp), ((inter // tp) * 2, hidden), (hidden, hidden // tp),
+                   ((hidden // tp) + ((hidden // tp) // gqa) * 2, hidden)]
+    return shapes
+
+
+# activation row counts of both reference sweeps (benchmark_gemm_a8w8_amd.py:42,
+# benchmark_dynamic_quant.py:14) and the row lengths of the dynamic-quant sweep (:10)
+SWEEP_M = [1, 10, 20, 30, 40, 764, 1024, 2048, 4096, 8192]
+DYNAMIC_QUANT_SWEEP_K = [1664, 3328, 8896, 13312, 17792, 35584]

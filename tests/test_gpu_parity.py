@@ -32,7 +32,8 @@ def _tag(dt):
 # ---------------------------------------------------------------------- dynamic quant
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(32, 32), (64, 64), (128, 128), (117, 987), (2560, 8000), (16, 4096),
-                                   (3, 11008), (5, 16384), (2, 35584), (1, 8)])
+                                   (3, 11008), (5, 16384), (2, 35584), (1, 8), (3, 17792), (2, 40960),
+                                   (2, 40968)])
 def test_dynamic_quant_bit_exact(dtype, shape):
     torch.manual_seed(0)
     x = (torch.rand(shape) * 2 - 1).to(dtype) if shape[0] % 2 else torch.randn(shape).to(dtype)
@@ -56,7 +57,8 @@ def test_dynamic_quant_outliers_and_zero_row():
 
 # -------------------------------------------------------------------- rmsnorm + quant
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(4, 128), (3, 32, 1024), (32, 8192), (7, 1000), (2, 20480)])
+@pytest.mark.parametrize("shape", [(4, 128), (3, 32, 1024), (32, 8192), (7, 1000), (2, 20480), (3, 35584),
+                                   (2, 40960), (1, 41000)])
 @pytest.mark.parametrize("gamma_dtype", [torch.float32, None])
 def test_rmsnorm_dquant_bit_exact(dtype, shape, gamma_dtype):
     torch.manual_seed(1)
@@ -89,6 +91,28 @@ def test_a8w8_accumulators_bit_exact(hip_lib, tile, mnk):
     finally:
         hip_lib.fnn_debug_force_a8w8_tile(0, 0)
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
+
+
+@pytest.mark.parametrize("tile", [(0, 0), (256, 192), (256, 128), (128, 128)])
+@pytest.mark.parametrize("mnk", [(300, 200, 544), (257, 385, 576), (64, 320, 608), (130, 100, 1056),
+                                 (10, 1920, 1760), (40, 260, 7392), (520, 390, 8896)])
+def test_a8w8_partial_last_slab_bit_exact(hip_lib, tile, mnk):
+    """K a multiple of 32 but not of 128 (the FFN shapes of models sharded over 4 or 8 GPUs): the
+    last 128-byte slab holds one to three k-steps; few-row problems take the tiled kernel too."""
+    M, N, K = mnk
+    a, b = _rand_i8((M, K), 21), _rand_i8((N, K), 22)
+    assert hip_lib.fnn_debug_force_a8w8_tile(*tile) == 0
+    try:
+        acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+        g = torch.Generator().manual_seed(23)
+        ar = (torch.rand(M, 1, generator=g) * 0.05).half()
+        ac = (torch.rand(1, N, generator=g) * 0.05).half()
+        out = flashnn_amd.GemmA8W8(torch.float16)(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV))
+    finally:
+        hip_lib.fnn_debug_force_a8w8_tile(0, 0)
+    want = O.gemm_a8w8_acc(a.numpy(), b.numpy())
+    assert np.array_equal(acc, want)
+    assert np.array_equal(out.float().cpu().numpy(), O.gemm_a8w8_epilogue_fp32(want, O.to_np(ar), O.to_np(ac), O.F16))
 
 
 @pytest.mark.parametrize("mnk", [(5, 7, 100), (130, 70, 1000), (64, 64, 8), (33, 65, 129)])
@@ -186,6 +210,41 @@ def test_a8w8_prefill_full_size(name):
     out = flashnn_amd.GemmA8W8(torch.bfloat16)(q, wd, s, ws.to(DEV))
     want = O.gemm_a8w8_epilogue_fp32(acc_rows, s_o.astype(np.float32)[rows], ws.numpy(), O.BF16)
     assert np.array_equal(out[torch.from_numpy(rows).to(DEV)].float().cpu().numpy(), want)
+
+
+_SWEEP_B = {}
+
+
+@pytest.mark.parametrize("M", [1, 10, 40, 764, 2048])
+@pytest.mark.parametrize("nk", workloads.sharded_model_gemm_shapes())
+def test_a8w8_reference_sweep_shapes(nk, M):
+    """The (N, K) pairs and row counts of the reference's A8W8 sweep, inputs drawn as its own test
+    draws them (benchmark/benchmark_gemm_a8w8_amd.py:104-124: randint(-12, 12), fp16 scales from
+    rand, fp16 out).  Sampled rows x sampled columns of the result, tile edges included, must equal
+    the oracle bit for bit; a checksum identity covers every accumulator."""
+    N, K = nk
+    g = torch.Generator(device=DEV).manual_seed(N * 31 + K)
+    if nk not in _SWEEP_B:
+        _SWEEP_B.clear()
+        _SWEEP_B[nk] = torch.randint(-12, 12, (N, K), dtype=torch.int8, device=DEV, generator=g)
+    b = _SWEEP_B[nk]
+    g.manual_seed(M * 7 + 1)
+    a = torch.randint(-12, 12, (M, K), dtype=torch.int8, device=DEV, generator=g)
+    ar = torch.rand(M, 1, device=DEV, generator=g).half()
+    ac = torch.rand(1, N, device=DEV, generator=g).half()
+    out = flashnn_amd.GemmA8W8(out_ty=torch.half)(a, b, ar, ac)
+    acc = launchers.hip_gemm_a8w8_int32(a, b)
+    rng = np.random.default_rng(M + N)
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 14)]))
+    cols = np.unique(np.concatenate([[0, N - 1, N - N % 192 - 1], rng.integers(0, N, 125)]))
+    ri, ci = torch.from_numpy(rows).to(DEV), torch.from_numpy(cols).to(DEV)
+    want = O.gemm_a8w8_acc(a[ri].cpu().numpy(), b[ci].cpu().numpy())
+    assert np.array_equal(acc[ri][:, ci].cpu().numpy(), want)
+    want_out = O.gemm_a8w8_epilogue_fp32(want, O.to_np(ar[ri].cpu()), O.to_np(ac[:, ci].cpu()), O.F16)
+    assert np.array_equal(out[ri][:, ci].float().cpu().numpy(), want_out)
+    # sum_n acc[m, n] = a[m, :] . sum_n b[n, :], in exact integers
+    colsum = b.sum(dim=0, dtype=torch.int64)
+    assert torch.equal(acc.sum(dim=1, dtype=torch.int64), (a.to(torch.int64) * colsum).sum(dim=1))
 
 
 # ------------------------------------------------------------------ weight-only GEMM
@@ -355,7 +414,8 @@ def test_rmsnorm_quant_gemm_chain(M):
 
 # ------------------------------------------- rmsnorm, layernorm, layernorm + quant
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(4, 128), (3, 64, 64), (7, 1000), (33, 4096), (16, 8192), (5, 50), (2, 16384), (3, 20000)])
+@pytest.mark.parametrize("shape", [(4, 128), (3, 64, 64), (7, 1000), (33, 4096), (16, 8192), (5, 50), (2, 16384), (3, 20000),
+                                   (2, 35584), (1, 40960)])
 @pytest.mark.parametrize("w_dtype", ["same", torch.float32])
 def test_rmsnorm_bit_exact(dtype, shape, w_dtype):
     g = torch.Generator().manual_seed(21)
@@ -371,7 +431,8 @@ def test_rmsnorm_bit_exact(dtype, shape, w_dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(4, 128), (2, 4, 128), (7, 1000), (33, 4096), (16, 8192), (5, 50), (2, 16384), (3, 20000)])
+@pytest.mark.parametrize("shape", [(4, 128), (2, 4, 128), (7, 1000), (33, 4096), (16, 8192), (5, 50), (2, 16384), (3, 20000),
+                                   (2, 35584), (1, 40960)])
 @pytest.mark.parametrize("w_dtype", ["same", torch.float32])
 def test_layernorm_and_dquant_bit_exact(dtype, shape, w_dtype):
     g = torch.Generator().manual_seed(22)
