@@ -178,7 +178,13 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
     const int m_base = pass * (MB * 16);
     const int row0 = (tile * RT + rt) * 16;
 
-    const int KT = p.K / 128;
+    // K = 128 * (KT - 1) + tail.  The last slab may be partial (tail = 32, 64 or 96 bytes): the lanes
+    // whose 16-byte chunk lies beyond K fetch the first chunk of their row piece instead (bytes that
+    // exist), and the weights of those chunks are replaced by zeros before they reach the MFMAs, so
+    // whatever the activation copies fetched there is multiplied by zero.
+    const int KT = (p.K + 127) / 128;
+    const int tail = p.K - (KT - 1) * 128;
+    const bool part_tail = tail < 128 && ks == KS - 1;   // wave-uniform: this K part ends in the partial slab
     const int sl0 = KT * ks / KS;
     const int nsl = KT * (ks + 1) / KS - sl0;
     const int n_iter = ((KT + KS - 1) / KS + 3) / 4 * 4;
@@ -186,8 +192,12 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
     const int r8 = lane >> 3, c8 = lane & 7;
     const char* wptr = (const char*)p.b + (int64_t)(row0 + r8) * p.ldb + c8 * 16 + (int64_t)sl0 * 128;
     const int64_t w_half = 8 * p.ldb;
+    const bool wzero = c8 * 16 >= tail;
+    const int wfix = wzero ? -(c8 * 16) : 0;
     auto load_w = [&](int jj, int half) -> v4i {
-        return *(const v4i*)(wptr + (int64_t)min(jj, nsl - 1) * 128 + half * w_half);
+        const int s = min(jj, nsl - 1);
+        const int fix = part_tail && s == nsl - 1 ? wfix : 0;
+        return *(const v4i*)(wptr + (int64_t)s * 128 + half * w_half + fix);
     };
     char* const wmine = wst + wave * 2048;
     int wwr[2], wrd[2];
@@ -201,17 +211,21 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
     const int t = rt * 64 + lane;
     const char* act_part = (const char*)p.a + (int64_t)sl0 * 128;
     int64_t goff[NCP];
+    int afix[NCP];
 #pragma unroll
     for (int i = 0; i < NCP; ++i) {
         const int row = i * (8 * RT) + (t >> 3);
         const int chunk = (t & 7) ^ ((row >> 1) & 7);
         goff[i] = (int64_t)min(m_base + row, p.M - 1) * p.lda + chunk * 16;
+        afix[i] = chunk * 16 >= tail ? -(chunk * 16) : 0;
     }
     auto copy_act = [&](char* stage, int jj) {
-        const char* src = act_part + (int64_t)min(jj, nsl - 1) * 128;
+        const int s = min(jj, nsl - 1);
+        const char* src = act_part + (int64_t)s * 128;
+        const bool last = part_tail && s == nsl - 1;
 #pragma unroll
         for (int i = 0; i < NCP; ++i)
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + goff[i]),
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + goff[i] + (last ? afix[i] : 0)),
                                              (lds_ptr_t)(stage + ks * SLAB + (i * RT * 64 + rt * 64) * 16), 16, 0, 0);
     };
     int rd[2];
@@ -239,8 +253,9 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
         copy_act(FREE, (JJ) + 3);                                                       \
         const bool mine_ = (JJ) < nsl;   /* wave-uniform */                             \
         if (mine_) {                                                                    \
-            *(v4i*)(wmine + wwr[0]) = wq[W][0];                                         \
-            *(v4i*)(wmine + wwr[1]) = wq[W][1];                                         \
+            const bool z_ = part_tail && (JJ) == nsl - 1 && wzero;                      \
+            *(v4i*)(wmine + wwr[0]) = z_ ? v4i{0, 0, 0, 0} : wq[W][0];                  \
+            *(v4i*)(wmine + wwr[1]) = z_ ? v4i{0, 0, 0, 0} : wq[W][1];                  \
         }                                                                               \
         wq[W][0] = load_w((JJ) + 4, 0);                                                 \
         wq[W][1] = load_w((JJ) + 4, 1);                                                 \
@@ -342,7 +357,7 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
 
 template <int MODE>
 static bool launch_a8_panel_t(A8W8Args& p, hipStream_t st) {
-    if (p.M > 64 || p.N % 16 != 0 || p.K % 128 != 0 || p.K < 8 * 128 || p.lda % 16 != 0 || p.ldb % 16 != 0 ||
+    if (p.M > 64 || p.N % 16 != 0 || p.K % 32 != 0 || p.K < 8 * 128 || p.lda % 16 != 0 || p.ldb % 16 != 0 ||
         ((uintptr_t)p.a % 16) != 0 || ((uintptr_t)p.b % 16) != 0)
         return false;
     // rows per workgroup by chip fill, as in the weight-only panel kernel
@@ -375,7 +390,8 @@ static bool launch_a8_panel_t(A8W8Args& p, hipStream_t st) {
 template <int MODE>
 static bool launch_skinny_t(A8W8Args& p, hipStream_t st) {
     // a single activation row gains nothing from shared slabs (measured 14.0 against 16.5 us at K = N = 8192)
-    if (p.M > 1 && launch_a8_panel_t<MODE>(p, st)) return true;
+    // (it takes the shared-slab kernel all the same when K is no multiple of 128, which only that one handles)
+    if ((p.M > 1 || p.K % 128 != 0) && launch_a8_panel_t<MODE>(p, st)) return true;
     if (p.M > 64 || p.K % 128 != 0 || p.lda % 16 != 0 || p.ldb % 16 != 0 ||
         ((uintptr_t)p.a % 16) != 0 || ((uintptr_t)p.b % 16) != 0)
         return false;

@@ -126,7 +126,9 @@ def test_a8w8_guarded_kernel_bit_exact(mnk):
 @pytest.mark.parametrize("M", [1, 7, 16, 17, 33, 48, 64])
 @pytest.mark.parametrize("nk", [(1000, 64), (16, 448), (4100, 4096), (520, 8192),
                                 # shared activation slabs: 16-, 32- and 64-row workgroups, uneven K parts
-                                (4096, 4096), (8192, 1152), (16384, 1024), (2048, 11008)])
+                                (4096, 4096), (8192, 1152), (16384, 1024), (2048, 11008),
+                                # K a multiple of 32 only: the last slab holds 32, 64 or 96 bytes
+                                (4096, 1056), (8192, 7392), (2048, 8896), (1920, 1120), (16, 1088)])
 def test_a8w8_few_rows_bit_exact(M, nk):
     """Up to 64 activation rows take the weight-streaming kernel: accumulators and scaled outputs,
     N not a multiple of the 16-row tile, fewer k-steps than waves."""
