@@ -127,6 +127,18 @@ def main():
     roofline = {"kernel": "gemm_a8w8_ring_kernel", "bound": "mfma", "achieved": round(gemm_tops, 2),
                 "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
                 "us_per_launch": round(ms_gemm * 1e3, 2), "traffic": _traffic("gemm_a8w8_ring_kernel")}
+    # what this device sustains on int8 MFMAs alone (operands in registers, about 0.1 s each): the
+    # clock follows the power drawn, so random operand bytes run well below the datasheet rate
+    import ctypes
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    sustained = {}
+    for label, rnd in (("random_operand_bytes", 1), ("constant_operands", 0)):
+        rate = ctypes.c_double(0.0)
+        _lib.check(_lib.load().fnn_debug_mfma_rate(_lib.ptr(sink), rnd, 20000, 40, ctypes.byref(rate),
+                                                   _lib.current_stream(torch.device(dev))))
+        sustained[label] = round(rate.value, 1)
+    roofline["mfma_only_sustained"] = dict(sustained, unit="TOP/s")
+    roofline["frac_of_sustained_random"] = round(gemm_tops / sustained["random_operand_bytes"], 4)
     secondary = []
     qbytes = 3.0 * M * K + 2.0 * M
     secondary.append({"workload": f"dynamic_quant fp16 M={M} K={K}", "kernel": "dynamic_quant_vec_kernel",

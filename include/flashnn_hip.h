@@ -153,6 +153,18 @@ int fnn_layernorm_dquant(void* q, void* scale, const void* x, const void* gamma,
  */
 int fnn_debug_force_a8w8_tile(int bm, int bn);
 
+/*
+ * Measurement aid, no counterpart in the reference: the rate, in 1e12 int8 operations per second,
+ * at which the current device sustains back-to-back 32x32x32 int8 MFMAs with operands held in
+ * registers (two waves per SIMD, no memory traffic).  random_operands != 0 feeds the matrix cores
+ * random bytes, as a GEMM on quantised data does; 0 feeds constants.  The clock follows the power
+ * drawn, and that follows the toggling of the operand bits, so the two rates differ; the first is the
+ * ceiling an A8W8 GEMM can approach on this device.  Runs 1 + launches kernels of `iters` loop
+ * iterations on `stream` and waits for them.  sink: 4 bytes of device memory (never written).
+ */
+int fnn_debug_mfma_rate(void* sink, int random_operands, int iters, int launches, double* tops,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif
