@@ -570,3 +570,47 @@ extern "C" int fnn_gemm_a8w8_i32(int32_t* acc, const void* a, const void* b, int
     dispatch<OUT_I32>(p, (hipStream_t)stream, g_force_bm, g_force_bn);
     return check_launch("fnn_gemm_a8w8_i32");
 }
+
+extern "C" int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const void* alpha_row,
+                                  const void* alpha_col, const void* topk_weights,
+                                  const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                  const int32_t* num_tokens_post_padded, int64_t N, int64_t K, int64_t EM,
+                                  int64_t num_valid_tokens, int64_t lda, int64_t stride_be, int64_t ldb,
+                                  int64_t ldc, int64_t stride_scale_be, int mul_routed_weight, int top_k,
+                                  int block_m, int out_dtype, int alpha_row_dtype, int alpha_col_dtype,
+                                  int topk_weights_dtype, void* stream) {
+    using namespace fnn;
+    const char* fn = "fnn_fused_moe_a8w8";
+    if (!c || !a || !b || !alpha_row || !alpha_col || !sorted_token_ids || !expert_ids || !num_tokens_post_padded ||
+        (mul_routed_weight && !topk_weights)) {
+        set_error("%s: null pointer argument", fn);
+        return FNN_ERR_ARG;
+    }
+    if (N < 0 || K <= 0 || EM < 0 || num_valid_tokens < 0 || top_k <= 0 || block_m <= 0 || lda < K || ldb < K ||
+        ldc < N || stride_be < 0 || stride_scale_be < 0) {
+        set_error("%s: bad shape N=%lld K=%lld EM=%lld tokens=%lld top_k=%d block_m=%d", fn, (long long)N,
+                  (long long)K, (long long)EM, (long long)num_valid_tokens, top_k, block_m);
+        return FNN_ERR_ARG;
+    }
+    if (N > 0x7FFFFFFFLL || K > 0x7FFFFFFFLL || EM > 0x7FFFFFFFLL || num_valid_tokens > 0x7FFFFFFFLL) {
+        set_error("%s: shape too large", fn);
+        return FNN_ERR_UNSUPPORTED;
+    }
+    if (!is16(out_dtype)) { set_error("%s: Output type must be float16 or bfloat16", fn); return FNN_ERR_UNSUPPORTED; }
+    if (!isflt(alpha_row_dtype) || !isflt(alpha_col_dtype) || (mul_routed_weight && !isflt(topk_weights_dtype))) {
+        set_error("%s: bad scale type", fn);
+        return FNN_ERR_UNSUPPORTED;
+    }
+    if (N == 0 || EM == 0 || num_valid_tokens == 0) return FNN_OK;
+    A8W8Args p{};
+    p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = c; p.arow = alpha_row; p.acol = alpha_col;
+    p.M = (int)EM; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    p.out_dtype = out_dtype; p.arow_dtype = alpha_row_dtype; p.acol_dtype = alpha_col_dtype;
+    MoeArgs q{};
+    q.sorted_ids = sorted_token_ids; q.expert_ids = expert_ids; q.ntpp = num_tokens_post_padded;
+    q.topk_w = topk_weights; q.topk_w_dtype = topk_weights_dtype; q.mul_w = mul_routed_weight ? 1 : 0;
+    q.top_k = top_k; q.block_m = block_m; q.num_valid = (int)num_valid_tokens; q.EM = (int)EM;
+    q.stride_be = stride_be; q.stride_scale_be = stride_scale_be;
+    launch_a8w8_moe(p, q, out_dtype == FNN_F16 ? OUT_F16 : OUT_BF16, (hipStream_t)stream);
+    return check_launch(fn);
+}

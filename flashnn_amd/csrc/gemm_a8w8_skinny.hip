@@ -148,8 +148,8 @@ __global__ __launch_bounds__(kSkWaves * 64) void gemm_a8w8_skinny_kernel(const A
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
-template <int MB, int RT, int MODE>
-__global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, const int passes) {
+template <int MB, int RT, int MODE, bool MOE = false>
+__global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, const int passes, const MoeArgs q) {
     constexpr int KS = 8 / RT;
     constexpr int SLAB = MB * 16 * 128;
     constexpr int STG = KS * SLAB;
@@ -177,6 +177,18 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
     if (tile >= tiles) return;
     const int m_base = pass * (MB * 16);
     const int row0 = (tile * RT + rt) * 16;
+    // mixture of experts: the pass covers sorted rows m_base .. of one expert; passes beyond the rows
+    // in use have nothing to do
+    int expert = 0;
+    if constexpr (MOE) {
+        if (m_base >= q.ntpp[0]) return;
+        expert = q.expert_ids[m_base / q.block_m];
+    }
+    // activation row and validity of local row r of this pass
+    auto token_of = [&](int r) -> int {
+        const int sidx = m_base + r;
+        return sidx < q.EM ? q.sorted_ids[sidx] : q.num_valid;
+    };
 
     // K = 128 * (KT - 1) + tail.  The last slab may be partial (tail = 32, 64 or 96 bytes): the lanes
     // whose 16-byte chunk lies beyond K fetch the first chunk of their row piece instead (bytes that
@@ -190,7 +202,8 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
     const int n_iter = ((KT + KS - 1) / KS + 3) / 4 * 4;
 
     const int r8 = lane >> 3, c8 = lane & 7;
-    const char* wptr = (const char*)p.b + (int64_t)(row0 + r8) * p.ldb + c8 * 16 + (int64_t)sl0 * 128;
+    const char* wptr = (const char*)p.b + (MOE ? (int64_t)expert * q.stride_be : 0) + (int64_t)(row0 + r8) * p.ldb +
+                       c8 * 16 + (int64_t)sl0 * 128;
     const int64_t w_half = 8 * p.ldb;
     const bool wzero = c8 * 16 >= tail;
     const int wfix = wzero ? -(c8 * 16) : 0;
@@ -216,7 +229,12 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
     for (int i = 0; i < NCP; ++i) {
         const int row = i * (8 * RT) + (t >> 3);
         const int chunk = (t & 7) ^ ((row >> 1) & 7);
-        goff[i] = (int64_t)min(m_base + row, p.M - 1) * p.lda + chunk * 16;
+        if constexpr (MOE) {
+            const int tok = token_of(row);
+            goff[i] = (int64_t)(tok < q.num_valid ? tok / q.top_k : 0) * p.lda + chunk * 16;
+        } else {
+            goff[i] = (int64_t)min(m_base + row, p.M - 1) * p.lda + chunk * 16;
+        }
         afix[i] = chunk * 16 >= tail ? -(chunk * 16) : 0;
     }
     auto copy_act = [&](char* stage, int jj) {
@@ -323,12 +341,22 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
     float ac[4];
     if constexpr (MODE != OUT_I32) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) ac[r] = load_as_f32(p.acol, n0 + r, p.acol_dtype);
+        for (int r = 0; r < 4; ++r)
+            ac[r] = load_as_f32(p.acol, (MOE ? (int64_t)expert * q.stride_scale_be : 0) + n0 + r, p.acol_dtype);
     }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-        const int m = m_base + mb * 16 + li;
-        if (m >= p.M) continue;
+        int m = m_base + mb * 16 + li;     // output row; for gathered rows the token id
+        int arow_idx = m;
+        float wroute = 1.f;
+        if constexpr (MOE) {
+            m = token_of(mb * 16 + li);
+            if (m >= q.num_valid) continue;
+            arow_idx = m / q.top_k;
+            if (q.mul_w) wroute = load_as_f32(q.topk_w, m, q.topk_w_dtype);
+        } else {
+            if (m >= p.M) continue;
+        }
         if constexpr (MODE == OUT_I32) {
             int32_t* dst = (int32_t*)p.out + (int64_t)m * p.ldc + n0;
             if ((p.ldc & 3) == 0 && ((uintptr_t)p.out & 15) == 0) *(v4i*)dst = acc[mb];
@@ -337,11 +365,14 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
                 for (int r = 0; r < 4; ++r) dst[r] = acc[mb][r];
             }
         } else {
-            const float ar = load_as_f32(p.arow, m, p.arow_dtype);
+            const float ar = load_as_f32(p.arow, arow_idx, p.arow_dtype);
             uint32_t h[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float f = rounded_f32(((float)acc[mb][r] * ar) * ac[r]);
+                float f = rounded_f32(((float)acc[mb][r] * ar) * ac[r]);
+                if constexpr (MOE) {
+                    if (q.mul_w) f = rounded_f32(f * wroute);
+                }
                 h[r] = MODE == OUT_F16 ? f32_to_f16_bits(f) : f32_to_bf16_bits(f);
             }
             uint16_t* dst = (uint16_t*)p.out + (int64_t)m * p.ldc + n0;
@@ -376,13 +407,13 @@ static bool launch_a8_panel_t(A8W8Args& p, hipStream_t st) {
     const int tiles = p.N / (16 * rt);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes), block(512);
     if (rt == 4) {
-        if (mb == 2) gemm_a8w8_panel_kernel<2, 4, MODE><<<grid, block, 0, st>>>(p, passes);
-        else gemm_a8w8_panel_kernel<4, 4, MODE><<<grid, block, 0, st>>>(p, passes);
+        if (mb == 2) gemm_a8w8_panel_kernel<2, 4, MODE><<<grid, block, 0, st>>>(p, passes, MoeArgs{});
+        else gemm_a8w8_panel_kernel<4, 4, MODE><<<grid, block, 0, st>>>(p, passes, MoeArgs{});
     } else if (rt == 2) {
-        if (mb == 1) gemm_a8w8_panel_kernel<1, 2, MODE><<<grid, block, 0, st>>>(p, passes);
-        else gemm_a8w8_panel_kernel<2, 2, MODE><<<grid, block, 0, st>>>(p, passes);
+        if (mb == 1) gemm_a8w8_panel_kernel<1, 2, MODE><<<grid, block, 0, st>>>(p, passes, MoeArgs{});
+        else gemm_a8w8_panel_kernel<2, 2, MODE><<<grid, block, 0, st>>>(p, passes, MoeArgs{});
     } else {
-        gemm_a8w8_panel_kernel<1, 1, MODE><<<grid, block, 0, st>>>(p, passes);
+        gemm_a8w8_panel_kernel<1, 1, MODE><<<grid, block, 0, st>>>(p, passes, MoeArgs{});
     }
     return true;
 }
@@ -401,6 +432,72 @@ static bool launch_skinny_t(A8W8Args& p, hipStream_t st) {
     else if (p.M <= 48) gemm_a8w8_skinny_kernel<3, MODE><<<grid, block, 0, st>>>(p);
     else gemm_a8w8_skinny_kernel<4, MODE><<<grid, block, 0, st>>>(p);
     return true;
+}
+
+// ------------------------------------------------------------------ mixture of experts
+// Any shape: one thread per output value, the row dotted byte by byte (4 at a time where aligned).
+template <int MODE>
+__global__ __launch_bounds__(256) void moe_a8w8_any_kernel(const A8W8Args p, const MoeArgs q) {
+    const int sidx = blockIdx.x;
+    if (sidx >= q.ntpp[0]) return;
+    const int tok = q.sorted_ids[sidx];
+    if (tok >= q.num_valid) return;
+    const int n = blockIdx.y * 256 + threadIdx.x;
+    if (n >= p.N) return;
+    const int expert = q.expert_ids[sidx / q.block_m];
+    const int8_t* a = p.a + (int64_t)(tok / q.top_k) * p.lda;
+    const int8_t* b = p.b + (int64_t)expert * q.stride_be + (int64_t)n * p.ldb;
+    int acc = 0;
+    int k = 0;
+    if ((((uintptr_t)a | (uintptr_t)b) & 3) == 0)
+        for (; k + 4 <= p.K; k += 4) acc = __builtin_amdgcn_sdot4(*(const int*)(a + k), *(const int*)(b + k), acc, false);
+    for (; k < p.K; ++k) acc += (int)a[k] * (int)b[k];
+    const float ar = load_as_f32(p.arow, tok / q.top_k, p.arow_dtype);
+    const float ac = load_as_f32(p.acol, (int64_t)expert * q.stride_scale_be + n, p.acol_dtype);
+    float f = rounded_f32(((float)acc * ar) * ac);
+    if (q.mul_w) f = rounded_f32(f * load_as_f32(q.topk_w, tok, q.topk_w_dtype));
+    ((uint16_t*)p.out)[(int64_t)tok * p.ldc + n] = (uint16_t)(MODE == OUT_F16 ? f32_to_f16_bits(f) : f32_to_bf16_bits(f));
+}
+
+template <int MODE>
+static bool launch_moe_t(A8W8Args& p, const MoeArgs& q, hipStream_t st) {
+    const bool fast = p.N % 16 == 0 && p.K % 32 == 0 && p.K >= 8 * 128 && p.lda % 16 == 0 && p.ldb % 16 == 0 &&
+                      q.stride_be % 16 == 0 && ((uintptr_t)p.a % 16) == 0 && ((uintptr_t)p.b % 16) == 0 &&
+                      q.block_m % 16 == 0 && q.EM % q.block_m == 0;
+    if (!fast) {
+        moe_a8w8_any_kernel<MODE><<<dim3(q.EM, (p.N + 255) / 256), dim3(256), 0, st>>>(p, q);
+        return true;
+    }
+    // a pass must stay within one expert's block: 16 * MB rows divide block_m
+    const int mb_max = q.block_m % 64 == 0 ? 4 : q.block_m % 32 == 0 ? 2 : 1;
+    int rt = 0;
+    double best = 0.0;
+    for (int cand = 4; cand >= 1; cand >>= 1) {
+        if (p.N % (16 * cand) != 0) continue;
+        if (cand == 4 && mb_max < 2) continue;          // RT = 4 shares slabs of at least 32 rows
+        const int t = p.N / (16 * cand);
+        const double fill = (double)t / (((t + 255) / 256) * 256);
+        const double score = fill * (cand == 4 ? 1.0 : cand == 2 ? 0.9 : 0.6);
+        if (score > best) { best = score; rt = cand; }
+    }
+    const int mb = rt == 4 ? (mb_max >= 4 ? 4 : 2) : rt == 2 ? (mb_max >= 2 ? 2 : 1) : 1;
+    const int passes = q.EM / (mb * 16);
+    const int tiles = p.N / (16 * rt);
+    const dim3 grid(((tiles + 7) / 8) * 8 * passes), block(512);
+    if (rt == 4) {
+        if (mb == 2) gemm_a8w8_panel_kernel<2, 4, MODE, true><<<grid, block, 0, st>>>(p, passes, q);
+        else gemm_a8w8_panel_kernel<4, 4, MODE, true><<<grid, block, 0, st>>>(p, passes, q);
+    } else if (rt == 2) {
+        if (mb == 1) gemm_a8w8_panel_kernel<1, 2, MODE, true><<<grid, block, 0, st>>>(p, passes, q);
+        else gemm_a8w8_panel_kernel<2, 2, MODE, true><<<grid, block, 0, st>>>(p, passes, q);
+    } else {
+        gemm_a8w8_panel_kernel<1, 1, MODE, true><<<grid, block, 0, st>>>(p, passes, q);
+    }
+    return true;
+}
+
+bool launch_a8w8_moe(A8W8Args& p, const MoeArgs& q, int mode, hipStream_t st) {
+    return mode == OUT_F16 ? launch_moe_t<OUT_F16>(p, q, st) : launch_moe_t<OUT_BF16>(p, q, st);
 }
 
 bool launch_a8w8_skinny(A8W8Args& p, int mode, hipStream_t st) {

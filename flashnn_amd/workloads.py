@@ -79,3 +79,30 @@ def sharded_model_gemm_shapes():
 # benchmark_dynamic_quant.py:14) and the row lengths of the dynamic-quant sweep (:10)
 SWEEP_M = [1, 10, 20, 30, 40, 764, 1024, 2048, 4096, 8192]
 DYNAMIC_QUANT_SWEEP_K = [1664, 3328, 8896, 13312, 17792, 35584]
+
+
+def moe_align_block_size(topk_ids, block_size, num_experts):
+    """Groups the routed rows by expert the way callers of fused_moe_*_forward prepare them (the
+    reference ships no such helper; its launcher's docstring describes the layout,
+    flashnn/triton_kernels/fused_moe_a8w8.py:203-207): returns int32 tensors
+    (sorted_token_ids [numel + num_experts*(block_size-1)], expert_ids [len(sorted)/block_size],
+    num_tokens_post_padded [1]).  Routed row i = position in topk_ids.flatten(); each expert's rows are
+    listed in ascending order and padded with numel to a multiple of block_size; the unused tail of
+    sorted_token_ids holds numel and the unused tail of expert_ids holds 0."""
+    flat = topk_ids.flatten().to(torch.int64)
+    numel = flat.numel()
+    cap = numel + num_experts * (block_size - 1)
+    cap = (cap + block_size - 1) // block_size * block_size
+    sorted_ids = torch.full((cap,), numel, dtype=torch.int32)
+    expert_ids = torch.zeros(cap // block_size, dtype=torch.int32)
+    pos = 0
+    for e in range(num_experts):
+        rows = torch.nonzero(flat == e).flatten()
+        n = rows.numel()
+        if n == 0:
+            continue
+        sorted_ids[pos:pos + n] = rows.to(torch.int32)
+        padded = (n + block_size - 1) // block_size * block_size
+        expert_ids[pos // block_size:(pos + padded) // block_size] = e
+        pos += padded
+    return sorted_ids, expert_ids, torch.tensor([pos], dtype=torch.int32)

@@ -147,6 +147,33 @@ int fnn_layernorm_dquant(void* q, void* scale, const void* x, const void* gamma,
                          int gb_dtype, void* stream);
 
 /*
+ * Replaces fused_moe_a8w8_forward(A, B, C, alpha_row_ptr, alpha_col_ptr, topk_weights, topk_ids,
+ * sorted_token_ids, expert_ids, num_tokens_post_padded, mul_routed_weight, top_k, BM)
+ * (flashnn/triton_kernels/fused_moe_a8w8.py:176-290; kernel :37-173), exported as
+ * flashnn.fused_moe_a8w8_forward (flashnn/__init__.py:14).
+ *
+ * a: int8 [M,K] tokens (row stride lda); b: int8 [E,N,K] expert weights (stride_be between experts, ldb
+ * between rows); c: fp16/bf16, addressed as [M*top_k, N] rows with row stride ldc (the reference's
+ * C[M, top_k, N] with ldc = C.stride(1)).  Sorted row i (i < *num_tokens_post_padded, a multiple of
+ * block_m) names the routed row t = sorted_token_ids[i]; t >= num_valid_tokens (= M*top_k) is padding.
+ * Every block of block_m sorted rows belongs to the expert expert_ids[i / block_m].  For valid rows
+ *   c[t, n] = (fp32(sum_k a[t / top_k, k] * b[e, n, k]) * alpha_row[t / top_k]) * alpha_col[e*stride_scale_be + n]
+ * times topk_weights[t] when mul_routed_weight != 0; every product rounded to fp32, the result rounded
+ * once to out_dtype (the reference always rounds to fp16, :162).  Rows of c that no valid sorted row names
+ * are left untouched.  sorted_token_ids [EM], expert_ids and num_tokens_post_padded [1] are int32 device
+ * arrays.  The weight-streaming kernel takes N % 16 == 0, K % 32 == 0, K >= 1024, block_m % 16 == 0,
+ * EM % block_m == 0 and 16-byte aligned rows; anything else takes a slow guarded kernel.
+ */
+int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const void* alpha_row,
+                       const void* alpha_col, const void* topk_weights,
+                       const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                       const int32_t* num_tokens_post_padded, int64_t N, int64_t K, int64_t EM,
+                       int64_t num_valid_tokens, int64_t lda, int64_t stride_be, int64_t ldb,
+                       int64_t ldc, int64_t stride_scale_be, int mul_routed_weight, int top_k,
+                       int block_m, int out_dtype, int alpha_row_dtype, int alpha_col_dtype,
+                       int topk_weights_dtype, void* stream);
+
+/*
  * Test hook, no counterpart in the reference: force the output tile (bm x bn) of the MFMA
  * A8W8 kernel for subsequent calls, so that every tile shape can be checked on small
  * problems; (0, 0) restores the automatic choice.  Valid tiles: 256x192, 256x128, 128x128.  Process-wide and not synchronised: for tests only.

@@ -165,6 +165,45 @@ def gemm_a8w8_epilogue_fp32(acc, alpha_row, alpha_col, out_dtype: str) -> np.nda
     return round_to((x * ar) * ac, out_dtype)
 
 
+def fused_moe_a8w8(a, b, c, alpha_row, alpha_col, topk_weights, sorted_token_ids, expert_ids,
+                   num_tokens_post_padded, mul_routed_weight: bool, top_k: int, block_m: int, out_dtype: str):
+    """Mixture-of-experts A8W8 GEMM, flashnn/triton_kernels/fused_moe_a8w8.py:74-173, block by block as
+    the kernel walks them: sorted rows [i*block_m, (i+1)*block_m) below num_tokens_post_padded (:94-96)
+    use expert expert_ids[i] (:107); routed row t = sorted_token_ids[..] is valid if t < M*top_k (:98);
+    its token is a[t // top_k] (:102-104); acc is the int32 contraction with b[e] (:118-144); then
+    fp32(acc) * alpha_row[t // top_k], * alpha_col[e, n] (:150-157), * topk_weights[t] if asked (:159-161),
+    each product rounded to fp32, one rounding to the output type (:163, fp16 in the reference), stored
+    at c[t] (:166-168).  `c` ([M*top_k, N] float32 holding out_dtype values) is updated in place and
+    returned: rows no valid sorted row names keep what they held.
+
+    The reference has no test or torch path for this function.  Pinned by: a per-element Python loop on
+    tiny inputs, the reduction to gemm_a8w8_epilogue_fp32 when every row goes to one expert, and
+    invariance under permutations of the sorted list within an expert (tests/test_oracle.py)."""
+    a = np.asarray(a)
+    b = np.asarray(b)
+    ar = np.asarray(alpha_row, dtype=np.float32).reshape(-1)
+    ac = np.asarray(alpha_col, dtype=np.float32).reshape(b.shape[0], b.shape[1])
+    w = None if topk_weights is None else np.asarray(topk_weights, dtype=np.float32).reshape(-1)
+    sorted_token_ids = np.asarray(sorted_token_ids).reshape(-1)
+    num_valid = c.shape[0]
+    used = int(np.asarray(num_tokens_post_padded).reshape(-1)[0])
+    for blk in range((len(sorted_token_ids) + block_m - 1) // block_m):
+        if blk * block_m >= used:
+            break
+        e = int(np.asarray(expert_ids).reshape(-1)[blk])
+        toks = sorted_token_ids[blk * block_m:(blk + 1) * block_m]
+        toks = toks[toks < num_valid].astype(np.int64)
+        if toks.size == 0:
+            continue
+        acc = gemm_a8w8_acc(a[toks // top_k], b[e]).astype(np.float32)
+        x = (acc * ar[toks // top_k].reshape(-1, 1)).astype(np.float32)
+        x = (x * ac[e].reshape(1, -1)).astype(np.float32)
+        if mul_routed_weight:
+            x = (x * w[toks].reshape(-1, 1)).astype(np.float32)
+        c[toks] = round_to(x, out_dtype)
+    return c
+
+
 # ------------------------------------------------------------------ weight-only GEMM
 def unpack_int4(qw: np.ndarray) -> np.ndarray:
     """[N/2,K] packed bytes -> [N,K] int8 in [-8,7].

@@ -249,6 +249,42 @@ def test_a8w8_reference_sweep_shapes(nk, M):
     assert torch.equal(acc.sum(dim=1, dtype=torch.int64), (a.to(torch.int64) * colsum).sum(dim=1))
 
 
+# ------------------------------------------------------------------ mixture of experts
+@pytest.mark.parametrize("out_ty", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mul_w", [False, True])
+@pytest.mark.parametrize("shape", [
+    # M, E, N, K, top_k, BM
+    (16, 8, 1024, 1024, 2, 16), (33, 8, 4096, 2048, 2, 32), (64, 4, 2064, 1056, 1, 64), (200, 8, 512, 1120, 2, 128),
+    (7, 16, 1040, 4096, 4, 16), (3, 60, 256, 1024, 6, 16),
+    # shapes of the guarded kernel: short K, block size not a multiple of 16
+    (9, 4, 48, 80, 2, 16), (20, 3, 64, 1024, 2, 8)])
+def test_fused_moe_a8w8_bit_exact(shape, mul_w, out_ty):
+    """fused_moe_a8w8_forward against the oracle: every routed row, bit for bit; rows that the sorted
+    list does not name keep the value they held."""
+    M, E, N, K, top_k, BM = shape
+    g = torch.Generator().manual_seed(M * 131 + E)
+    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g)
+    b = torch.randint(-128, 128, (E, N, K), dtype=torch.int8, generator=g)
+    ar = (torch.rand(M, generator=g) * 0.05).to(out_ty)
+    ac = (torch.rand(E, N, generator=g) * 0.05).float()
+    w, ids = torch.topk(torch.softmax(torch.randn(M, E, generator=g), -1), top_k, dim=-1)
+    w = w.float().contiguous()
+    s, e, used = workloads.moe_align_block_size(ids, BM, E)
+    for cut in (False, True):
+        if cut:                      # pretend the list ends after its first block
+            used = torch.tensor([BM], dtype=torch.int32)
+        c = torch.full((M, top_k, N), 3.0, dtype=out_ty)
+        want = O.fused_moe_a8w8(a.numpy(), b.numpy(), c.float().reshape(M * top_k, N).numpy().copy(), O.to_np(ar),
+                                ac.numpy(), w.numpy(), s.numpy(), e.numpy(), used.numpy(), mul_w, top_k, BM, _tag(out_ty))
+        cd = c.to(DEV)
+        got = flashnn_amd.fused_moe_a8w8_forward(a.to(DEV), b.to(DEV), cd, ar.to(DEV), ac.to(DEV), w.to(DEV), ids.to(DEV),
+                                                 s.to(DEV), e.to(DEV), used.to(DEV), mul_w, top_k, BM)
+        assert got is cd
+        assert np.array_equal(cd.float().cpu().reshape(M * top_k, N).numpy(), want)
+        if cut:
+            assert (want == 3.0).any()
+
+
 # ------------------------------------------------------------------ weight-only GEMM
 def _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp, with_bias, seed):
     g = torch.Generator().manual_seed(seed)

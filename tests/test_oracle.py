@@ -355,3 +355,75 @@ def test_layernorm_dquant_matches_torch_ops(dtype, shape):
     n_t = T.layernorm(x, w, b, 1e-5)
     q_x, s_x = O.dynamic_quantize(O.to_np(n_t).reshape(-1, K), O.tag_of(x), scale_dtype=O.tag_of(x), clamp=True)
     assert np.array_equal(q_x, q_t.numpy().reshape(-1, K)) and np.array_equal(s_x, s_t.float().numpy()[:, 0])
+
+
+# ------------------------------------------------------------------- mixture of experts
+def _moe_case(M, E, N, K, top_k, block_m, seed):
+    from flashnn_amd import workloads
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g)
+    b = torch.randint(-128, 128, (E, N, K), dtype=torch.int8, generator=g)
+    ar = (torch.rand(M, generator=g) * 0.05).half()
+    ac = (torch.rand(E, N, generator=g) * 0.05).half()
+    logits = torch.randn(M, E, generator=g)
+    w, ids = torch.topk(torch.softmax(logits, -1), top_k, dim=-1)
+    sorted_ids, expert_ids, used = workloads.moe_align_block_size(ids, block_m, E)
+    return a, b, ar, ac, w.float().contiguous(), ids, sorted_ids, expert_ids, used
+
+
+def test_moe_align_block_size_layout():
+    from flashnn_amd import workloads
+    ids = torch.tensor([[0, 2], [2, 1], [2, 0]])
+    s, e, used = workloads.moe_align_block_size(ids, 4, 3)
+    # expert 0 owns routed rows 0 and 5, expert 1 row 3, expert 2 rows 1, 2, 4; 6 = padding
+    assert s.tolist()[:12] == [0, 5, 6, 6, 3, 6, 6, 6, 1, 2, 4, 6]
+    assert e.tolist()[:3] == [0, 1, 2] and used.item() == 12
+    assert s.dtype == torch.int32 and len(s) % 4 == 0 and set(s.tolist()[12:]) <= {6}
+    # an expert without rows takes no block
+    s, e, used = workloads.moe_align_block_size(torch.tensor([[2], [2]]), 16, 3)
+    assert used.item() == 16 and e[0] == 2 and s.tolist()[:3] == [0, 1, 2]
+
+
+@pytest.mark.parametrize("mul_w", [False, True])
+def test_fused_moe_a8w8_against_per_element_loop(mul_w):
+    M, E, N, K, top_k, BM = 5, 3, 8, 32, 2, 4
+    a, b, ar, ac, w, ids, s, e, used = _moe_case(M, E, N, K, top_k, BM, 40)
+    c = np.full((M * top_k, N), -7.0, np.float32)
+    O.fused_moe_a8w8(a.numpy(), b.numpy(), c, O.to_np(ar), O.to_np(ac), w.numpy(), s.numpy(), e.numpy(), used.numpy(),
+                     mul_w, top_k, BM, O.F16)
+    flat = ids.flatten().tolist()
+    for t in range(M * top_k):          # every routed row is listed exactly once, under its own expert
+        ex = flat[t]
+        for n in range(N):
+            acc = sum(int(a[t // top_k, k]) * int(b[ex, n, k]) for k in range(K))
+            f = np.float32(np.float32(np.float32(acc) * np.float32(ar[t // top_k])) * np.float32(ac[ex, n]))
+            if mul_w:
+                f = np.float32(f * w.flatten()[t].numpy())
+            assert c[t, n] == np.float32(np.float16(f)), (t, n)
+
+
+def test_fused_moe_a8w8_reductions_and_invariants():
+    M, E, N, K, top_k, BM = 9, 4, 16, 64, 2, 4
+    a, b, ar, ac, w, ids, s, e, used = _moe_case(M, E, N, K, top_k, BM, 41)
+    args = (O.to_np(ar), O.to_np(ac), w.numpy())
+    c = O.fused_moe_a8w8(a.numpy(), b.numpy(), np.zeros((M * top_k, N), np.float32), *args, s.numpy(), e.numpy(),
+                         used.numpy(), True, top_k, BM, O.BF16)
+    # one expert, top_k = 1, identity order: the plain A8W8 GEMM with the fp32 epilogue
+    one = O.fused_moe_a8w8(a.numpy(), b.numpy()[1:2], np.zeros((M, N), np.float32), O.to_np(ar), O.to_np(ac)[1:2], None,
+                           np.r_[np.arange(M), [M] * 3].astype(np.int32), np.zeros(3, np.int32), np.array([12]),
+                           False, 1, BM, O.F16)
+    want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.numpy(), b.numpy()[1]), O.to_np(ar), O.to_np(ac)[1], O.F16)
+    assert np.array_equal(one, want)
+    # the order of the rows inside an expert's blocks does not matter
+    s2 = s.clone()
+    s2[0:BM] = s[0:BM].flip(0)
+    c2 = O.fused_moe_a8w8(a.numpy(), b.numpy(), np.zeros((M * top_k, N), np.float32), *args, s2.numpy(), e.numpy(),
+                          used.numpy(), True, top_k, BM, O.BF16)
+    assert np.array_equal(c, c2)
+    # rows beyond num_tokens_post_padded are not touched: cutting the list after the first block
+    # leaves every row of the other blocks at its old value
+    c3 = O.fused_moe_a8w8(a.numpy(), b.numpy(), np.full((M * top_k, N), 3.0, np.float32), *args, s.numpy(), e.numpy(),
+                          np.array([BM]), True, top_k, BM, O.BF16)
+    first = [t for t in s[:BM].tolist() if t < M * top_k]
+    rest = [t for t in range(M * top_k) if t not in first]
+    assert np.array_equal(c3[first], c[first]) and (c3[rest] == 3.0).all()
