@@ -58,7 +58,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: a8w8,a16w4,rows,calib (default: all but calib)")
+    ap.add_argument("--only", default="", help="comma list of legs: a8w8,a16w4,rows,moe,calib (default: all but calib)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (one MI355X per box); run with --gpus 1. "
@@ -73,7 +73,7 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = "cuda:0"
-    legs = set(args.only.split(",")) if args.only else {"a8w8", "a16w4", "rows"}
+    legs = set(args.only.split(",")) if args.only else {"a8w8", "a16w4", "rows", "moe"}
     props = torch.cuda.get_device_properties(0)
     result = {}
 
@@ -271,6 +271,34 @@ def main():
                                            "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                            "frac": round(nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
         del hs
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------ mixture of experts, int8 (decode-sized batches)
+    if "moe" in legs:
+        E, Nm, Km, top_k, BMm = 8, 28672, 4096, 2, 16     # Mixtral-8x7B-like gate+up projection
+        g = torch.Generator(device=dev).manual_seed(7)
+        bm = torch.randint(-127, 128, (E, Nm, Km), dtype=torch.int8, device=dev, generator=g)
+        acm = torch.rand(E, Nm, device=dev, generator=g) * 0.01
+        for Mt in (16, 64):
+            am = torch.randint(-127, 128, (Mt, Km), dtype=torch.int8, device=dev, generator=g)
+            arm = torch.rand(Mt, device=dev, generator=g).half()
+            tw, tid = torch.topk(torch.softmax(torch.randn(Mt, E, generator=torch.Generator().manual_seed(8)), -1), top_k)
+            sid, eid, used = workloads.moe_align_block_size(tid, BMm, E)
+            active = len(set(tid.flatten().tolist()))
+            tw, tid, sid, eid, used = (t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used))
+            cm = torch.empty(Mt, top_k, Nm, dtype=torch.bfloat16, device=dev)
+            f = lambda i: flashnn_amd.fused_moe_a8w8_forward(am, bm, cm, arm, acm, tw, tid, sid, eid, used, True, top_k, BMm)
+            for i in range(3):
+                f(i)
+            ms = _events_ms(f, 20, torch)
+            mb_ = float(active) * Nm * Km + 2.0 * Mt * top_k * Nm      # weights of the experts in use + output
+            secondary.append({"workload": f"fused_moe_a8w8 tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={BMm} "
+                                          f"({active} experts in use)", "kernel": "gemm_a8w8_panel_kernel",
+                              "us_per_launch": round(ms * 1e3, 2),
+                              "roofline": {"bound": "hbm", "achieved": round(mb_ / (ms * 1e-3) / 1e9, 1),
+                                           "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                           "frac": round(mb_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+        del bm
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ CPU baseline
