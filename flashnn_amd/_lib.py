@@ -9,6 +9,7 @@ LIB_PATH = os.path.join(_HERE, "libflashnn_hip.so")
 
 FNN_F16, FNN_BF16, FNN_F32 = 0, 1, 2
 _DTYPE_CODE = {torch.float16: FNN_F16, torch.bfloat16: FNN_BF16, torch.float32: FNN_F32}
+FNN_I8 = 3   # accepted for the zero points of fnn_fused_moe_a16w4 only
 
 _i64, _int, _ptr, _f32 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_float
 
@@ -26,6 +27,7 @@ _SIGNATURES = {
     "fnn_gemm_a16w8": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],
     "fnn_gemm_a16w4": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],
     "fnn_fused_moe_a8w8": [_ptr] * 9 + [_i64] * 9 + [_int] * 7 + [_ptr],
+    "fnn_fused_moe_a16w4": [_ptr] * 9 + [_i64] * 14 + [_int] * 8 + [_ptr],
     "fnn_debug_force_a8w8_tile": [_int, _int],
     "fnn_debug_mfma_rate": [_ptr, _int, _int, _int, ctypes.POINTER(ctypes.c_double), _ptr],
 }

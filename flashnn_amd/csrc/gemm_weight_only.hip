@@ -1094,3 +1094,102 @@ extern "C" int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const 
     return run_wo<4>("fnn_gemm_a16w4", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group,
                      act_dtype, out_dtype, scale_dtype, zp_dtype, bias_dtype, stream);
 }
+
+// ------------------------------------------------------------------ mixture of experts, int4 weights
+namespace fnn {
+
+constexpr int FNN_I8 = 3;   // zero points may be integers
+
+__device__ __forceinline__ float load_zp_f32(const void* p, int64_t i, int dtype) {
+    return dtype == FNN_I8 ? (float)((const int8_t*)p)[i] : load_as_f32(p, i, dtype);
+}
+
+// Any shape, per-channel or grouped scales with any strides: one thread per output value.
+// out[t, n] = sum over K blocks g of scale[e, n, g] * sum_{k in g} act[t / top_k, k] * (nibble(e, n, k) - zp[e, n, g])
+template <int ADT>
+__global__ __launch_bounds__(256) void moe_a16w4_any_kernel(const WoArgs p, const MoeArgs q) {
+    const int sidx = blockIdx.x;
+    if (sidx >= q.ntpp[0]) return;
+    const int tok = q.sorted_ids[sidx];
+    if (tok >= q.num_valid) return;
+    const int n = blockIdx.y * 256 + threadIdx.x;
+    if (n >= p.N) return;
+    const int expert = q.expert_ids[sidx / q.block_m];
+    const uint16_t* a = (const uint16_t*)p.act + (int64_t)(tok / q.top_k) * p.lda;
+    const int8_t* w = p.qw + (int64_t)expert * q.stride_be + (int64_t)(n >> 1) * p.ldw;
+    const int g = p.group > 0 ? p.group : p.K;
+    float acc = 0.f;
+    for (int k0 = 0, kb = 0; k0 < p.K; k0 += g, ++kb) {
+        const float zp = p.zp ? load_zp_f32(p.zp, expert * q.stride_zp_be + n * q.stride_zp_n + kb * q.stride_zp_k, p.zp_dtype)
+                              : 0.f;
+        float part = 0.f;
+        const int k1 = min(k0 + g, p.K);
+        for (int k = k0; k < k1; ++k) {
+            const int b = w[k];
+            const int nib = (n & 1) ? (b >> 4) : ((int)(int8_t)((uint8_t)b << 4) >> 4);
+            part += bits_to_f32<ADT>(a[k]) * ((float)nib - zp);
+        }
+        acc += part * load_as_f32(p.scale, expert * q.stride_scale_be + n * q.stride_scale_n + kb * q.stride_scale_k,
+                                  p.scale_dtype);
+    }
+    if (q.mul_w) acc *= load_as_f32(q.topk_w, tok, q.topk_w_dtype);
+    ((uint16_t*)p.out)[(int64_t)tok * p.ldc + n] = (uint16_t)f32_to_bits<ADT>(acc);
+}
+
+}  // namespace fnn
+
+extern "C" int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const void* scale_b,
+                                   const void* zero_points, const void* topk_weights,
+                                   const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                   const int32_t* num_tokens_post_padded, int64_t N, int64_t K, int64_t EM,
+                                   int64_t num_valid_tokens, int64_t lda, int64_t stride_be, int64_t ldb,
+                                   int64_t ldc, int64_t stride_scale_be, int64_t stride_scale_n,
+                                   int64_t stride_scale_k, int64_t stride_zp_be, int64_t stride_zp_n,
+                                   int64_t stride_zp_k, int group, int mul_routed_weight, int top_k, int block_m,
+                                   int act_dtype, int scale_dtype, int zp_dtype, int topk_weights_dtype,
+                                   void* stream) {
+    using namespace fnn;
+    const char* fn = "fnn_fused_moe_a16w4";
+    if (!c || !a || !b || !scale_b || !sorted_token_ids || !expert_ids || !num_tokens_post_padded ||
+        (mul_routed_weight && !topk_weights)) {
+        set_error("%s: null pointer argument", fn);
+        return FNN_ERR_ARG;
+    }
+    if (N < 0 || K <= 0 || EM < 0 || num_valid_tokens < 0 || top_k <= 0 || block_m <= 0 || lda < K || ldb < K ||
+        ldc < 2 * N || group < 0 || (group > 0 && K % group != 0)) {
+        set_error("%s: bad shape N=%lld K=%lld EM=%lld tokens=%lld top_k=%d block_m=%d group=%d", fn, (long long)N,
+                  (long long)K, (long long)EM, (long long)num_valid_tokens, top_k, block_m, group);
+        return FNN_ERR_ARG;
+    }
+    if (2 * N > 0x7FFFFFFFLL || K > 0x7FFFFFFFLL || EM > 0x7FFFFFFFLL || num_valid_tokens > 0x7FFFFFFFLL) {
+        set_error("%s: shape too large", fn);
+        return FNN_ERR_UNSUPPORTED;
+    }
+    if (!is16(act_dtype)) { set_error("%s: activations must be float16 or bfloat16", fn); return FNN_ERR_UNSUPPORTED; }
+    if (!isflt(scale_dtype) || (zero_points && !isflt(zp_dtype) && zp_dtype != FNN_I8) ||
+        (mul_routed_weight && !isflt(topk_weights_dtype))) {
+        set_error("%s: bad scale, zero point or routing weight type", fn);
+        return FNN_ERR_UNSUPPORTED;
+    }
+    if (N == 0 || EM == 0 || num_valid_tokens == 0) return FNN_OK;
+    WoArgs p{};
+    p.act = a; p.qw = (const int8_t*)b; p.scale = scale_b; p.zp = zero_points; p.bias = nullptr; p.out = c;
+    p.M = (int)EM; p.N = (int)(2 * N); p.K = (int)K; p.lda = lda; p.ldw = ldb; p.ldc = ldc; p.group = group;
+    p.out_dtype = act_dtype; p.scale_dtype = scale_dtype; p.zp_dtype = zp_dtype; p.bias_dtype = act_dtype;
+    MoeArgs q{};
+    q.sorted_ids = sorted_token_ids; q.expert_ids = expert_ids; q.ntpp = num_tokens_post_padded;
+    q.topk_w = topk_weights; q.topk_w_dtype = topk_weights_dtype; q.mul_w = mul_routed_weight ? 1 : 0;
+    q.top_k = top_k; q.block_m = block_m; q.num_valid = (int)num_valid_tokens; q.EM = (int)EM;
+    q.stride_be = stride_be; q.stride_scale_be = stride_scale_be; q.stride_zp_be = stride_zp_be;
+    q.stride_scale_n = stride_scale_n; q.stride_scale_k = stride_scale_k;
+    q.stride_zp_n = stride_zp_n; q.stride_zp_k = stride_zp_k;
+    hipStream_t st = (hipStream_t)stream;
+    // the weight-streaming kernel folds per-channel scales stored one after another
+    const bool fast = group == 0 && stride_scale_n == 1 && (!zero_points || (stride_zp_n == 1 && zp_dtype != FNN_I8));
+    if (!(fast && launch_wo_panel_moe(p, q, act_dtype, st))) {
+        const dim3 grid((unsigned)EM, (unsigned)((2 * N + 255) / 256));
+        if (act_dtype == FNN_F16) moe_a16w4_any_kernel<FNN_F16><<<grid, dim3(256), 0, st>>>(p, q);
+        else moe_a16w4_any_kernel<FNN_BF16><<<grid, dim3(256), 0, st>>>(p, q);
+    }
+    return check_launch(fn);
+}

@@ -63,8 +63,9 @@ __device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4
 // D: slabs of weights in flight per wave (8 loads per lane in flight stream faster than 16: measured
 // 19.8 against 21.7 us for 117 MB in a load-only model).  NTL: non-temporal weight loads, for a
 // single pass over the weights.
-template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL>
-__global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, const int passes) {
+template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL, bool MOE = false>
+__global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, const int passes, const MoeArgs q) {
+    static_assert(!MOE || !G128, "the gathered form folds per-channel scales only");
     constexpr int KS = 8 / RT;
     typedef MfmaT<ADT> MT;
     constexpr int NH = WBITS == 4 ? 2 : 1;      // channels per weight row
@@ -100,6 +101,17 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     if (tile >= tiles) return;
     const int m_base = p.m_base + pass * (MB * 16);
     const int row0 = (tile * RT + rt) * 16;
+    // mixture of experts: the pass covers sorted rows m_base .. of one expert; passes beyond the rows
+    // in use have nothing to do
+    int expert = 0;
+    if constexpr (MOE) {
+        if (m_base >= q.ntpp[0]) return;
+        expert = q.expert_ids[m_base / q.block_m];
+    }
+    auto token_of = [&](int r) -> int {
+        const int sidx = m_base + r;
+        return sidx < q.EM ? q.sorted_ids[sidx] : q.num_valid;
+    };
 
     const int KT = p.K / 128;
     const int sl0 = KT * ks / KS;               // this wave's slabs: sl0 .. sl0 + nsl - 1
@@ -111,7 +123,8 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     // a quarter slower from HBM).  A wave-private 2 KB staging area in LDS turns the two loads
     // into the operand layout: row i at i*128, its 16-byte chunk c at slot c ^ ((i >> 1) & 7).
     const int wr8 = lane >> 3, wc8 = lane & 7;
-    const char* wptr = (const char*)p.qw + (int64_t)(row0 + wr8) * p.ldw + wc8 * 16 + (int64_t)sl0 * 128;
+    const char* wptr = (const char*)p.qw + (MOE ? (int64_t)expert * q.stride_be : 0) + (int64_t)(row0 + wr8) * p.ldw +
+                       wc8 * 16 + (int64_t)sl0 * 128;
     const int64_t w_half = 8 * p.ldw;
     auto load_w = [&](int jj, int half) -> v4u {
         const int j = min(jj, nsl - 1);
@@ -138,7 +151,12 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     for (int i = 0; i < NCP; ++i) {
         const int tok = i * (4 * RT) + tokq;
         const int chunk = (t & 15) ^ (tok & 15);
-        goff[i] = (int64_t)min(m_base + tok, p.M - 1) * p.lda * 2 + chunk * 16;
+        if constexpr (MOE) {
+            const int id = token_of(tok);
+            goff[i] = (int64_t)(id < q.num_valid ? id / q.top_k : 0) * p.lda * 2 + chunk * 16;
+        } else {
+            goff[i] = (int64_t)min(m_base + tok, p.M - 1) * p.lda * 2 + chunk * 16;
+        }
     }
     auto copy_act = [&](char* stage, int jj) {
         const int j = min(jj, nsl - 1);
@@ -321,8 +339,9 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         float sc[NCL], zc[NCL];
 #pragma unroll
         for (int c = 0; c < NCL; ++c) {
-            sc[c] = load_as_f32(p.scale, n0 + c, p.scale_dtype);
-            zc[c] = c_off + (has_zp ? load_as_f32(p.zp, n0 + c, p.zp_dtype) : 0.f);
+            sc[c] = load_as_f32(p.scale, (MOE ? (int64_t)expert * q.stride_scale_be : 0) + n0 + c, p.scale_dtype);
+            zc[c] = c_off + (has_zp ? load_as_f32(p.zp, (MOE ? (int64_t)expert * q.stride_zp_be : 0) + n0 + c, p.zp_dtype)
+                                    : 0.f);
         }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
@@ -371,13 +390,20 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     const bool out_f16 = p.out_dtype == FNN_F16;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-        const int m = m_base + mb * 16 + li;
-        if (m >= p.M) continue;
+        int m = m_base + mb * 16 + li;      // output row; for gathered rows the routed-row id
+        float wroute = 1.f;
+        if constexpr (MOE) {
+            m = token_of(mb * 16 + li);
+            if (m >= q.num_valid) continue;
+            if (q.mul_w) wroute = load_as_f32(q.topk_w, m, q.topk_w_dtype);
+        } else {
+            if (m >= p.M) continue;
+        }
         uint32_t pk[NCL / 2];
 #pragma unroll
         for (int c = 0; c < NCL; c += 2) {
-            const float v0 = (NH == 2 ? outv[mb][0][c >> 1] : outv[mb][0][c]) + bias[c];
-            const float v1 = (NH == 2 ? outv[mb][1][c >> 1] : outv[mb][0][c + 1]) + bias[c + 1];
+            const float v0 = ((NH == 2 ? outv[mb][0][c >> 1] : outv[mb][0][c]) + bias[c]) * wroute;
+            const float v1 = ((NH == 2 ? outv[mb][1][c >> 1] : outv[mb][0][c + 1]) + bias[c + 1]) * wroute;
             const uint32_t b0 = out_f16 ? f32_to_f16_bits(v0) : f32_to_bf16_bits(v0);
             const uint32_t b1 = out_f16 ? f32_to_f16_bits(v1) : f32_to_bf16_bits(v1);
             pk[c >> 1] = (b0 & 0xFFFFu) | (b1 << 16);
@@ -426,8 +452,8 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     p.m_base = 0;
 #define FNN_PANEL2(G, SDTV, MBV, RTV)                                                                    \
     do {                                                                                                 \
-        if (passes == 1) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, true><<<grid, dim3(512), 0, st>>>(p, passes); \
-        else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, false><<<grid, dim3(512), 0, st>>>(p, passes);         \
+        if (passes == 1) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, true><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{}); \
+        else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, false><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{});         \
     } while (0)
 #define FNN_PANEL(G, SDTV)                                   \
     do {                                                     \
@@ -451,6 +477,48 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
 #undef FNN_PANEL
 #undef FNN_PANEL2
     return true;
+}
+
+template <int ADT>
+static bool launch_panel_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
+    const int wrows = p.N / 2;
+    if (p.N % 32 != 0 || p.K % 128 != 0 || p.K < 8 * 128 || p.group != 0 || q.block_m % 16 != 0 || q.EM % q.block_m != 0 ||
+        p.lda % 8 != 0 || p.ldw % 16 != 0 || q.stride_be % 16 != 0 || ((uintptr_t)p.act % 16) != 0 ||
+        ((uintptr_t)p.qw % 16) != 0)
+        return false;
+    const int mb_max = q.block_m % 64 == 0 ? 4 : q.block_m % 32 == 0 ? 2 : 1;   // a pass stays within one expert's block
+    int rt = 0;
+    double best = 0.0;
+    for (int cand = 4; cand >= 1; cand >>= 1) {
+        if (wrows % (16 * cand) != 0) continue;
+        const int t = wrows / (16 * cand);
+        const double fill = (double)t / (((t + 255) / 256) * 256);
+        const double score = fill * (cand == 4 ? 1.0 : cand == 2 ? 0.9 : 0.6);
+        if (score > best) { best = score; rt = cand; }
+    }
+    const int mb = mb_max < rt ? mb_max : rt;
+    const int tiles = wrows / (16 * rt);
+    const int passes = q.EM / (mb * 16);
+    const dim3 grid(((tiles + 7) / 8) * 8 * passes);
+    p.m_base = 0;
+#define FNN_MOE(MBV, RTV) \
+    gemm_wo_panel_kernel<4, ADT, false, FNN_F16, MBV, RTV, 4, false, true><<<grid, dim3(512), 0, st>>>(p, passes, q)
+    if (rt == 4) {
+        if (mb == 1) FNN_MOE(1, 4);
+        else if (mb == 2) FNN_MOE(2, 4);
+        else FNN_MOE(4, 4);
+    } else if (rt == 2) {
+        if (mb == 1) FNN_MOE(1, 2);
+        else FNN_MOE(2, 2);
+    } else {
+        FNN_MOE(1, 1);
+    }
+#undef FNN_MOE
+    return true;
+}
+
+bool launch_wo_panel_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t st) {
+    return act_dtype == FNN_F16 ? launch_panel_moe_t<FNN_F16>(p, q, st) : launch_panel_moe_t<FNN_BF16>(p, q, st);
 }
 
 bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st) {

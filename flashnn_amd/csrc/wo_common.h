@@ -3,6 +3,7 @@
 #pragma once
 
 #include "fnn_common.h"
+#include "moe_common.h"
 
 namespace fnn {
 
@@ -98,5 +99,7 @@ __device__ __forceinline__ v4u perm_act_w4(const v4u a) {
 
 // gemm_wo_panel.hip: 9 .. a few hundred activation rows; false if the shape does not suit it
 bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
+// the int4 per-channel kernel over gathered rows of a mixture of experts; false if the shape does not suit it
+bool launch_wo_panel_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t st);
 
 }  // namespace fnn

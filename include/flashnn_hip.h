@@ -174,6 +174,37 @@ int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const void* alpha_
                        int topk_weights_dtype, void* stream);
 
 /*
+ * Replaces fused_moe_a16w4_forward(A, B, C, scale_b, zero_points, topk_weights, topk_ids,
+ * sorted_token_ids, expert_ids, num_tokens_post_padded, mul_routed_weight, top_k, BM)
+ * (flashnn/triton_kernels/fused_moe_a16w4.py:326-466; kernels :50-206 per channel, :209-323 per K block),
+ * exported as flashnn.fused_moe_a16w4_forward (flashnn/__init__.py:15).
+ *
+ * a: fp16/bf16 [M,K] tokens; b: int8-typed [E,N,K], byte [e,j,k] holding output channel 2j in its low
+ * nibble and 2j+1 in its high nibble, both two's complement (:146-147); c: same type as a, [M*top_k, 2N]
+ * rows with stride ldc.  Routing arguments as for fnn_fused_moe_a8w8.  For a valid routed row t of expert e
+ *   c[t, n] = sum_g scale[e, n, g] * sum_{k in block g} a[t / top_k, k] * (nibble[e, n, k] - zp[e, n, g])
+ * times topk_weights[t] when mul_routed_weight != 0, accumulated in fp32 and rounded once.  group = 0:
+ * one scale and zero point per channel (scale_b [E, 2N]); group = g > 0: per block of g values of K
+ * (scale_b [E, 2N, K/g]).  scale[e, n, g] is read at e*stride_scale_be + n*stride_scale_n + g*stride_scale_k
+ * (zero points alike; zero_points may be NULL).  zp_dtype: FNN_F16/BF16/F32 or 3 for int8.
+ * The weight-streaming kernel takes group = 0 with unit channel stride, floating zero points, N % 16 == 0,
+ * K % 128 == 0, K >= 1024, block_m % 16 == 0, EM % block_m == 0 and 16-byte aligned rows; anything
+ * else (all grouped scales included) takes a slow guarded kernel.  The reference multiplies the dequantised
+ * weights of a K block by their scale before the dot product and rounds them to the scale type; here the
+ * block's dot product is scaled afterwards, in fp32.
+ */
+int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const void* scale_b,
+                        const void* zero_points, const void* topk_weights,
+                        const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                        const int32_t* num_tokens_post_padded, int64_t N, int64_t K, int64_t EM,
+                        int64_t num_valid_tokens, int64_t lda, int64_t stride_be, int64_t ldb,
+                        int64_t ldc, int64_t stride_scale_be, int64_t stride_scale_n,
+                        int64_t stride_scale_k, int64_t stride_zp_be, int64_t stride_zp_n,
+                        int64_t stride_zp_k, int group, int mul_routed_weight, int top_k, int block_m,
+                        int act_dtype, int scale_dtype, int zp_dtype, int topk_weights_dtype,
+                        void* stream);
+
+/*
  * Test hook, no counterpart in the reference: force the output tile (bm x bn) of the MFMA
  * A8W8 kernel for subsequent calls, so that every tile shape can be checked on small
  * problems; (0, 0) restores the automatic choice.  Valid tiles: 256x192, 256x128, 128x128.  Process-wide and not synchronised: for tests only.

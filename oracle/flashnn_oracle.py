@@ -294,6 +294,56 @@ def weight_only_gemm_f64(act, w_nk, scale, zp, bias, group: int) -> np.ndarray:
     return out
 
 
+def fused_moe_a16w4(a, b_packed, c, scale_b, zero_points, topk_weights, sorted_token_ids, expert_ids,
+                    num_tokens_post_padded, mul_routed_weight: bool, top_k: int, block_m: int,
+                    act_dtype: str, scale_dtype: str):
+    """Mixture-of-experts A16W4 GEMM, flashnn/triton_kernels/fused_moe_a16w4.py.  Routing as in
+    fused_moe_a8w8.  b_packed [E, N, K] bytes unpack to 2N channels, low nibble = channel 2j (:146-147).
+    Per channel (scale_b [E, 2N], kernel :50-206): the integers nibble - zp are exact in the activation
+    type (:148-151); fp32 dot product with the tokens (:153); times scale in fp32 (:160-164).
+    Per K block (scale_b [E, 2N, K/g], kernel :209-323): (nibble - zp) * scale is formed in the scale
+    type (:281-303, a rounding per weight), then the fp32 dot product (:306).  Then times
+    topk_weights[t] if asked and one rounding to the activation type (:166-170, :311-315).
+    Dot products are taken in float64 and rounded to fp32 (any fp32 summation order is within a few
+    ulp of that).  `c` ([M*top_k, 2N] float32) is updated in place and returned.
+
+    The reference has no test or torch path for this function.  Pinned by a float64 per-element loop on
+    tiny inputs, the exact integer case and the reduction to weight_only_gemm_f64 (tests/test_oracle.py)."""
+    a = np.asarray(a, dtype=np.float32)
+    b_packed = np.asarray(b_packed)
+    E = b_packed.shape[0]
+    s = np.asarray(scale_b, dtype=np.float32)
+    z = None if zero_points is None else np.asarray(zero_points, dtype=np.float32)
+    w = None if topk_weights is None else np.asarray(topk_weights, dtype=np.float32).reshape(-1)
+    sorted_token_ids = np.asarray(sorted_token_ids).reshape(-1)
+    num_valid = c.shape[0]
+    used = int(np.asarray(num_tokens_post_padded).reshape(-1)[0])
+    K = a.shape[1]
+    for blk in range((len(sorted_token_ids) + block_m - 1) // block_m):
+        if blk * block_m >= used:
+            break
+        e = int(np.asarray(expert_ids).reshape(-1)[blk])
+        toks = sorted_token_ids[blk * block_m:(blk + 1) * block_m]
+        toks = toks[toks < num_valid].astype(np.int64)
+        if toks.size == 0:
+            continue
+        wi = unpack_int4(b_packed[e]).astype(np.float32)            # [2N, K]
+        act = a[toks // top_k].astype(np.float64)
+        if s.ndim == 2:
+            zz = 0.0 if z is None else z[e].reshape(-1, 1)
+            x = (act @ (wi - zz).astype(np.float64).T).astype(np.float32)
+            x = (x * s[e].reshape(1, -1)).astype(np.float32)
+        else:
+            g = K // s.shape[-1]
+            zz = 0.0 if z is None else np.repeat(z[e], g, axis=1)
+            dq = round_to(((wi - zz) * np.repeat(s[e], g, axis=1)).astype(np.float32), scale_dtype)
+            x = (act @ dq.astype(np.float64).T).astype(np.float32)
+        if mul_routed_weight:
+            x = (x * w[toks].reshape(-1, 1)).astype(np.float32)
+        c[toks] = round_to(x, act_dtype)
+    return c
+
+
 # --------------------------------------------------------------------- RMSNorm+quant
 def rmsnorm_dquant(x, gamma, eps: float, dtype: str):
     """Fused RMSNorm + per-token int8 quantisation, flashnn/norm.py:45-60.

@@ -285,6 +285,50 @@ def test_fused_moe_a8w8_bit_exact(shape, mul_w, out_ty):
             assert (want == 3.0).any()
 
 
+@pytest.mark.parametrize("act_ty", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("group,zp_kind", [(0, "float"), (0, None), (0, "int8"), (128, "float"), (64, "int8")])
+@pytest.mark.parametrize("shape", [
+    # M, E, packed rows (half the output channels), K, top_k, BM
+    (16, 8, 512, 1024, 2, 16), (33, 4, 1024, 2048, 2, 32), (70, 4, 528, 1152, 1, 64), (5, 16, 128, 4096, 4, 16),
+    # the guarded kernel: short K, block size not a multiple of 16
+    (9, 3, 16, 128, 2, 16), (12, 3, 32, 1024, 2, 8)])
+def test_fused_moe_a16w4_close(shape, group, zp_kind, act_ty):
+    """fused_moe_a16w4_forward against the oracle within the tolerance stated for 16-bit GEMM outputs;
+    per-channel scales with floating zero points take the weight-streaming kernel, everything else the
+    guarded one.  Rows the sorted list does not name keep their value."""
+    M, E, N2, K, top_k, BM = shape
+    g = torch.Generator().manual_seed(M * 17 + E + group)
+    a = torch.randn(M, K, generator=g).to(act_ty)
+    w = torch.randint(-8, 8, (E, 2 * N2, K), dtype=torch.int8, generator=g)
+    packed = torch.stack([torch.from_numpy(O.pack_int4(w[e].numpy())) for e in range(E)])
+    sshape = (E, 2 * N2) if group == 0 else (E, 2 * N2, K // group)
+    scale = torch.empty(sshape).uniform_(1e-3, 1e-2, generator=g).to(act_ty)
+    zp = None
+    if zp_kind is not None:
+        zp = torch.randint(-3, 4, sshape, generator=g)
+        zp = zp.to(torch.int8) if zp_kind == "int8" else zp.to(act_ty)
+    tw, ids = torch.topk(torch.softmax(torch.randn(M, E, generator=g), -1), top_k, dim=-1)
+    tw = tw.float().contiguous()
+    s, e, used = workloads.moe_align_block_size(ids, BM, E)
+    c = torch.full((M, top_k, 2 * N2), 3.0, dtype=act_ty)
+    want = O.fused_moe_a16w4(O.to_np(a), packed.numpy(), c.float().reshape(M * top_k, 2 * N2).numpy().copy(), O.to_np(scale),
+                             None if zp is None else O.to_np(zp.float()), tw.numpy(), s.numpy(), e.numpy(), used.numpy(),
+                             True, top_k, BM, _tag(act_ty), _tag(act_ty))
+    cd = c.to(DEV)
+    flashnn_amd.fused_moe_a16w4_forward(a.to(DEV), packed.to(DEV), cd, scale.to(DEV), None if zp is None else zp.to(DEV),
+                                        tw.to(DEV), ids.to(DEV), s.to(DEV), e.to(DEV), used.to(DEV), True, top_k, BM)
+    np.testing.assert_allclose(cd.float().cpu().reshape(M * top_k, 2 * N2).numpy(), want, rtol=RTOL, atol=ATOL)
+    # the same list cut after its first block: every other routed row keeps the fill value
+    cd2 = c.to(DEV)
+    flashnn_amd.fused_moe_a16w4_forward(a.to(DEV), packed.to(DEV), cd2, scale.to(DEV), None if zp is None else zp.to(DEV),
+                                        tw.to(DEV), ids.to(DEV), s.to(DEV), e.to(DEV),
+                                        torch.tensor([BM], dtype=torch.int32, device=DEV), False, top_k, BM)
+    first = [t for t in s[:BM].tolist() if t < M * top_k]
+    rest = [t for t in range(M * top_k) if t not in first]
+    got2 = cd2.float().cpu().reshape(M * top_k, 2 * N2)
+    assert bool((got2[rest] == 3.0).all()) and not bool((got2[first] == 3.0).all())
+
+
 # ------------------------------------------------------------------ weight-only GEMM
 def _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp, with_bias, seed):
     g = torch.Generator().manual_seed(seed)

@@ -427,3 +427,62 @@ def test_fused_moe_a8w8_reductions_and_invariants():
     first = [t for t in s[:BM].tolist() if t < M * top_k]
     rest = [t for t in range(M * top_k) if t not in first]
     assert np.array_equal(c3[first], c[first]) and (c3[rest] == 3.0).all()
+
+
+def _moe_w4_case(M, E, N2, K, top_k, block_m, group, seed, zp_int=False):
+    """N2 = packed rows (2*N2 output channels)."""
+    from flashnn_amd import workloads
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(M, K, generator=g).half()
+    w = torch.randint(-8, 8, (E, 2 * N2, K), dtype=torch.int8, generator=g)
+    packed = torch.stack([torch.from_numpy(O.pack_int4(w[e].numpy())) for e in range(E)])
+    sshape = (E, 2 * N2) if group == 0 else (E, 2 * N2, K // group)
+    scale = torch.empty(sshape).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(-3, 4, sshape, generator=g)
+    zp = zp.to(torch.int8) if zp_int else zp.half()
+    tw, ids = torch.topk(torch.softmax(torch.randn(M, E, generator=g), -1), top_k, dim=-1)
+    s, e, used = workloads.moe_align_block_size(ids, block_m, E)
+    return a, w, packed, scale, zp, tw.float().contiguous(), ids, s, e, used
+
+
+@pytest.mark.parametrize("group", [0, 16])
+def test_fused_moe_a16w4_against_f64_loop(group):
+    M, E, N2, K, top_k, BM = 4, 3, 4, 32, 2, 4
+    a, w, packed, scale, zp, tw, ids, s, e, used = _moe_w4_case(M, E, N2, K, top_k, BM, group, 50)
+    c = O.fused_moe_a16w4(O.to_np(a), packed.numpy(), np.zeros((M * top_k, 2 * N2), np.float32), O.to_np(scale),
+                          O.to_np(zp), tw.numpy(), s.numpy(), e.numpy(), used.numpy(), True, top_k, BM, O.F16, O.F16)
+    flat = ids.flatten().tolist()
+    for t in range(M * top_k):
+        ex = flat[t]
+        for n in range(2 * N2):
+            v = mag = 0.0
+            for k in range(K):
+                sg = scale[ex, n] if group == 0 else scale[ex, n, k // group]
+                zg = zp[ex, n] if group == 0 else zp[ex, n, k // group]
+                term = float(a[t // top_k, k]) * (float(w[ex, n, k]) - float(zg)) * float(sg)
+                v += term
+                mag += abs(term)
+            v *= float(tw.flatten()[t])
+            mag *= float(tw.flatten()[t])
+            # one rounding of each dequantised weight to 11 bits (per K block) and one of the result
+            assert abs(c[t, n] - v) <= 2.0 ** -10 * mag + 2.0 ** -10 * abs(v), (t, n, c[t, n], v)
+
+
+def test_fused_moe_a16w4_exact_and_reductions():
+    M, E, N2, K, top_k, BM = 6, 2, 8, 64, 1, 4
+    a, w, packed, scale, zp, tw, ids, s, e, used = _moe_w4_case(M, E, N2, K, top_k, BM, 0, 51, zp_int=True)
+    # integer activations, unit scales, integer zero points: every product and sum is exact
+    ai = torch.randint(-4, 5, (M, K)).half()
+    ones = torch.ones(E, 2 * N2).half()
+    c = O.fused_moe_a16w4(O.to_np(ai), packed.numpy(), np.zeros((M, 2 * N2), np.float32), O.to_np(ones), zp.numpy(),
+                          None, s.numpy(), e.numpy(), used.numpy(), False, 1, BM, O.F16, O.F16)
+    for t in range(M):
+        ex = ids.flatten()[t].item()
+        want = ai[t].double() @ (w[ex].double() - zp[ex].double().reshape(-1, 1)).T
+        assert np.array_equal(c[t], want.numpy().astype(np.float32))
+    # one expert, identity order: GemmWeightOnly's mathematical value (per channel)
+    one = O.fused_moe_a16w4(O.to_np(a), packed.numpy()[1:2], np.zeros((M, 2 * N2), np.float32), O.to_np(scale)[1:2],
+                            zp.numpy()[1:2], None, np.r_[np.arange(M), [M] * 2].astype(np.int32), np.zeros(2, np.int32),
+                            np.array([8]), False, 1, BM, O.F16, O.F16)
+    ref = O.weight_only_gemm_f64(O.to_np(a), w[1].numpy(), O.to_np(scale)[1], zp[1].numpy(), None, 0)
+    np.testing.assert_allclose(one, ref, rtol=2e-3, atol=1e-5)
