@@ -33,27 +33,6 @@ namespace fnn {
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
-// 16 bytes = 16 k of two channels -> operands in natural k order (one byte shuffle per dword
-// puts the nibbles of k and k+1 into the two halves of a dword).
-template <int ADT>
-__device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4u& o0, v4u& o1) {
-    constexpr uint32_t msk = 0x000F000Fu;
-    constexpr uint32_t cst = (ADT == FNN_F16 ? 0x64006400u : 0x43004300u) ^ 0x00080008u;
-    uint32_t e[8], o[8];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const uint32_t y = __builtin_amdgcn_perm(w[q], w[q], 0x03010200u);   // bytes k0 k2 k1 k3
-        e[2 * q] = (y & msk) ^ cst;
-        e[2 * q + 1] = ((y >> 8) & msk) ^ cst;
-        o[2 * q] = ((y >> 4) & msk) ^ cst;
-        o[2 * q + 1] = ((y >> 12) & msk) ^ cst;
-    }
-    e0 = v4u{e[0], e[1], e[2], e[3]};
-    e1 = v4u{e[4], e[5], e[6], e[7]};
-    o0 = v4u{o[0], o[1], o[2], o[3]};
-    o1 = v4u{o[4], o[5], o[6], o[7]};
-}
-
 // G128: per-group tables with group size 128, entries of type SDT (fp16 or bf16), zero points in
 // the same type; otherwise per-channel scales of any type, applied once at the end.
 // RT: 16-row weight tiles per workgroup (4, 2 or 1); the 8 waves are RT tiles x KS = 8 / RT parts of K.

@@ -97,6 +97,28 @@ __device__ __forceinline__ v4u perm_act_w4(const v4u a) {
                __builtin_amdgcn_perm(a[3], a[2], 0x05040100u), __builtin_amdgcn_perm(a[3], a[2], 0x07060302u)};
 }
 
+// 16 bytes = 16 k of two channels -> operands in natural k order (one byte shuffle per dword
+// puts the nibbles of k and k+1 into the two halves of a dword).
+template <int ADT>
+__device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4u& o0, v4u& o1) {
+    constexpr uint32_t msk = 0x000F000Fu;
+    constexpr uint32_t cst = (ADT == FNN_F16 ? 0x64006400u : 0x43004300u) ^ 0x00080008u;
+    uint32_t e[8], o[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t y = __builtin_amdgcn_perm(w[q], w[q], 0x03010200u);   // bytes k0 k2 k1 k3
+        e[2 * q] = (y & msk) ^ cst;
+        e[2 * q + 1] = ((y >> 8) & msk) ^ cst;
+        o[2 * q] = ((y >> 4) & msk) ^ cst;
+        o[2 * q + 1] = ((y >> 12) & msk) ^ cst;
+    }
+    e0 = v4u{e[0], e[1], e[2], e[3]};
+    e1 = v4u{e[4], e[5], e[6], e[7]};
+    o0 = v4u{o[0], o[1], o[2], o[3]};
+    o1 = v4u{o[4], o[5], o[6], o[7]};
+}
+
+
 // gemm_wo_panel.hip: 9 .. a few hundred activation rows; false if the shape does not suit it
 bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
 // the int4 per-channel kernel over gathered rows of a mixture of experts; false if the shape does not suit it
