@@ -23,6 +23,7 @@ _SIGNATURES = {
     "fnn_layernorm": [_ptr, _ptr, _ptr, _ptr, _f32, _i64, _i64, _i64, _i64, _int, _int, _ptr],
     "fnn_layernorm_dquant": [_ptr, _ptr, _ptr, _ptr, _ptr, _f32, _i64, _i64, _i64, _i64, _int, _int, _ptr],
     "fnn_gemm_a8w8": [_ptr] * 5 + [_i64] * 6 + [_int] * 3 + [_ptr],
+    "fnn_gemm_a8w8_tiled": [_ptr] * 5 + [_i64] * 6 + [_int] * 5 + [_ptr],
     "fnn_gemm_a8w8_i32": [_ptr] * 3 + [_i64] * 6 + [_ptr],
     "fnn_gemm_a16w8": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],
     "fnn_gemm_a16w4": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],

@@ -529,34 +529,55 @@ static int check_args(const char* fn, const void* out, const void* a, const void
 
 using namespace fnn;
 
+static bool valid_tile(int bm, int bn);
+
 // Test hook: force a tile shape (bm, bn) for the next calls on any thread; (0, 0) = automatic.
 static int g_force_bm = 0, g_force_bn = 0;
 extern "C" int fnn_debug_force_a8w8_tile(int bm, int bn) {
-    const bool ok = (bm == 0 && bn == 0) || (bm == 256 && (bn == 192 || bn == 128)) ||
-                    (bm == 128 && bn == 128);
-    if (!ok) { set_error("fnn_debug_force_a8w8_tile: no such tile %dx%d", bm, bn); return FNN_ERR_ARG; }
+    if (!valid_tile(bm, bn)) { set_error("fnn_debug_force_a8w8_tile: no such tile %dx%d", bm, bn); return FNN_ERR_ARG; }
     g_force_bm = bm;
     g_force_bn = bn;
     return FNN_OK;
+}
+
+static bool valid_tile(int bm, int bn) {
+    return (bm == 0 && bn == 0) || (bm == 256 && (bn == 192 || bn == 128)) || (bm == 128 && bn == 128);
+}
+
+static int gemm_a8w8_entry(const char* fn, void* out, const void* a, const void* b, const void* alpha_row,
+                           const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                           int64_t ldc, int out_dtype, int alpha_row_dtype, int alpha_col_dtype, int tile_m,
+                           int tile_n, void* stream) {
+    int rc = check_args(fn, out, a, b, M, N, K, lda, ldb, ldc);
+    if (rc != FNN_OK) return rc;
+    if (!alpha_row || !alpha_col) { set_error("%s: null scale pointer", fn); return FNN_ERR_ARG; }
+    if (!is16(out_dtype)) { set_error("%s: Output type must be float16 or bfloat16", fn); return FNN_ERR_UNSUPPORTED; }
+    if (!isflt(alpha_row_dtype) || !isflt(alpha_col_dtype)) { set_error("%s: bad scale type", fn); return FNN_ERR_UNSUPPORTED; }
+    if (!valid_tile(tile_m, tile_n)) { set_error("%s: no such tile %dx%d", fn, tile_m, tile_n); return FNN_ERR_ARG; }
+    if (M == 0 || N == 0) return FNN_OK;
+    A8W8Args p{};
+    p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = out; p.arow = alpha_row; p.acol = alpha_col;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    p.out_dtype = out_dtype; p.arow_dtype = alpha_row_dtype; p.acol_dtype = alpha_col_dtype;
+    if (out_dtype == FNN_F16) dispatch<OUT_F16>(p, (hipStream_t)stream, tile_m, tile_n);
+    else dispatch<OUT_BF16>(p, (hipStream_t)stream, tile_m, tile_n);
+    return check_launch(fn);
 }
 
 extern "C" int fnn_gemm_a8w8(void* out, const void* a, const void* b, const void* alpha_row,
                              const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
                              int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
                              int alpha_col_dtype, void* stream) {
-    int rc = check_args("fnn_gemm_a8w8", out, a, b, M, N, K, lda, ldb, ldc);
-    if (rc != FNN_OK) return rc;
-    if (!alpha_row || !alpha_col) { set_error("fnn_gemm_a8w8: null scale pointer"); return FNN_ERR_ARG; }
-    if (!is16(out_dtype)) { set_error("fnn_gemm_a8w8: Output type must be float16 or bfloat16"); return FNN_ERR_UNSUPPORTED; }
-    if (!isflt(alpha_row_dtype) || !isflt(alpha_col_dtype)) { set_error("fnn_gemm_a8w8: bad scale type"); return FNN_ERR_UNSUPPORTED; }
-    if (M == 0 || N == 0) return FNN_OK;
-    A8W8Args p{};
-    p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = out; p.arow = alpha_row; p.acol = alpha_col;
-    p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
-    p.out_dtype = out_dtype; p.arow_dtype = alpha_row_dtype; p.acol_dtype = alpha_col_dtype;
-    if (out_dtype == FNN_F16) dispatch<OUT_F16>(p, (hipStream_t)stream, g_force_bm, g_force_bn);
-    else dispatch<OUT_BF16>(p, (hipStream_t)stream, g_force_bm, g_force_bn);
-    return check_launch("fnn_gemm_a8w8");
+    return gemm_a8w8_entry("fnn_gemm_a8w8", out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc, out_dtype,
+                           alpha_row_dtype, alpha_col_dtype, g_force_bm, g_force_bn, stream);
+}
+
+extern "C" int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, const void* alpha_row,
+                                   const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                   int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
+                                   int alpha_col_dtype, int tile_m, int tile_n, void* stream) {
+    return gemm_a8w8_entry("fnn_gemm_a8w8_tiled", out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc, out_dtype,
+                           alpha_row_dtype, alpha_col_dtype, tile_m, tile_n, stream);
 }
 
 extern "C" int fnn_gemm_a8w8_i32(int32_t* acc, const void* a, const void* b, int64_t M, int64_t N,

@@ -19,7 +19,9 @@ def get_autotune_triton_kernels():
 
 
 def set_autotune_triton_kernels(v: bool):
-    """Accepted for compatibility; the HIP kernels pick their tiles from a static table."""
+    """True: the first launch of a shape times the candidate tiles of the A8W8 MFMA kernel and records
+    the best in the tuned-configuration file (flashnn_amd/tuned_configs.py); False (the default): recorded
+    configurations are used, other shapes take the library's static choice."""
     global autotune_triton_kernels
     autotune_triton_kernels = v
 

@@ -1,0 +1,111 @@
+"""Shape-keyed tuned configurations with an on-disk JSON file - the role that
+compile_and_cache_kernels and configs/triton_autotune_best_configs.json play in the reference
+(flashnn/triton_kernels/triton_utils.py:14-24, 38-80, 84-151).
+
+A kernel launch is named by a method name ("gemm_a8w8_M_N_K", the reference's own,
+triton_kernels/gemm_a8w8.py:199).  The first time a method name is met while tuning is switched on
+(set_autotune_triton_kernels(True), as in the reference) the candidates are timed on the caller's
+operands and the best one is recorded, in memory and in the JSON file; afterwards, and in later
+processes, the recorded configuration is used without timing anything.  With tuning switched off
+recorded configurations are still honoured; shapes without one take the library's static choice.
+
+File format (the reference's, triton_utils.py:38-57): {method_name: [kwargs, launch_options]} with
+kwargs = {"BLOCK_M": .., "BLOCK_N": ..} ((0, 0) = the library's own choice) and launch_options = {}.
+The file lives at $FLASHNN_AMD_TUNED_CONFIGS or flashnn_amd/configs/hip_autotune_best_configs.json.
+FORECE_RE_TUNE_TRITON_KERNELS (the reference's spelling, triton_utils.py:22-24) lists method-name
+prefixes, separated by ';', that are tuned again even if recorded.
+"""
+import json
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+JSON_FILENAME = "hip_autotune_best_configs.json"
+
+# candidate output tiles of the A8W8 MFMA kernel; (0, 0) = static choice (which may be a few-row kernel)
+A8W8_CANDIDATES = [(0, 0), (256, 192), (256, 128), (128, 128)]
+
+
+def json_file_path():
+    return os.environ.get("FLASHNN_AMD_TUNED_CONFIGS") or os.path.join(_HERE, "configs", JSON_FILENAME)
+
+
+def _force_list():
+    return [k for k in os.getenv("FORECE_RE_TUNE_TRITON_KERNELS", "None").split(";") if k]
+
+
+def force_re_tune(method_name):
+    return any(method_name.startswith(kernel) for kernel in _force_list())
+
+
+def serialize_best_config(tile):
+    return [{"BLOCK_M": int(tile[0]), "BLOCK_N": int(tile[1])}, {}]
+
+
+def deserialize_best_config(entry):
+    kwargs = entry[0]
+    return int(kwargs["BLOCK_M"]), int(kwargs["BLOCK_N"])
+
+
+class TunedConfigs:
+    """In-memory view of the JSON file (read once per path; written through on every new record)."""
+
+    def __init__(self):
+        self._path = None
+        self._data = {}
+        self._tuned_now = set()      # method names tuned by this process (a forced re-tune runs once)
+
+    def _load(self):
+        path = json_file_path()
+        if path != self._path:
+            self._path = path
+            self._data = {}
+            self._tuned_now = set()
+            if os.path.exists(path):
+                with open(path, "r", encoding="utf-8") as f:
+                    self._data = json.load(f)
+        return self._data
+
+    def lookup(self, method_name):
+        """The recorded tile of `method_name`, or None (also when a re-tune is forced and still due)."""
+        data = self._load()
+        if method_name not in data:
+            return None
+        if force_re_tune(method_name) and method_name not in self._tuned_now:
+            return None
+        return deserialize_best_config(data[method_name])
+
+    def record(self, method_name, tile):
+        data = self._load()
+        data[method_name] = serialize_best_config(tile)
+        self._tuned_now.add(method_name)
+        os.makedirs(os.path.dirname(self._path), exist_ok=True)
+        tmp = self._path + ".tmp"
+        with open(tmp, "w", encoding="utf-8") as f:
+            json.dump(data, f, indent=4)
+        os.replace(tmp, self._path)
+
+
+CACHE = TunedConfigs()
+
+
+def tune(method_name, candidates, run, reps=5):
+    """Times run(candidate) for every candidate with GPU events (one warm-up call, then the median of
+    `reps` calls each), records and returns the fastest."""
+    import torch
+    best, best_ms = candidates[0], float("inf")
+    for cand in candidates:
+        run(cand)
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(reps):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            run(cand)
+            e.record()
+            e.synchronize()
+            times.append(s.elapsed_time(e))
+        ms = sorted(times)[len(times) // 2]
+        if ms < best_ms:
+            best, best_ms = cand, ms
+    CACHE.record(method_name, best)
+    return best

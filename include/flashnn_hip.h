@@ -147,6 +147,19 @@ int fnn_layernorm_dquant(void* q, void* scale, const void* x, const void* gamma,
                          int gb_dtype, void* stream);
 
 /*
+ * fnn_gemm_a8w8 with the output tile of the MFMA kernel chosen by the caller: (tile_m, tile_n) one of
+ * 256x192, 256x128, 128x128, or (0, 0) for the library's own choice.  A forced tile also bypasses the
+ * few-row kernels.  This is what a shape-keyed tuned-configuration cache calls - the role that
+ * compile_and_cache_kernels and its JSON file play in the reference
+ * (flashnn/triton_kernels/triton_utils.py:84-151; method name "gemm_a8w8_M_N_K", gemm_a8w8.py:199).
+ * Results are bit-identical for every tile.
+ */
+int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, const void* alpha_row,
+                        const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
+                        int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
+                        int alpha_col_dtype, int tile_m, int tile_n, void* stream);
+
+/*
  * Replaces fused_moe_a8w8_forward(A, B, C, alpha_row_ptr, alpha_col_ptr, topk_weights, topk_ids,
  * sorted_token_ids, expert_ids, num_tokens_post_padded, mul_routed_weight, top_k, BM)
  * (flashnn/triton_kernels/fused_moe_a8w8.py:176-290; kernel :37-173), exported as

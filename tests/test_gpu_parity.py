@@ -249,6 +249,37 @@ def test_a8w8_reference_sweep_shapes(nk, M):
     assert torch.equal(acc.sum(dim=1, dtype=torch.int64), (a.to(torch.int64) * colsum).sum(dim=1))
 
 
+def test_a8w8_tuned_config_cache(tmp_path, monkeypatch):
+    """With tuning on, the first launch of a shape times the candidate tiles and records the best under
+    the reference's method name; the next launch (and a fresh reader of the file) uses the record; the
+    result is the same bits either way."""
+    import json
+    from flashnn_amd import tuned_configs as TC
+    path = tmp_path / "best.json"
+    monkeypatch.setenv("FLASHNN_AMD_TUNED_CONFIGS", str(path))
+    M, N, K = 300, 520, 1024
+    a, b = _rand_i8((M, K), 31), _rand_i8((N, K), 32)
+    g = torch.Generator().manual_seed(33)
+    ar, ac = (torch.rand(M, 1, generator=g) * 0.05).half(), (torch.rand(1, N, generator=g) * 0.05).half()
+    op = flashnn_amd.GemmA8W8(torch.float16)
+    plain = op(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV)).cpu()
+    assert not path.exists()
+    flashnn_amd.set_autotune_triton_kernels(True)
+    try:
+        tuned = op(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV)).cpu()
+    finally:
+        flashnn_amd.set_autotune_triton_kernels(False)
+    data = json.load(open(path))
+    assert list(data) == [f"gemm_a8w8_{M}_{N}_{K}"]
+    tile = TC.deserialize_best_config(data[f"gemm_a8w8_{M}_{N}_{K}"])
+    assert tile in TC.A8W8_CANDIDATES
+    again = op(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV)).cpu()     # from the record, tuning off
+    assert torch.equal(plain, tuned) and torch.equal(plain, again)
+    assert TC.TunedConfigs().lookup(f"gemm_a8w8_{M}_{N}_{K}") == tile
+    want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.numpy(), b.numpy()), O.to_np(ar), O.to_np(ac), O.F16)
+    assert np.array_equal(plain.float().numpy(), want)
+
+
 # ------------------------------------------------------------------ mixture of experts
 @pytest.mark.parametrize("out_ty", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("mul_w", [False, True])

@@ -142,3 +142,38 @@ def test_launcher_asserts_match_the_reference_messages():
     with pytest.raises(AssertionError, match="input must be contiguous"):
         L.hip_dynamic_quantize(torch.empty(4, 64, dtype=torch.int8), torch.zeros(4, 128).half()[:, ::2],
                                torch.empty(4).half())
+
+
+def test_tuned_config_file_format_and_lookup(tmp_path, monkeypatch):
+    """The tuned-configuration cache keeps the reference's file format
+    (flashnn/triton_kernels/triton_utils.py:38-57, 60-75): {method_name: [kwargs, launch options]}."""
+    import json
+    from flashnn_amd import tuned_configs as TC
+    path = tmp_path / "cfg" / "best.json"
+    monkeypatch.setenv("FLASHNN_AMD_TUNED_CONFIGS", str(path))
+    monkeypatch.delenv("FORECE_RE_TUNE_TRITON_KERNELS", raising=False)
+    cache = TC.TunedConfigs()
+    assert cache.lookup("gemm_a8w8_2048_12288_4096") is None
+    cache.record("gemm_a8w8_2048_12288_4096", (256, 192))
+    cache.record("gemm_a8w8_16_4096_4096", (0, 0))
+    data = json.load(open(path))
+    assert data == {"gemm_a8w8_2048_12288_4096": [{"BLOCK_M": 256, "BLOCK_N": 192}, {}],
+                    "gemm_a8w8_16_4096_4096": [{"BLOCK_M": 0, "BLOCK_N": 0}, {}]}
+    # a fresh view (another process) reads the file back
+    other = TC.TunedConfigs()
+    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 192) and other.lookup("gemm_a8w8_1_1_1") is None
+    # forced re-tune by method-name prefix, once per process
+    monkeypatch.setenv("FORECE_RE_TUNE_TRITON_KERNELS", "gemm_a8w8_2048;fuse_moe")
+    assert TC.force_re_tune("gemm_a8w8_2048_12288_4096") and not TC.force_re_tune("gemm_a8w8_16_4096_4096")
+    assert other.lookup("gemm_a8w8_2048_12288_4096") is None and other.lookup("gemm_a8w8_16_4096_4096") == (0, 0)
+    other.record("gemm_a8w8_2048_12288_4096", (256, 128))
+    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 128)
+    assert TC.serialize_best_config((128, 128)) == [{"BLOCK_M": 128, "BLOCK_N": 128}, {}]
+    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 192}, {}]) == (256, 192)
+
+
+def test_tiled_entry_rejects_unknown_tiles(hip_lib):
+    one = ctypes.c_void_p(16)
+    null = ctypes.c_void_p(0)
+    rc = hip_lib.fnn_gemm_a8w8_tiled(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 0, 0, 0, 64, 64, null)
+    assert rc == -1 and b"no such tile 64x64" in hip_lib.fnn_last_error()
