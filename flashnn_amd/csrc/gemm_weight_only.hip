@@ -1021,6 +1021,8 @@ template <int WBITS, int ADT>
 static void dispatch_wo(WoArgs& p, hipStream_t st) {
     const bool fast = p.K % 64 == 0 && (p.group == 0 || p.group % 64 == 0) && p.ldw % 16 == 0 &&
                       p.lda % 8 == 0 && ((uintptr_t)p.qw % 16) == 0 && ((uintptr_t)p.act % 16) == 0;
+    // per-channel scales with K a multiple of 32 only: the panel kernel handles the partial last slab
+    if (p.group == 0 && p.K % 128 != 0 && launch_wo_panel(p, WBITS, ADT, st)) return;
     if (!fast) {
         const int64_t total = (int64_t)p.M * p.N;
         gemm_wo_any_kernel<WBITS, ADT><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(p);

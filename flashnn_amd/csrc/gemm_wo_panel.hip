@@ -92,7 +92,13 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         return sidx < q.EM ? q.sorted_ids[sidx] : q.num_valid;
     };
 
-    const int KT = p.K / 128;
+    // K = 128 * (KT - 1) + tail_k.  With per-channel scales the last slab may be partial (tail_k = 32, 64
+    // or 96): lanes whose 16-byte chunk lies beyond K fetch the first chunk of their row piece instead
+    // (bytes that exist), and the activation fragments of those k are replaced by zeros before the MFMAs,
+    // which removes them from the products and from the activation sums alike.
+    const int KT = (p.K + 127) / 128;
+    const int tail_k = p.K - (KT - 1) * 128;
+    const bool part_tail = tail_k < 128 && ks == KS - 1;   // wave-uniform
     const int sl0 = KT * ks / KS;               // this wave's slabs: sl0 .. sl0 + nsl - 1
     const int nsl = KT * (ks + 1) / KS - sl0;
     const int n_iter = ((KT + KS - 1) / KS + D - 1) / D * D;   // iterations of every wave
@@ -105,9 +111,10 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     const char* wptr = (const char*)p.qw + (MOE ? (int64_t)expert * q.stride_be : 0) + (int64_t)(row0 + wr8) * p.ldw +
                        wc8 * 16 + (int64_t)sl0 * 128;
     const int64_t w_half = 8 * p.ldw;
+    const int wfix = wc8 * 16 >= tail_k ? -(wc8 * 16) : 0;
     auto load_w = [&](int jj, int half) -> v4u {
         const int j = min(jj, nsl - 1);
-        const v4u* src = (const v4u*)(wptr + (int64_t)j * 128 + half * w_half);
+        const v4u* src = (const v4u*)(wptr + (int64_t)j * 128 + half * w_half + (part_tail && j == nsl - 1 ? wfix : 0));
         return NTL ? __builtin_nontemporal_load(src) : *src;
     };
     char* const wmine = wst + wave * 2048;
@@ -126,10 +133,12 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     const int tokq = t >> 4;
     const char* act_part = (const char*)p.act + (int64_t)sl0 * 256;
     int64_t goff[NCP];
+    int afix[NCP];
 #pragma unroll
     for (int i = 0; i < NCP; ++i) {
         const int tok = i * (4 * RT) + tokq;
         const int chunk = (t & 15) ^ (tok & 15);
+        afix[i] = chunk * 8 >= tail_k ? -(chunk * 16) : 0;
         if constexpr (MOE) {
             const int id = token_of(tok);
             goff[i] = (int64_t)(id < q.num_valid ? id / q.top_k : 0) * p.lda * 2 + chunk * 16;
@@ -140,9 +149,10 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     auto copy_act = [&](char* stage, int jj) {
         const int j = min(jj, nsl - 1);
         const char* src = act_part + (int64_t)j * 256;
+        const bool last = part_tail && j == nsl - 1;
 #pragma unroll
         for (int i = 0; i < NCP; ++i)
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + goff[i]),
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + goff[i] + (last ? afix[i] : 0)),
                                              (lds_ptr_t)(stage + ks * SLAB + (i * RT * 64 + rt * 64) * 16), 16, 0, 0);
     };
     // ---- activation fragment reads: lane (li, lg) reads chunks 8 s + 2 lg + h of row 16 mb + li
@@ -216,7 +226,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
 
     // All activation fragments of the slab are requested first, the weights are converted while
     // those reads are in flight, and the MFMAs then run back to back behind a single wait.
-    auto compute = [&](const char* stage, const v4u w0, const v4u w1) {
+    auto compute = [&](const char* stage, const v4u w0, const v4u w1, const bool last) {
         v4u bf[2][MB][2];
 #pragma unroll
         for (int s = 0; s < 2; ++s)
@@ -225,6 +235,16 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
                 bf[s][mb][0] = *(const v4u*)(stage + rd[s][0] + mb * 4096);
                 bf[s][mb][1] = *(const v4u*)(stage + rd[s][1] + mb * 4096);
             }
+        if (last) {   // partial slab: fragment (s, h) of this lane holds k = 8 * (8 s + 2 lg + h) .. + 7
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const bool beyond = (8 * s + 2 * lg + h) * 8 >= tail_k;
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) bf[s][mb][h] = beyond ? v4u{0, 0, 0, 0} : bf[s][mb][h];
+                }
+        }
         if constexpr (WBITS == 4) {
             v4u e[2][2], o[2][2];
             convert_w4_nat<ADT>(w0, e[0][0], e[0][1], o[0][0], o[0][1]);
@@ -269,7 +289,8 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         wq[W][1] = load_w((JJ) + D, 1);                                    \
         __builtin_amdgcn_sched_barrier(0);                                 \
         if (mine_) {                                                       \
-            compute(CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1])); \
+            compute(CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1]), \
+                    !G128 && part_tail && (JJ) == nsl - 1);                \
             if constexpr (G128) fold(sq[Q], zq[Q]);                        \
         }                                                                  \
         if constexpr (G128) {                                              \
@@ -403,8 +424,10 @@ template <int WBITS, int ADT>
 static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     constexpr int NH = WBITS == 4 ? 2 : 1;
     const int wrows = WBITS == 4 ? p.N / 2 : p.N;
-    if (wrows % 16 != 0 || p.K % 128 != 0 || p.K < 8 * 128) return false;
+    if (wrows % 16 != 0 || p.K % 32 != 0 || p.K < 8 * 128) return false;
     if (p.group != 0 && p.group != 128) return false;
+    if (p.group == 128 && p.K % 128 != 0) return false;
+    if (p.lda % 8 != 0 || p.ldw % 16 != 0 || ((uintptr_t)p.qw % 16) != 0 || ((uintptr_t)p.act % 16) != 0) return false;
     if (p.group == 128) {
         const bool tables16 = is16(p.scale_dtype) && (!p.zp || p.zp_dtype == p.scale_dtype) &&
                               p.N % (4 * NH) == 0 && ((uintptr_t)p.scale % (8 * NH)) == 0 &&
@@ -461,7 +484,7 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
 template <int ADT>
 static bool launch_panel_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
     const int wrows = p.N / 2;
-    if (p.N % 32 != 0 || p.K % 128 != 0 || p.K < 8 * 128 || p.group != 0 || q.block_m % 16 != 0 || q.EM % q.block_m != 0 ||
+    if (p.N % 32 != 0 || p.K % 32 != 0 || p.K < 8 * 128 || p.group != 0 || q.block_m % 16 != 0 || q.EM % q.block_m != 0 ||
         p.lda % 8 != 0 || p.ldw % 16 != 0 || q.stride_be % 16 != 0 || ((uintptr_t)p.act % 16) != 0 ||
         ((uintptr_t)p.qw % 16) != 0)
         return false;

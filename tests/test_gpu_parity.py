@@ -321,6 +321,7 @@ def test_fused_moe_a8w8_bit_exact(shape, mul_w, out_ty):
 @pytest.mark.parametrize("shape", [
     # M, E, packed rows (half the output channels), K, top_k, BM
     (16, 8, 512, 1024, 2, 16), (33, 4, 1024, 2048, 2, 32), (70, 4, 528, 1152, 1, 64), (5, 16, 128, 4096, 4, 16),
+    (16, 4, 256, 1056, 2, 16),     # K a multiple of 32 only (per-channel scales stay on the fast kernel)
     # the guarded kernel: short K, block size not a multiple of 16
     (9, 3, 16, 128, 2, 16), (12, 3, 32, 1024, 2, 8)])
 def test_fused_moe_a16w4_close(shape, group, zp_kind, act_ty):
@@ -451,6 +452,36 @@ def test_weight_only_many_rows_small_matrices(bits, group, M, N8, K):
     act_ty = torch.float16 if M % 2 else torch.bfloat16
     case = _wo_inputs(M, N, K, group, bits, act_ty, torch.float16, with_zp=M != 20, with_bias=M == 5, seed=100 + M)
     _wo_check(*case, group, bits, act_ty)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("M", [1, 5, 33, 70])
+@pytest.mark.parametrize("N8,K", [(1024, 1056), (512, 7392), (2064, 1120), (256, 8896)])
+def test_weight_only_partial_last_slab(bits, M, N8, K):
+    """Per-channel scales with K a multiple of 32 but not of 128 (K = 7392, 8896: the FFN shapes of models
+    sharded over 4 or 8 GPUs): the last 128-k slab holds 32, 64 or 96 values.  Zero points and bias on."""
+    N = N8 * (2 if bits == 4 else 1)
+    act_ty = torch.float16 if M % 2 else torch.bfloat16
+    case = _wo_inputs(M, N, K, 0, bits, act_ty, torch.float16, with_zp=True, with_bias=M == 5, seed=300 + M)
+    _wo_check(*case, 0, bits, act_ty)
+
+
+def test_weight_only_partial_last_slab_one_hot():
+    """One-hot activation rows whose single entry lies in the partial last slab, or just before it, pick
+    single weight columns exactly; an entry of ones shows that nothing beyond K is added."""
+    M, N, K = 6, 512, 1120          # 8 slabs of 128 + 96
+    act = torch.zeros(M, K, dtype=torch.float16)
+    cols = [1023, 1024, 1055, 1056, 1119]
+    for i, c in enumerate(cols):
+        act[i, c] = 1.0
+    act[5] = 1.0
+    g = torch.Generator().manual_seed(7)
+    w = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=g)
+    scale = torch.ones(N, dtype=torch.float16)
+    out = flashnn_amd.GemmWeightOnly(torch.float16)(act.to(DEV), w.to(DEV), scale.to(DEV)).float().cpu()
+    for i, c in enumerate(cols):
+        assert torch.equal(out[i], w[:, c].float())
+    assert torch.equal(out[5], w.float().sum(dim=1).half().float())
 
 
 def test_weight_only_many_rows_one_hot():
