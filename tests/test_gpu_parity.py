@@ -537,7 +537,7 @@ def test_a16w4_group128_config(M):
 
 
 # ------------------------------------------------------- rmsnorm+quant -> A8W8 chain
-@pytest.mark.parametrize("M", [1, 32, 512])
+@pytest.mark.parametrize("M", [1, 32, 512, 8192])
 def test_rmsnorm_quant_gemm_chain(M):
     K = N = 8192
     h = workloads.activations(M, K, torch.bfloat16, seed=51, outlier_frac=0.01)
@@ -625,3 +625,67 @@ def test_norm_layers_against_torch_reference_shapes():
         ref = (inp.float() * torch.rsqrt(inp.float().pow(2).mean(-1, keepdim=True) + 1e-5)).type_as(inp) * w
         out = flashnn_amd.RMSNorm(hidden, eps=1e-5).half().to(DEV)(inp.to(DEV))
         torch.testing.assert_close(out.cpu(), ref, atol=1e-3, rtol=1e-3)
+
+
+# ------------------------------------------------------------ streams and graph capture
+def test_kernels_follow_the_current_stream():
+    """Launches go to torch's current stream: work queued on a side stream behind a long-running kernel
+    must see that kernel's output, and the default stream must not be needed for correctness."""
+    x = workloads.activations(512, 4096, torch.float16, seed=61).to(DEV)
+    w, ws = workloads.int8_weights(1024, 4096, seed=62)
+    wd, wsd = w.to(DEV), ws.to(DEV)
+    q_ref, s_ref = flashnn_amd.DynamicQuantize()(x)
+    want = flashnn_amd.GemmA8W8(torch.bfloat16)(q_ref, wd, s_ref, wsd)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        big = torch.randn(4096, 4096, device=DEV)
+        for _ in range(4):
+            big = big @ big * 1e-3              # keeps the side stream busy ahead of the launches below
+        x2 = x + 0                               # produced on the side stream
+        q, s = flashnn_amd.DynamicQuantize()(x2)
+        out = flashnn_amd.GemmA8W8(torch.bfloat16)(q, wd, s, wsd)
+    side.synchronize()
+    assert torch.equal(out, want) and torch.equal(q, q_ref)
+
+
+def test_quant_gemm_step_under_graph_capture():
+    """The C ABI neither allocates nor synchronises, so a DynamicQuant + A8W8 step (and a weight-only
+    decode step) can be captured into a HIP graph; every replay, with fresh inputs copied into the
+    captured buffers and eager work between the replays, must equal the eager result."""
+    M, K, N = 64, 4096, 2048
+    w, ws = workloads.int8_weights(N, K, seed=72)
+    wd, wsd = w.to(DEV), ws.to(DEV)
+    packed, scale, zp, _, _ = workloads.int4_group_weights(1024, K, 128, torch.float16, seed=73)
+    packed, scale, zp = packed.to(DEV), scale.to(DEV), zp.to(DEV)
+    x = torch.zeros(M, K, dtype=torch.float16, device=DEV)
+    q = torch.empty(M, K, dtype=torch.int8, device=DEV)
+    s = torch.empty(M, dtype=torch.float16, device=DEV)
+    out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+    out4 = torch.empty(1, 1024, dtype=torch.float16, device=DEV)
+
+    def step():
+        launchers.hip_dynamic_quantize(q, x, s)
+        launchers.hip_gemm_a8w8_forward(out, q, wd, s, wsd)
+        launchers.hip_gemm_a16w4_forward(out4, x[:1], packed, scale, zero_points=zp)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        xin = workloads.activations(M, K, torch.float16, seed=80 + rep).to(DEV)
+        x.copy_(xin)
+        graph.replay()
+        torch.cuda.synchronize()
+        got, got4 = out.clone(), out4.clone()
+        out.zero_()
+        out4.zero_()
+        step()                                   # eager, same buffers
+        torch.cuda.synchronize()
+        assert torch.equal(got, out) and torch.equal(got4, out4), f"replay {rep}"
+        assert bool(out.abs().sum() > 0)
