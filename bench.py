@@ -323,6 +323,26 @@ def main():
                               "roofline": {"bound": "hbm", "achieved": round(mb_ / (ms * 1e-3) / 1e9, 1),
                                            "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                            "frac": round(mb_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+        # ... and with scales and zero points per group of 128, [E, N, K/128] as the reference lays them out
+        sc4g = (torch.rand(E, Nm, Km // 128, device=dev, generator=g) * 0.01).to(torch.bfloat16)
+        zp4g = torch.randint(-3, 4, (E, Nm, Km // 128), device=dev, generator=g).to(torch.bfloat16)
+        a4 = torch.randn(16, Km, device=dev, generator=g).to(torch.bfloat16)
+        tw, tid = torch.topk(torch.softmax(torch.randn(16, E, generator=torch.Generator().manual_seed(8)), -1), top_k)
+        sid, eid, used = workloads.moe_align_block_size(tid, BMm, E)
+        active = len(set(tid.flatten().tolist()))
+        tw, tid, sid, eid, used = (t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used))
+        cm = torch.empty(16, top_k, Nm, dtype=torch.bfloat16, device=dev)
+        f = lambda i: flashnn_amd.fused_moe_a16w4_forward(a4, b4, cm, sc4g, zp4g, tw, tid, sid, eid, used, True, top_k, BMm)
+        for i in range(3):
+            f(i)
+        ms = _events_ms(f, 20, torch)
+        mb_ = float(active) * (N2 * Km + 4.0 * Nm * (Km // 128)) + 2.0 * 16 * top_k * Nm
+        secondary.append({"workload": f"fused_moe_a16w4 group 128 tokens=16 E={E} top_k={top_k} K={Km} N={Nm} "
+                                      f"block={BMm} ({active} experts in use)", "kernel": "gemm_wo_panel_kernel",
+                          "us_per_launch": round(ms * 1e3, 2),
+                          "roofline": {"bound": "hbm", "achieved": round(mb_ / (ms * 1e-3) / 1e9, 1),
+                                       "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                       "frac": round(mb_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
         del b4
         torch.cuda.empty_cache()
 

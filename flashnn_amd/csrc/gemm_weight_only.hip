@@ -1186,8 +1186,8 @@ extern "C" int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const 
     q.stride_scale_n = stride_scale_n; q.stride_scale_k = stride_scale_k;
     q.stride_zp_n = stride_zp_n; q.stride_zp_k = stride_zp_k;
     hipStream_t st = (hipStream_t)stream;
-    // the weight-streaming kernel folds per-channel scales stored one after another
-    const bool fast = group == 0 && stride_scale_n == 1 && (!zero_points || (stride_zp_n == 1 && zp_dtype != FNN_I8));
+    // the weight-streaming kernel takes per-channel scales and groups of 128 (launch_wo_panel_moe checks the layout)
+    const bool fast = (group == 0 || group == 128) && (!zero_points || zp_dtype != FNN_I8);
     if (!(fast && launch_wo_panel_moe(p, q, act_dtype, st))) {
         const dim3 grid((unsigned)EM, (unsigned)((2 * N + 255) / 256));
         if (act_dtype == FNN_F16) moe_a16w4_any_kernel<FNN_F16><<<grid, dim3(256), 0, st>>>(p, q);

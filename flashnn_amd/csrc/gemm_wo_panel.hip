@@ -44,7 +44,13 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // single pass over the weights.
 template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL, bool MOE = false>
 __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, const int passes, const MoeArgs q) {
-    static_assert(!MOE || !G128, "the gathered form folds per-channel scales only");
+    // Gathered form with group tables: the reference's mixture-of-experts launcher lays them out
+    // [expert][channel][group] (flashnn/triton_kernels/fused_moe_a16w4.py:336-344), the transpose of the
+    // [group][channel] tables above, so 16-byte loads of 8 neighbouring channels do not exist.  The
+    // workgroup's slice of both tables (its channels x all groups, at most 32 KB) is transposed into LDS
+    // once, and the per-slab table reads come from there instead of from memory.
+    constexpr bool TABLDS = MOE && G128;
+    constexpr bool TABG = G128 && !TABLDS;      // tables fetched from memory, slab by slab
     constexpr int KS = 8 / RT;
     typedef MfmaT<ADT> MT;
     constexpr int NH = WBITS == 4 ? 2 : 1;      // channels per weight row
@@ -185,7 +191,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
 
     // loads issued per iteration, in this order: NCP copies, 2 weight loads, 2 table loads
-    constexpr int C = NCP + 2 + (G128 ? 2 : 0);
+    constexpr int C = NCP + 2 + (TABG ? 2 : 0);
     // the newest load slab j depends on is its last copy, issued three iterations earlier; after
     // it came the rest of that iteration and two whole ones
     constexpr int X = (C - NCP) + 2 * C;
@@ -200,6 +206,14 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
 
     v4u wq[D][2];
     tab_t sq[4], zq[4];
+    constexpr int CHW = RT * 16 * NH;           // channels of the workgroup
+    constexpr int TABG_MAX = 64;                // groups the LDS tables hold (K <= 8192)
+    __shared__ __attribute__((aligned(16))) uint16_t tabs[TABLDS ? 2 * TABG_MAX * CHW : 8];
+    const int chl = NH * (rt * 16 + 4 * lg);    // the lane's first channel within the workgroup
+    auto lds_tab = [&](int which, int jj) -> tab_t {
+        const int kg = sl0 + min(jj, nsl - 1);
+        return *(const tab_t*)(tabs + (which * TABG_MAX + kg) * CHW + chl);
+    };
 
     auto fold = [&](const tab_t sv, const tab_t zv) {
         float sc[NCL], zc[NCL];
@@ -291,9 +305,10 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         if (mine_) {                                                       \
             compute(CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1]), \
                     !G128 && part_tail && (JJ) == nsl - 1);                \
-            if constexpr (G128) fold(sq[Q], zq[Q]);                        \
+            if constexpr (TABLDS) fold(lds_tab(0, (JJ)), lds_tab(1, (JJ))); \
+            else if constexpr (G128) fold(sq[Q], zq[Q]);                   \
         }                                                                  \
-        if constexpr (G128) {                                              \
+        if constexpr (TABG) {                                              \
             sq[Q] = load_tab(sptr, (JJ) + 4);                              \
             zq[Q] = load_tab(zptr, (JJ) + 4);                              \
         }                                                                  \
@@ -307,24 +322,44 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         wq[d][0] = load_w(d, 0);
         wq[d][1] = load_w(d, 1);
     }
-    if constexpr (G128) { sq[0] = load_tab(sptr, 0); zq[0] = load_tab(zptr, 0); }
+    if constexpr (TABG) { sq[0] = load_tab(sptr, 0); zq[0] = load_tab(zptr, 0); }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st0, 0);
     wq[D - 3][0] = load_w(D - 3, 0);
     wq[D - 3][1] = load_w(D - 3, 1);
-    if constexpr (G128) { sq[1] = load_tab(sptr, 1); zq[1] = load_tab(zptr, 1); }
+    if constexpr (TABG) { sq[1] = load_tab(sptr, 1); zq[1] = load_tab(zptr, 1); }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st1, 1);
     wq[D - 2][0] = load_w(D - 2, 0);
     wq[D - 2][1] = load_w(D - 2, 1);
-    if constexpr (G128) { sq[2] = load_tab(sptr, 2); zq[2] = load_tab(zptr, 2); }
+    if constexpr (TABG) { sq[2] = load_tab(sptr, 2); zq[2] = load_tab(zptr, 2); }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st2, 2);
     wq[D - 1][0] = load_w(D - 1, 0);
     wq[D - 1][1] = load_w(D - 1, 1);
-    if constexpr (G128) { sq[3] = load_tab(sptr, 3); zq[3] = load_tab(zptr, 3); }
+    if constexpr (TABG) { sq[3] = load_tab(sptr, 3); zq[3] = load_tab(zptr, 3); }
     __builtin_amdgcn_sched_barrier(0);
 
+    if constexpr (TABLDS) {
+        // every channel's groups are contiguous in memory: 16-byte loads of 8 groups, written to
+        // [group][channel]; behind the barrier everything the prologue asked for has landed as well
+        const int G = p.K / 128;
+        const int ch0 = NH * tile * RT * 16;
+        const uint16_t* sg = (const uint16_t*)p.scale + (int64_t)expert * q.stride_scale_be + (int64_t)ch0 * G;
+        const uint16_t* zg = p.zp ? (const uint16_t*)p.zp + (int64_t)expert * q.stride_zp_be + (int64_t)ch0 * G : sg;
+        const int per_ch = G / 8;
+        for (int v = threadIdx.x; v < CHW * per_ch; v += 512) {
+            const int ch = v / per_ch, g8 = v % per_ch;
+            const v4u a = *(const v4u*)(sg + (int64_t)ch * G + g8 * 8);
+            const v4u b = *(const v4u*)(zg + (int64_t)ch * G + g8 * 8);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                tabs[(g8 * 8 + i) * CHW + ch] = (uint16_t)(a[i >> 1] >> (16 * (i & 1)));
+                tabs[(TABG_MAX + g8 * 8 + i) * CHW + ch] = (uint16_t)(b[i >> 1] >> (16 * (i & 1)));
+            }
+        }
+        __syncthreads();
+    }
     static_assert(D == 4, "the unrolled loop below walks four weight slots");
     for (int jj = 0; jj < n_iter; jj += D) {
         FNN_PANEL_ITER(0, 0, st0, st3, jj);
@@ -484,11 +519,22 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
 template <int ADT>
 static bool launch_panel_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
     const int wrows = p.N / 2;
-    if (p.N % 32 != 0 || p.K % 32 != 0 || p.K < 8 * 128 || p.group != 0 || q.block_m % 16 != 0 || q.EM % q.block_m != 0 ||
-        p.lda % 8 != 0 || p.ldw % 16 != 0 || q.stride_be % 16 != 0 || ((uintptr_t)p.act % 16) != 0 ||
-        ((uintptr_t)p.qw % 16) != 0)
+    if (p.N % 32 != 0 || p.K % 32 != 0 || p.K < 8 * 128 || (p.group != 0 && p.group != 128) || q.block_m % 16 != 0 ||
+        q.EM % q.block_m != 0 || p.lda % 8 != 0 || p.ldw % 16 != 0 || q.stride_be % 16 != 0 ||
+        ((uintptr_t)p.act % 16) != 0 || ((uintptr_t)p.qw % 16) != 0)
         return false;
-    const int mb_max = q.block_m % 64 == 0 ? 4 : q.block_m % 32 == 0 ? 2 : 1;   // a pass stays within one expert's block
+    const int G = p.K / 128;
+    if (p.group == 128) {
+        // tables [expert][channel][group] of one 16-bit type, every channel's groups contiguous and 16-byte aligned
+        const bool ok = p.K % 128 == 0 && G % 8 == 0 && G <= 64 && is16(p.scale_dtype) && q.stride_scale_k == 1 &&
+                        q.stride_scale_n == G && q.stride_scale_be % 8 == 0 && ((uintptr_t)p.scale % 16) == 0 &&
+                        (!p.zp || (p.zp_dtype == p.scale_dtype && q.stride_zp_k == 1 && q.stride_zp_n == G &&
+                                   q.stride_zp_be % 8 == 0 && ((uintptr_t)p.zp % 16) == 0));
+        if (!ok) return false;
+    } else if (q.stride_scale_n != 1 || (p.zp && q.stride_zp_n != 1)) {
+        return false;
+    }
+    int mb_max = q.block_m % 64 == 0 ? 4 : q.block_m % 32 == 0 ? 2 : 1;   // a pass stays within one expert's block
     int rt = 0;
     double best = 0.0;
     for (int cand = 4; cand >= 1; cand >>= 1) {
@@ -498,24 +544,36 @@ static bool launch_panel_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
         const double score = fill * (cand == 4 ? 1.0 : cand == 2 ? 0.9 : 0.6);
         if (score > best) { best = score; rt = cand; }
     }
+    // the transposed tables take LDS from the activation stages
+    if (p.group == 128) mb_max = rt == 4 ? (mb_max < 2 ? mb_max : 2) : 1;
     const int mb = mb_max < rt ? mb_max : rt;
     const int tiles = wrows / (16 * rt);
     const int passes = q.EM / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);
     p.m_base = 0;
-#define FNN_MOE(MBV, RTV) \
-    gemm_wo_panel_kernel<4, ADT, false, FNN_F16, MBV, RTV, 4, false, true><<<grid, dim3(512), 0, st>>>(p, passes, q)
-    if (rt == 4) {
-        if (mb == 1) FNN_MOE(1, 4);
-        else if (mb == 2) FNN_MOE(2, 4);
-        else FNN_MOE(4, 4);
-    } else if (rt == 2) {
-        if (mb == 1) FNN_MOE(1, 2);
-        else FNN_MOE(2, 2);
+#define FNN_MOE2(G, SDTV, MBV, RTV) \
+    gemm_wo_panel_kernel<4, ADT, G, SDTV, MBV, RTV, 4, false, true><<<grid, dim3(512), 0, st>>>(p, passes, q)
+#define FNN_MOE(G, SDTV)                                   \
+    do {                                                   \
+        if (rt == 4) {                                     \
+            if (mb == 1) FNN_MOE2(G, SDTV, 1, 4);          \
+            else if (mb == 2) FNN_MOE2(G, SDTV, 2, 4);     \
+            else if constexpr (!G) FNN_MOE2(G, SDTV, 4, 4); \
+        } else if (rt == 2) {                              \
+            if (mb == 1) FNN_MOE2(G, SDTV, 1, 2);          \
+            else if constexpr (!G) FNN_MOE2(G, SDTV, 2, 2); \
+        } else {                                           \
+            FNN_MOE2(G, SDTV, 1, 1);                       \
+        }                                                  \
+    } while (0)
+    if (p.group == 128) {
+        if (p.scale_dtype == FNN_F16) FNN_MOE(true, FNN_F16);
+        else FNN_MOE(true, FNN_BF16);
     } else {
-        FNN_MOE(1, 1);
+        FNN_MOE(false, FNN_F16);
     }
 #undef FNN_MOE
+#undef FNN_MOE2
     return true;
 }
 

@@ -200,11 +200,12 @@ int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const void* alpha_
  * one scale and zero point per channel (scale_b [E, 2N]); group = g > 0: per block of g values of K
  * (scale_b [E, 2N, K/g]).  scale[e, n, g] is read at e*stride_scale_be + n*stride_scale_n + g*stride_scale_k
  * (zero points alike; zero_points may be NULL).  zp_dtype: FNN_F16/BF16/F32 or 3 for int8.
- * The weight-streaming kernel takes group = 0 with unit channel stride, floating zero points, N % 16 == 0,
- * K % 128 == 0, K >= 1024, block_m % 16 == 0, EM % block_m == 0 and 16-byte aligned rows; anything
- * else (all grouped scales included) takes a slow guarded kernel.  The reference multiplies the dequantised
- * weights of a K block by their scale before the dot product and rounds them to the scale type; here the
- * block's dot product is scaled afterwards, in fp32.
+ * The weight-streaming kernel takes group = 0 (unit channel stride, K % 32 == 0) or group = 128 (contiguous
+ * [E, 2N, K/128] tables of one 16-bit type, K/128 a multiple of 8 and at most 64), floating zero points,
+ * N % 16 == 0, K >= 1024, block_m % 16 == 0, EM % block_m == 0 and 16-byte aligned rows; anything else
+ * takes a slow guarded kernel.  The reference multiplies the dequantised weights of a K block by their scale
+ * before the dot product and rounds them to the scale type; here the block's dot product is scaled
+ * afterwards, in fp32.
  */
 int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const void* scale_b,
                         const void* zero_points, const void* topk_weights,

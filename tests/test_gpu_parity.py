@@ -317,7 +317,7 @@ def test_fused_moe_a8w8_bit_exact(shape, mul_w, out_ty):
 
 
 @pytest.mark.parametrize("act_ty", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("group,zp_kind", [(0, "float"), (0, None), (0, "int8"), (128, "float"), (64, "int8")])
+@pytest.mark.parametrize("group,zp_kind", [(0, "float"), (0, None), (0, "int8"), (128, "float"), (128, None), (64, "int8")])
 @pytest.mark.parametrize("shape", [
     # M, E, packed rows (half the output channels), K, top_k, BM
     (16, 8, 512, 1024, 2, 16), (33, 4, 1024, 2048, 2, 32), (70, 4, 528, 1152, 1, 64), (5, 16, 128, 4096, 4, 16),
