@@ -352,7 +352,8 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     } else {
         constexpr int TSTRIDE = WTN * 2 + 16;      // bytes per staged row; the pad staggers the banks
         constexpr int PR = WTN * 2 / 16;           // 16-byte pieces per row
-        static_assert(64 * TSTRIDE <= BN * BK, "transpose buffer must fit a stage");
+        constexpr int RC = FM >= 2 ? 2 : 1;        // 32-row fragments staged at a time
+        static_assert(RC * 32 * TSTRIDE <= BN * BK && RC * 32 * TSTRIDE <= BM * BK, "transpose buffer must fit a stage");
         char* tbuf = wave == 0 ? sa0 : wave == 1 ? sa1 : wave == 2 ? (BDEEP ? sb1 : sa2) : sb0;
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0x0070);   // all copies and LDS reads of this wave are done
@@ -360,9 +361,9 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         asm volatile("" ::: "memory");
         const bool vec_ok = (p.ldc & 7) == 0;
 #pragma unroll
-        for (int jc = 0; jc < FM; jc += 2) {
+        for (int jc = 0; jc < FM; jc += RC) {
 #pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
+            for (int jj = 0; jj < RC; ++jj) {
                 const int j = jc + jj;
                 const float ar = sc_row[wm * WTM + j * 32 + frow];
 #pragma unroll
@@ -388,10 +389,10 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             }
             // rows jc*32 .. jc*32+63 of the wave tile are staged; write them out row by row
 #pragma unroll
-            for (int it = 0; it < (64 * PR + 63) / 64; ++it) {
+            for (int it = 0; it < (RC * 32 * PR + 63) / 64; ++it) {
                 const int e = it * 64 + lane;
                 const int row = e / PR, c = e % PR;
-                if (e < 64 * PR) {
+                if (e < RC * 32 * PR) {
                     const v4u val = *(const v4u*)(tbuf + row * TSTRIDE + c * 16);
                     const int m = wm0 + jc * 32 + row;
                     const int n = wn0 + c * 8;
@@ -469,7 +470,7 @@ struct TileChoice { int bm, bn; };
 // Pick the tile whose last, partly filled round of workgroups costs least on 256 CUs.
 static TileChoice choose_tile(int64_t M, int64_t N) {
     static const struct { int bm, bn; double eff; } cand[] = {
-        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.72}};   // throughput per tile area, measured at K = N = 8192 (at smaller shapes the smaller tiles come closer)
+        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.72}, {64, 128, 0.45}};   // throughput per tile area, measured at K = N = 8192 (at smaller shapes the smaller tiles come closer; a 64x128 tile takes 0.8 of the time of a 128x128 one, so it pays where it doubles the workgroups without adding a round)
     double best = 1e300;
     TileChoice c{128, 128};
     for (const auto& t : cand) {
@@ -507,6 +508,7 @@ static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
     if (force_bm > 0) c = {force_bm, force_bn};
     if (c.bm == 256 && c.bn == 192) launch_mfma<256, 192, MODE>(p, st);
     else if (c.bm == 256 && c.bn == 128) launch_mfma<256, 128, MODE>(p, st);
+    else if (c.bm == 64 && c.bn == 128) launch_mfma<64, 128, MODE>(p, st);
     else launch_mfma<128, 128, MODE>(p, st);
 }
 
@@ -541,7 +543,8 @@ extern "C" int fnn_debug_force_a8w8_tile(int bm, int bn) {
 }
 
 static bool valid_tile(int bm, int bn) {
-    return (bm == 0 && bn == 0) || (bm == 256 && (bn == 192 || bn == 128)) || (bm == 128 && bn == 128);
+    return (bm == 0 && bn == 0) || (bm == 256 && (bn == 192 || bn == 128)) || (bm == 128 && bn == 128) ||
+           (bm == 64 && bn == 128);
 }
 
 static int gemm_a8w8_entry(const char* fn, void* out, const void* a, const void* b, const void* alpha_row,

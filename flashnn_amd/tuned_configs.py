@@ -22,7 +22,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 JSON_FILENAME = "hip_autotune_best_configs.json"
 
 # candidate output tiles of the A8W8 MFMA kernel; (0, 0) = static choice (which may be a few-row kernel)
-A8W8_CANDIDATES = [(0, 0), (256, 192), (256, 128), (128, 128)]
+A8W8_CANDIDATES = [(0, 0), (256, 192), (256, 128), (128, 128), (64, 128)]
 
 
 def json_file_path():

@@ -148,7 +148,7 @@ int fnn_layernorm_dquant(void* q, void* scale, const void* x, const void* gamma,
 
 /*
  * fnn_gemm_a8w8 with the output tile of the MFMA kernel chosen by the caller: (tile_m, tile_n) one of
- * 256x192, 256x128, 128x128, or (0, 0) for the library's own choice.  A forced tile also bypasses the
+ * 256x192, 256x128, 128x128, 64x128, or (0, 0) for the library's own choice.  A forced tile also bypasses the
  * few-row kernels.  This is what a shape-keyed tuned-configuration cache calls - the role that
  * compile_and_cache_kernels and its JSON file play in the reference
  * (flashnn/triton_kernels/triton_utils.py:84-151; method name "gemm_a8w8_M_N_K", gemm_a8w8.py:199).
@@ -221,7 +221,7 @@ int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const void* scale
 /*
  * Test hook, no counterpart in the reference: force the output tile (bm x bn) of the MFMA
  * A8W8 kernel for subsequent calls, so that every tile shape can be checked on small
- * problems; (0, 0) restores the automatic choice.  Valid tiles: 256x192, 256x128, 128x128.  Process-wide and not synchronised: for tests only.
+ * problems; (0, 0) restores the automatic choice.  Valid tiles: 256x192, 256x128, 128x128, 64x128.  Process-wide and not synchronised: for tests only.
  */
 int fnn_debug_force_a8w8_tile(int bm, int bn);
 

@@ -79,7 +79,7 @@ def _rand_i8(shape, seed, lo=-128, hi=128):
     return torch.randint(lo, hi, shape, generator=g, dtype=torch.int8)
 
 
-@pytest.mark.parametrize("tile", [(0, 0), (256, 192), (256, 128), (128, 128)])
+@pytest.mark.parametrize("tile", [(0, 0), (256, 192), (256, 128), (128, 128), (64, 128)])
 @pytest.mark.parametrize("mnk", [(128, 128, 128), (300, 200, 512), (512, 768, 1024), (16, 4096, 4096),
                                  (257, 129, 640), (64, 320, 1152), (130, 100, 2048)])
 def test_a8w8_accumulators_bit_exact(hip_lib, tile, mnk):
@@ -93,7 +93,7 @@ def test_a8w8_accumulators_bit_exact(hip_lib, tile, mnk):
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
 
 
-@pytest.mark.parametrize("tile", [(0, 0), (256, 192), (256, 128), (128, 128)])
+@pytest.mark.parametrize("tile", [(0, 0), (256, 192), (256, 128), (128, 128), (64, 128)])
 @pytest.mark.parametrize("mnk", [(300, 200, 544), (257, 385, 576), (64, 320, 608), (130, 100, 1056),
                                  (10, 1920, 1760), (40, 260, 7392), (520, 390, 8896)])
 def test_a8w8_partial_last_slab_bit_exact(hip_lib, tile, mnk):
