@@ -62,7 +62,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (one MI355X per box); run with --gpus 1. "
-                 "How the path would shard across GPUs is described in DESIGN.md.")
+                 "The configurations are per-GPU shapes: column-parallel layers shard N without any exchange, "
+                 "row-parallel layers shard K and all-reduce the [M, N] partial results.")
 
     import torch
 
