@@ -689,3 +689,39 @@ def test_quant_gemm_step_under_graph_capture():
         torch.cuda.synchronize()
         assert torch.equal(got, out) and torch.equal(got4, out4), f"replay {rep}"
         assert bool(out.abs().sum() > 0)
+
+
+# ------------------------------------------------------------------ strides through the C ABI
+def test_c_abi_row_strides(hip_lib):
+    """The launchers keep the reference's contiguity asserts, the C ABI takes row strides: operands and
+    outputs that are column slices of wider buffers (lda > K, ldb > K, ldc > N) give the same bits."""
+    M, N, K = 70, 144, 1056
+    abuf, bbuf = _rand_i8((M, K + 64), 41).to(DEV), _rand_i8((N, K + 32), 42).to(DEV)
+    a, b = abuf[:, 16:16 + K], bbuf[:, 32:32 + K]          # 16-byte aligned starts, strided rows
+    g = torch.Generator().manual_seed(43)
+    ar = (torch.rand(M, generator=g) * 0.05).half().to(DEV)
+    ac = (torch.rand(N, generator=g) * 0.05).half().to(DEV)
+    obuf = torch.full((M, N + 40), 7.0, dtype=torch.float16, device=DEV)
+    out = obuf[:, 8:8 + N]
+    rc = hip_lib.fnn_gemm_a8w8(out.data_ptr(), a.data_ptr(), b.data_ptr(), ar.data_ptr(), ac.data_ptr(), M, N, K,
+                               a.stride(0), b.stride(0), out.stride(0), 0, 0, 0,
+                               _lib.current_stream(torch.device(DEV)))
+    assert rc == 0, hip_lib.fnn_last_error()
+    torch.cuda.synchronize()
+    want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.cpu().numpy(), b.cpu().numpy()), O.to_np(ar.cpu()),
+                                     O.to_np(ac.cpu()), O.F16)
+    assert np.array_equal(out.float().cpu().numpy(), want)
+    assert bool((obuf[:, :8] == 7).all()) and bool((obuf[:, 8 + N:] == 7).all())     # nothing written outside
+    # dynamic quant with strided input and output rows
+    xbuf = torch.randn(33, 1024 + 64, device=DEV).half()
+    x = xbuf[:, 8:8 + 1024]
+    qbuf = torch.full((33, 1024 + 16), 5, dtype=torch.int8, device=DEV)
+    q = qbuf[:, 8:8 + 1024]
+    sc = torch.empty(33, dtype=torch.float16, device=DEV)
+    rc = hip_lib.fnn_dynamic_quant(q.data_ptr(), sc.data_ptr(), x.data_ptr(), 33, 1024, x.stride(0), q.stride(0), 0,
+                                   _lib.current_stream(torch.device(DEV)))
+    assert rc == 0, hip_lib.fnn_last_error()
+    torch.cuda.synchronize()
+    q_o, s_o = O.dynamic_quantize(O.to_np(x.cpu()), O.F16)
+    assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(sc.cpu().numpy(), s_o)
+    assert bool((qbuf[:, :8] == 5).all()) and bool((qbuf[:, 8 + 1024:] == 5).all())
