@@ -47,11 +47,30 @@ __global__ __launch_bounds__(kRowThreads) void norm_vec_kernel(const NormArgs p)
     const v4u* xr = (const v4u*)(p.x + row * p.ldx);
     const int nvec = p.K >> 3;
     float n[NV][8];
-    double acc = 0.0, acc1 = 0.0;   // sum of squares; sum
+    // short rows: gamma and beta are requested together with the row, so that their latency is not paid
+    // a second time behind the first reduction (a single row is one chain of latencies)
+    constexpr bool PRE = NV <= 4;
+    float gpre[PRE ? NV : 1][8], bpre[PRE && OP != OP_RMS ? NV : 1][8];
+    v4u xv[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int idx = threadIdx.x + i * kRowThreads;
-        const v4u v = idx < nvec ? xr[idx] : v4u{0, 0, 0, 0};
+        xv[i] = idx < nvec ? xr[idx] : v4u{0, 0, 0, 0};
+    }
+    if constexpr (PRE) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int idx = threadIdx.x + i * kRowThreads;
+            if (idx < nvec) {
+                load_gamma8(p.gamma, p.gb_dtype, (int64_t)idx * 8, gpre[i]);
+                if constexpr (OP != OP_RMS) load_gamma8(p.beta, p.gb_dtype, (int64_t)idx * 8, bpre[i]);
+            }
+        }
+    }
+    double acc = 0.0, acc1 = 0.0;   // sum of squares; sum
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const v4u v = xv[i];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             n[i][2 * j] = bits_to_f32<DT>(v[j] & 0xFFFFu);
@@ -85,8 +104,16 @@ __global__ __launch_bounds__(kRowThreads) void norm_vec_kernel(const NormArgs p)
         const int idx = threadIdx.x + i * kRowThreads;
         if (idx < nvec) {
             float g[8], b[8];
-            load_gamma8(p.gamma, p.gb_dtype, (int64_t)idx * 8, g);
-            if constexpr (OP != OP_RMS) load_gamma8(p.beta, p.gb_dtype, (int64_t)idx * 8, b);
+            if constexpr (PRE) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    g[j] = gpre[i][j];
+                    if constexpr (OP != OP_RMS) b[j] = bpre[i][j];
+                }
+            } else {
+                load_gamma8(p.gamma, p.gb_dtype, (int64_t)idx * 8, g);
+                if constexpr (OP != OP_RMS) load_gamma8(p.beta, p.gb_dtype, (int64_t)idx * 8, b);
+            }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 if constexpr (OP == OP_RMS) n[i][j] = round_dt<DT>(round_dt<DT>(n[i][j] * mul) * g[j]);

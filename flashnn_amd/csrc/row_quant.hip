@@ -87,11 +87,27 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_vec_kernel(
     const v4u* xr = (const v4u*)(x + row * ldx);
     const int nvec = K >> 3;
     float n[NV][8];
-    double ssq = 0.0;
+    // short rows: gamma is requested together with the row, so that its latency is not paid a second
+    // time behind the first reduction (a single row is one chain of latencies)
+    constexpr bool PRE = NV <= 4;
+    float gpre[PRE ? NV : 1][8];
+    v4u xv[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int idx = threadIdx.x + i * kRowThreads;
-        const v4u v = idx < nvec ? xr[idx] : v4u{0, 0, 0, 0};
+        xv[i] = idx < nvec ? xr[idx] : v4u{0, 0, 0, 0};
+    }
+    if constexpr (PRE) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int idx = threadIdx.x + i * kRowThreads;
+            if (idx < nvec) load_gamma8(gamma, gamma_dtype, (int64_t)idx * 8, gpre[i]);
+        }
+    }
+    double ssq = 0.0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const v4u v = xv[i];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             n[i][2 * j] = bits_to_f32<DT>(v[j] & 0xFFFFu);
@@ -109,7 +125,12 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_vec_kernel(
         const int idx = threadIdx.x + i * kRowThreads;
         if (idx < nvec) {
             float g[8];
-            load_gamma8(gamma, gamma_dtype, (int64_t)idx * 8, g);
+            if constexpr (PRE) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) g[j] = gpre[i][j];
+            } else {
+                load_gamma8(gamma, gamma_dtype, (int64_t)idx * 8, g);
+            }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 n[i][j] = (n[i][j] * rs) * g[j];
