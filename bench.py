@@ -229,18 +229,20 @@ def main():
             nset8 = max(3, int(600e6 // (k8 * n8)) + 1)
             w8 = [torch.randint(-127, 128, (n8, k8), dtype=torch.int8, device=dev) for _ in range(nset8)]
             s8 = torch.rand(n8, device=dev).half() * 0.01
-            act = workloads.activations(1, k8, torch.float16, seed=4).to(dev)
-            o8 = torch.empty(1, n8, dtype=torch.float16, device=dev)
-            f = lambda i: launchers.hip_gemm_a16w8_forward(o8, act, w8[i % nset8], s8)
-            for i in range(10):
-                f(i)
-            ms = _events_ms(f, 100, torch)
-            b8 = n8 * k8 + 2.0 * n8 + 2.0 * k8 + 2.0 * n8
-            secondary.append({"workload": f"a16w8 decode M=1 K={k8} N={n8} fp16", "kernel": "gemm_wo_decode_lds_kernel",
-                              "us_per_launch": round(ms * 1e3, 2),
-                              "roofline": {"bound": "hbm", "achieved": round(b8 / (ms * 1e-3) / 1e9, 1),
-                                           "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                           "frac": round(b8 / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+            for m8 in (1, 8, 32):
+                act = workloads.activations(m8, k8, torch.float16, seed=4).to(dev)
+                o8 = torch.empty(m8, n8, dtype=torch.float16, device=dev)
+                f = lambda i: launchers.hip_gemm_a16w8_forward(o8, act, w8[i % nset8], s8)
+                for i in range(10):
+                    f(i)
+                ms = _events_ms(f, 100, torch)
+                b8 = n8 * k8 + 2.0 * n8 + 2.0 * m8 * k8 + 2.0 * m8 * n8
+                secondary.append({"workload": f"a16w8 decode M={m8} K={k8} N={n8} fp16",
+                                  "kernel": "gemm_wo_decode_lds_kernel" if m8 == 1 else "gemm_wo_panel_kernel",
+                                  "us_per_launch": round(ms * 1e3, 2),
+                                  "roofline": {"bound": "hbm", "achieved": round(b8 / (ms * 1e-3) / 1e9, 1),
+                                               "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                               "frac": round(b8 / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
             del w8
         Mr, Kr = 8192, 8192
         hs = [workloads.activations(Mr, Kr, torch.bfloat16, seed=5, outlier_frac=0.01).to(dev) for _ in range(3)]

@@ -391,18 +391,25 @@ static bool launch_a8_panel_t(A8W8Args& p, hipStream_t st) {
     if (p.M > 64 || p.N % 16 != 0 || p.K % 32 != 0 || p.K < 8 * 128 || p.lda % 16 != 0 || p.ldb % 16 != 0 ||
         ((uintptr_t)p.a % 16) != 0 || ((uintptr_t)p.b % 16) != 0)
         return false;
-    // rows per workgroup by chip fill, as in the weight-only panel kernel
-    int rt = 0;
+    // Rows per workgroup (16 rt) and 16-row activation blocks per pass (RT = 4 takes 2 or 4, RT = 2 takes 1 or
+    // 2, RT = 1 takes 1; fewer blocks than the rows allow make more, cheaper passes): the cheapest under the model of the weight-only panel kernel - a workgroup costs
+    // about eight loop iterations of start-up and wind-down plus ceil(KT * rt / 8) iterations, dearer with
+    // more row blocks, and the grid runs in rounds of 256 workgroups.
+    int rt = 0, mb = 1;
     double best = 0.0;
+    const int KT = (int)((p.K + 127) / 128);
+    static const double per_iter[5] = {0, 1.0, 1.2, 0, 1.8};
+    const int need = p.M <= 16 ? 1 : p.M <= 32 ? 2 : 4;
     for (int cand = 4; cand >= 1; cand >>= 1) {
         if (p.N % (16 * cand) != 0) continue;
-        const int t = p.N / (16 * cand);
-        const double fill = (double)t / (((t + 255) / 256) * 256);
-        const double score = fill * (cand == 4 ? 1.0 : cand == 2 ? 0.9 : 0.6);
-        if (score > best) { best = score; rt = cand; }
+        const int m_lo = cand == 4 ? 2 : 1;                   // the kernel is built for (4,4) (4,2) (2,2) (2,1) (1,1)
+        for (int m = cand == 1 ? 1 : cand; m >= m_lo; m >>= 1) {
+            if (m > need && m > m_lo) continue;               // more row blocks than there are rows
+            const int64_t wgs = (int64_t)(p.N / (16 * cand)) * ((p.M + m * 16 - 1) / (m * 16));
+            const double cost = (double)((wgs + 255) / 256) * (8.0 + (double)((KT * cand + 7) / 8) * per_iter[m]);
+            if (rt == 0 || cost < best) { best = cost; rt = cand; mb = m; }
+        }
     }
-    // 16-row activation blocks per pass: RT = 4 takes 2 or 4, RT = 2 takes 1 or 2, RT = 1 takes 1
-    const int mb = rt == 4 ? (p.M <= 32 ? 2 : 4) : rt == 2 ? (p.M <= 16 ? 1 : 2) : 1;
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const int tiles = p.N / (16 * rt);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes), block(512);

@@ -454,6 +454,34 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     }
 }
 
+// Rows per workgroup (64, 32 or 16, as rt = 4, 2, 1) and 16-row activation blocks per pass for M rows: the
+// cheapest under a coarse model of the kernel.  A workgroup pays a start-up and wind-down worth about eight
+// loop iterations, then ceil(KT * rt / 8) iterations whose cost grows with the row blocks per pass (MFMAs,
+// fragment reads, folds: measured 1 : 1.2 : 1.8 for 1, 2, 4 blocks), and the grid runs in rounds of 256
+// workgroups, one per CU.  Fewer rows per workgroup make more and shorter workgroups but allow fewer
+// activation rows per pass (mb <= rt, the LDS ring's limit), hence more passes over the weights; fewer
+// row blocks than the rows would allow make more, cheaper passes (the passes of a tile run on one XCD and
+// share the weights through its L2).
+// Measured on A16W8, N=4096: M=64 takes 12.6 us with 32 rows per workgroup and two passes, 27.5 us with 16
+// rows and four passes, 22.1 us with 64 rows and one pass of 64 workgroups.
+static int choose_rows(int wrows, int64_t M, int KT, int* mb_out) {
+    const int need = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    static const double per_iter[5] = {0, 1.0, 1.2, 0, 1.8};
+    int rt = 0;
+    double best = 0.0;
+    for (int cand = 4; cand >= 1; cand >>= 1) {
+        if (wrows % (16 * cand) != 0) continue;
+        for (int mb = cand < need ? cand : need; mb >= 1; mb >>= 1) {
+            const int64_t passes = (M + 16 * mb - 1) / (16 * mb);
+            const int64_t wgs = (int64_t)(wrows / (16 * cand)) * passes;
+            const int64_t rounds = (wgs + 255) / 256;
+            const double cost = (double)rounds * (8.0 + (double)((KT * cand + 7) / 8) * per_iter[mb]);
+            if (rt == 0 || cost < best) { best = cost; rt = cand; *mb_out = mb; }
+        }
+    }
+    return rt;
+}
+
 // Launches the panel kernel if the shape suits it; returns false otherwise.
 template <int WBITS, int ADT>
 static bool launch_panel_t(WoArgs& p, hipStream_t st) {
@@ -469,20 +497,8 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
                               (!p.zp || ((uintptr_t)p.zp % (8 * NH)) == 0);
         if (!tables16) return false;
     }
-    // rows per workgroup: 64, 32 or 16.  Fewer rows make more workgroups (a better fill of the 256
-    // CUs, counted in whole rounds) but share each activation slab between fewer waves and allow
-    // fewer activation rows per pass, hence the bonus for the larger ones.
-    int rt = 0;
-    double best = 0.0;
-    for (int cand = 4; cand >= 1; cand >>= 1) {
-        if (wrows % (16 * cand) != 0) continue;
-        const int t = wrows / (16 * cand);
-        const double fill = (double)t / (((t + 255) / 256) * 256);
-        const double score = fill * (cand == 4 ? 1.0 : cand == 2 ? 0.9 : 0.6);
-        if (score > best) { best = score; rt = cand; }
-    }
-    const int mb_max = rt;   // 16-row activation blocks per pass
-    const int mb = p.M <= 16 ? 1 : p.M <= 32 ? (mb_max >= 2 ? 2 : 1) : (mb_max >= 4 ? 4 : mb_max);
+    int mb = 1;
+    const int rt = choose_rows(wrows, p.M, (int)((p.K + 127) / 128), &mb);
     const int tiles = wrows / (16 * rt);
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);
