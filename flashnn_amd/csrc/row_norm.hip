@@ -39,7 +39,7 @@ template <int DT> __device__ __forceinline__ float round_dt(float v) {
     return bits_to_f32<DT>(f32_to_bits<DT>(rounded_f32(v)));
 }
 
-template <int DT, int NV, int OP>
+template <int DT, int NV, int OP, bool EARLY>
 __global__ __launch_bounds__(kRowThreads) void norm_vec_kernel(const NormArgs p) {
     __shared__ double redd[8];
     __shared__ float red[4];
@@ -47,9 +47,12 @@ __global__ __launch_bounds__(kRowThreads) void norm_vec_kernel(const NormArgs p)
     const v4u* xr = (const v4u*)(p.x + row * p.ldx);
     const int nvec = p.K >> 3;
     float n[NV][8];
-    // short rows: gamma and beta are requested together with the row, so that their latency is not paid
-    // a second time behind the first reduction (a single row is one chain of latencies)
-    constexpr bool PRE = NV <= 4;
+    // short rows, few of them (EARLY): gamma and beta are requested together with the row, so that their
+    // latency is not paid a second time behind the first reduction - a handful of rows is one chain of
+    // latencies (M=1, K=8192: 4.0 -> 3.6 us).  With thousands of rows the registers this takes cost more in
+    // resident waves than the latency is worth (layer norm 8192 x 8192: 59 -> 68 us), so the launcher keeps
+    // the late loads there.
+    constexpr bool PRE = EARLY && NV <= 4;
     float gpre[PRE ? NV : 1][8], bpre[PRE && OP != OP_RMS ? NV : 1][8];
     v4u xv[NV];
 #pragma unroll
@@ -207,7 +210,12 @@ static void launch_norm(const NormArgs& p, int64_t M, hipStream_t st) {
                      (OP == OP_RMS || ((uintptr_t)p.beta % 16) == 0);
     if (vec) {
         const int nv = (p.K / 8 + kRowThreads - 1) / kRowThreads;
-#define FNN_NORM(NV) norm_vec_kernel<DT, NV, OP><<<grid, block, 0, st>>>(p)
+        // up to four workgroups per CU are "few rows": every row is then resident at once either way
+#define FNN_NORM(NV)                                                                   \
+    do {                                                                               \
+        if (M <= 1024 && NV <= 4) norm_vec_kernel<DT, NV <= 4 ? NV : 1, OP, true><<<grid, block, 0, st>>>(p); \
+        else norm_vec_kernel<DT, NV, OP, false><<<grid, block, 0, st>>>(p);            \
+    } while (0)
         FNN_ROW_DISPATCH_NV(nv, FNN_NORM);
 #undef FNN_NORM
     } else {

@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kRowThreads) void dynamic_quant_any_kernel(
 }
 
 // ---------------------------------------------------------------- rmsnorm + quant
-template <int DT, int NV>
+template <int DT, int NV, bool EARLY>
 __global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_vec_kernel(
     int8_t* __restrict__ q, uint16_t* __restrict__ scale, const uint16_t* __restrict__ x,
     const void* __restrict__ gamma, int gamma_dtype, float eps, int K, int64_t ldx, int64_t ldq) {
@@ -87,9 +87,10 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_dquant_vec_kernel(
     const v4u* xr = (const v4u*)(x + row * ldx);
     const int nvec = K >> 3;
     float n[NV][8];
-    // short rows: gamma is requested together with the row, so that its latency is not paid a second
-    // time behind the first reduction (a single row is one chain of latencies)
-    constexpr bool PRE = NV <= 4;
+    // short rows, few of them (EARLY): gamma is requested together with the row, so that its latency is not
+    // paid a second time behind the first reduction (a handful of rows is one chain of latencies); with
+    // thousands of rows the registers are worth more as resident waves, and the launcher keeps the late load
+    constexpr bool PRE = EARLY && NV <= 4;
     float gpre[PRE ? NV : 1][8];
     v4u xv[NV];
 #pragma unroll
@@ -208,8 +209,12 @@ static void launch_rq(int8_t* q, uint16_t* scale, const uint16_t* x, const void*
     const dim3 grid((unsigned)M), block(kRowThreads);
     if (vec_ok(x, q, K, ldx, ldq) && ((uintptr_t)gamma % 16) == 0) {
         const int nv = (K / 8 + kRowThreads - 1) / kRowThreads;
-#define FNN_RQ(NV) \
-    rmsnorm_dquant_vec_kernel<DT, NV><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq)
+#define FNN_RQ(NV)                                                                                          \
+    do {                                                                                                    \
+        if (M <= 1024 && NV <= 4)                                                                           \
+            rmsnorm_dquant_vec_kernel<DT, NV <= 4 ? NV : 1, true><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq); \
+        else rmsnorm_dquant_vec_kernel<DT, NV, false><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);             \
+    } while (0)
         FNN_ROW_DISPATCH_NV(nv, FNN_RQ);
 #undef FNN_RQ
     } else {
