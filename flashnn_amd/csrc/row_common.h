@@ -11,14 +11,15 @@ namespace fnn {
 
 constexpr int kRowThreads = 256;
 
+// Block reductions over the four waves of a workgroup.  `red` serves ONE reduction per kernel (nothing
+// guards it against being written again while a slow wave still reads it): every kernel here reduces once
+// through each of its arrays.
 __device__ __forceinline__ float block_max(float v, float* red) {
     v = wave_max(v);
     const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) red[w] = v;
     __syncthreads();
-    float r = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-    return r;
+    return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 }
 
 __device__ __forceinline__ double block_sum(double v, double* red) {
@@ -26,9 +27,7 @@ __device__ __forceinline__ double block_sum(double v, double* red) {
     const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) red[w] = v;
     __syncthreads();
-    double r = (red[0] + red[1]) + (red[2] + red[3]);
-    __syncthreads();
-    return r;
+    return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
 // two sums at once (one pair of barriers)
@@ -40,7 +39,6 @@ __device__ __forceinline__ void block_sum2(double& a, double& b, double* red) {
     __syncthreads();
     a = (red[0] + red[1]) + (red[2] + red[3]);
     b = (red[4] + red[5]) + (red[6] + red[7]);
-    __syncthreads();
 }
 
 // Correctly rounded fp32 quotient x / s from r = RN(1/s) (one IEEE division per row):
@@ -59,6 +57,26 @@ template <int DT> __device__ __forceinline__ int quant_in_dtype(float x, float s
     const float t = rounded_f32(div_by(x, s, r));
     const float th = bits_to_f32<DT>(f32_to_bits<DT>(t));
     return (int)rintf(th);
+}
+
+// The same with the result left as an integer-valued float (for the packing below).
+template <int DT> __device__ __forceinline__ float quant_in_dtype_f(float x, float s, float r) {
+    const float t = rounded_f32(div_by(x, s, r));
+    return rintf(bits_to_f32<DT>(f32_to_bits<DT>(t)));
+}
+
+// Reciprocal to hand to div_by: 1/s, or 0 for an all-zero row, whose quotients then come out as 0
+// instead of 0 * inf (so the per-element test for s == 0 can go).
+__device__ __forceinline__ float quant_rcp(float s) { return s == 0.f ? 0.f : 1.0f / s; }
+
+// Byte j of w <- the integer-valued float r as int8, saturated to [-128, 127]: r + 128 is exact, lands in
+// [0, 255] as an unsigned byte, and v_cvt_pk_u8_f32 saturates, converts and inserts it in one instruction
+// (conversion, clamp and packing took five).  The finished dword still needs its sign bits flipped:
+// w ^ 0x80808080.  Only for the operators whose reference clamps (the norm + quant layers): plain dynamic
+// quantisation casts without a clamp, and a bf16 row whose scale rounded down does reach 128 there, which
+// the cast wraps to -128.
+__device__ __forceinline__ uint32_t put_biased_byte(float r, int j, uint32_t w) {
+    return __builtin_amdgcn_cvt_pk_u8_f32(r + 128.f, (uint32_t)j, w);
 }
 
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {

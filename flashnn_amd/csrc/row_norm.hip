@@ -137,17 +137,17 @@ __global__ __launch_bounds__(kRowThreads) void norm_vec_kernel(const NormArgs p)
         const uint32_t sbits = f32_to_bits<DT>(mx / 127.0f);
         const float s = bits_to_f32<DT>(sbits);
         if (threadIdx.x == 0) p.scale[row] = (uint16_t)sbits;
-        const float rcp = 1.0f / s;
+        const float rcp = quant_rcp(s);
         v2u* qr = (v2u*)((int8_t*)p.out + row * p.ldo);
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int idx = threadIdx.x + i * kRowThreads;
             if (idx < nvec) {
-                int o[8];
+                uint32_t w[2] = {0, 0};
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    o[j] = s == 0.f ? 0 : min(max(quant_in_dtype<DT>(n[i][j], s, rcp), -128), 127);
-                qr[idx] = v2u{pack4(o[0], o[1], o[2], o[3]), pack4(o[4], o[5], o[6], o[7])};
+                    w[j >> 2] = put_biased_byte(quant_in_dtype_f<DT>(n[i][j], s, rcp), j & 3, w[j >> 2]);
+                qr[idx] = v2u{w[0] ^ 0x80808080u, w[1] ^ 0x80808080u};
             }
         }
     }

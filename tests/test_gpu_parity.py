@@ -58,7 +58,10 @@ def test_dynamic_quant_outliers_and_zero_row():
 # -------------------------------------------------------------------- rmsnorm + quant
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(4, 128), (3, 32, 1024), (32, 8192), (7, 1000), (2, 20480), (3, 35584),
-                                   (2, 40960), (1, 41000)])
+                                   (2, 40960), (1, 41000),
+                                   # many short rows: the one-wave-per-row kernel (1, 2 and 4 vectors per lane,
+                                   # ragged last vector row, a row count that is no multiple of four)
+                                   (2050, 2048), (2049, 1000), (4096, 512), (2051, 264), (3, 700, 1024)])
 @pytest.mark.parametrize("gamma_dtype", [torch.float32, None])
 def test_rmsnorm_dquant_bit_exact(dtype, shape, gamma_dtype):
     torch.manual_seed(1)
