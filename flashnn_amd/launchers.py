@@ -31,29 +31,30 @@ def hip_rmsnorm_dquant_forward(x, weight, eps):
     _lib.require_gpu(x, weight)
     lib = _lib.load()
     y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
-    x_arg = x.reshape(-1, x.shape[-1])
-    if not x_arg.is_contiguous():
-        x_arg = x_arg.contiguous()
+    x_arg = _rows(x)
     M, N = x_arg.shape
-    scale = torch.empty((M,), dtype=x.dtype, device=x.device)
-    w = weight.detach()
-    if not w.is_contiguous():
-        w = w.contiguous()
-    assert w.numel() == N, "weight must have one entry per channel"
+    # one scale per row, already in the shape the operator returns (a contiguous block of M entries)
+    scale = torch.empty(x.shape[:-1], dtype=x.dtype, device=x.device)
+    w = _vec(weight, N, "weight")
     _lib.check(lib.fnn_rmsnorm_dquant(_lib.ptr(y), _lib.ptr(scale), _lib.ptr(x_arg), _lib.ptr(w),
                                       float(eps), M, N, N, N, _lib.dtype_code(x.dtype),
                                       _lib.dtype_code(w.dtype), _lib.current_stream(x.device)))
-    return y, scale.reshape(x.shape[:-1])
+    return y, scale
 
 
 def _rows(x):
+    """x as a contiguous matrix of rows (no view is made of what already is one: a view costs a microsecond)."""
+    if x.dim() == 2 and x.is_contiguous():
+        return x
     x_arg = x.reshape(-1, x.shape[-1])
     return x_arg if x_arg.is_contiguous() else x_arg.contiguous()
 
 
 def _vec(t, n, what):
-    t = t.detach().reshape(-1)
     assert t.numel() == n, f"{what} must have one entry per channel"
+    if t.dim() == 1 and t.is_contiguous():
+        return t            # only the address is taken: no detached view needed
+    t = t.detach().reshape(-1)
     return t if t.is_contiguous() else t.contiguous()
 
 
