@@ -514,7 +514,8 @@ static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
 
 static int check_args(const char* fn, const void* out, const void* a, const void* b, int64_t M,
                       int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc) {
-    if (!out || !a || !b) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
+    // an empty tensor has no address: pointers are only required when there is something to compute
+    if (M != 0 && N != 0 && (!out || !a || !b)) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
     if (M < 0 || N < 0 || K <= 0 || lda < K || ldb < K || ldc < N) {
         set_error("%s: bad shape M=%lld N=%lld K=%lld lda=%lld ldb=%lld ldc=%lld", fn, (long long)M,
                   (long long)N, (long long)K, (long long)lda, (long long)ldb, (long long)ldc);
@@ -553,7 +554,7 @@ static int gemm_a8w8_entry(const char* fn, void* out, const void* a, const void*
                            int tile_n, void* stream) {
     int rc = check_args(fn, out, a, b, M, N, K, lda, ldb, ldc);
     if (rc != FNN_OK) return rc;
-    if (!alpha_row || !alpha_col) { set_error("%s: null scale pointer", fn); return FNN_ERR_ARG; }
+    if (M != 0 && N != 0 && (!alpha_row || !alpha_col)) { set_error("%s: null scale pointer", fn); return FNN_ERR_ARG; }
     if (!is16(out_dtype)) { set_error("%s: Output type must be float16 or bfloat16", fn); return FNN_ERR_UNSUPPORTED; }
     if (!isflt(alpha_row_dtype) || !isflt(alpha_col_dtype)) { set_error("%s: bad scale type", fn); return FNN_ERR_UNSUPPORTED; }
     if (!valid_tile(tile_m, tile_n)) { set_error("%s: no such tile %dx%d", fn, tile_m, tile_n); return FNN_ERR_ARG; }

@@ -1050,7 +1050,8 @@ static int run_wo(const char* fn, void* out, const void* act, const void* qw, co
                   const void* bias, const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldw, int64_t ldc, int64_t group, int act_dtype, int out_dtype,
                   int scale_dtype, int zp_dtype, int bias_dtype, void* stream) {
-    if (!out || !act || !qw || !scale) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
+    // an empty tensor has no address: pointers are only required when there is something to compute
+    if (M != 0 && N != 0 && (!out || !act || !qw || !scale)) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
     if (M < 0 || N < 0 || K <= 0 || lda < K || ldw < K || ldc < N || group < 0) {
         set_error("%s: bad shape M=%lld N=%lld K=%lld lda=%lld ldw=%lld ldc=%lld group=%lld", fn,
                   (long long)M, (long long)N, (long long)K, (long long)lda, (long long)ldw,

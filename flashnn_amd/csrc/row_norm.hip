@@ -227,7 +227,8 @@ template <int OP>
 static int run_norm(const char* fn, void* out, void* scale, const void* x, const void* gamma,
                     const void* beta, float eps, int64_t M, int64_t K, int64_t ldx, int64_t ldo,
                     int x_dtype, int gb_dtype, void* stream) {
-    if (!out || !x || !gamma || (OP != OP_RMS && !beta) || (OP == OP_LNQ && !scale)) {
+    // an empty tensor has no address: pointers are only required when there are rows
+    if (M != 0 && (!out || !x || !gamma || (OP != OP_RMS && !beta) || (OP == OP_LNQ && !scale))) {
         set_error("%s: null pointer argument", fn);
         return FNN_ERR_ARG;
     }

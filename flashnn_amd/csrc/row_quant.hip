@@ -308,7 +308,8 @@ using namespace fnn;
 
 static int check_rows(const char* fn, const void* q, const void* scale, const void* x, int64_t M,
                       int64_t K, int64_t ldx, int64_t ldq, int x_dtype) {
-    if (!q || !scale || !x) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
+    // an empty tensor has no address: pointers are only required when there are rows
+    if (M != 0 && (!q || !scale || !x)) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
     if (M < 0 || K <= 0 || ldx < K || ldq < K) {
         set_error("%s: bad shape M=%lld K=%lld ldx=%lld ldq=%lld", fn, (long long)M, (long long)K,
                   (long long)ldx, (long long)ldq);
@@ -337,7 +338,7 @@ extern "C" int fnn_rmsnorm_dquant(void* q, void* scale, const void* x, const voi
                                   int gamma_dtype, void* stream) {
     int rc = check_rows("fnn_rmsnorm_dquant", q, scale, x, M, K, ldx, ldq, x_dtype);
     if (rc != FNN_OK) return rc;
-    if (!gamma) { set_error("fnn_rmsnorm_dquant: null gamma"); return FNN_ERR_ARG; }
+    if (M != 0 && !gamma) { set_error("fnn_rmsnorm_dquant: null gamma"); return FNN_ERR_ARG; }
     if (!isflt(gamma_dtype)) { set_error("fnn_rmsnorm_dquant: bad gamma type"); return FNN_ERR_UNSUPPORTED; }
     if (M == 0) return FNN_OK;
     hipStream_t st = (hipStream_t)stream;

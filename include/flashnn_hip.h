@@ -12,6 +12,8 @@
  *   - all pointers are device pointers unless stated; sizes/strides are in ELEMENTS;
  *   - matrices are row-major with an explicit leading dimension (row stride);
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *   - a call with no rows (M = 0) or no output channels (N = 0) is valid, launches nothing and
+ *     may pass NULL for its tensors (an empty tensor has no address);
  *   - return value: 0 ok, FNN_ERR_ARG (-1) bad argument, FNN_ERR_UNSUPPORTED (-2)
  *     shape/dtype not handled, FNN_ERR_HIP (-3) HIP runtime error.  After a non-zero
  *     return fnn_last_error() gives a thread-local, human-readable message.

@@ -728,3 +728,27 @@ def test_c_abi_row_strides(hip_lib):
     q_o, s_o = O.dynamic_quantize(O.to_np(x.cpu()), O.F16)
     assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(sc.cpu().numpy(), s_o)
     assert bool((qbuf[:, :8] == 5).all()) and bool((qbuf[:, 8 + 1024:] == 5).all())
+
+
+# ----------------------------------------------------------------------------- empty inputs
+def test_empty_inputs_through_the_operators():
+    """No rows (or no channels) is a valid call: nothing is launched, the outputs have the right shapes."""
+    x = torch.empty(0, 4096, dtype=torch.float16, device=DEV)
+    q, s = flashnn_amd.DynamicQuantize()(x)
+    assert q.shape == (0, 4096) and q.dtype == torch.int8 and s.shape == (0,) and s.dtype == torch.float16
+    w = _rand_i8((256, 4096), 51).to(DEV)
+    wscale = torch.rand(256, device=DEV).half()
+    out = flashnn_amd.GemmA8W8(torch.float16)(q, w, s, wscale)
+    assert out.shape == (0, 256) and out.dtype == torch.float16
+    out = flashnn_amd.GemmWeightOnly(torch.float16)(x, w, wscale)
+    assert out.shape == (0, 256)
+    mod = flashnn_amd.RMSNormDquant(4096).to(DEV)
+    q, s = mod(torch.empty(0, 4096, dtype=torch.bfloat16, device=DEV))
+    assert q.shape == (0, 4096) and s.shape == (0,) and s.dtype == torch.bfloat16
+    q, s = mod(torch.empty(2, 0, 4096, dtype=torch.bfloat16, device=DEV))
+    assert q.shape == (2, 0, 4096) and s.shape == (2, 0)
+    y = flashnn_amd.RMSNorm(4096).to(DEV)(torch.empty(0, 4096, dtype=torch.bfloat16, device=DEV))
+    assert y.shape == (0, 4096)
+    y = flashnn_amd.LayerNorm(4096).to(DEV)(torch.empty(0, 4096, dtype=torch.float16, device=DEV))
+    assert y.shape == (0, 4096)
+    torch.cuda.synchronize()

@@ -177,3 +177,19 @@ def test_tiled_entry_rejects_unknown_tiles(hip_lib):
     null = ctypes.c_void_p(0)
     rc = hip_lib.fnn_gemm_a8w8_tiled(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 0, 0, 0, 64, 64, null)
     assert rc == -1 and b"no such tile 64x64" in hip_lib.fnn_last_error()
+
+
+def test_empty_calls_need_no_addresses(hip_lib):
+    """M = 0 / N = 0 returns before anything is launched and accepts NULL tensors (an empty torch tensor
+    has data_ptr() == 0); with rows present the same NULLs are rejected."""
+    null = ctypes.c_void_p(0)
+    assert hip_lib.fnn_dynamic_quant(null, null, null, 0, 4096, 4096, 4096, 0, null) == 0
+    assert hip_lib.fnn_dynamic_quant(null, null, null, 1, 4096, 4096, 4096, 0, null) == -1
+    assert b"null pointer" in hip_lib.fnn_last_error()
+    assert hip_lib.fnn_rmsnorm_dquant(null, null, null, null, 1e-6, 0, 4096, 4096, 4096, 1, 2, null) == 0
+    assert hip_lib.fnn_layernorm(null, null, null, null, 1e-5, 0, 4096, 4096, 4096, 0, 0, null) == 0
+    assert hip_lib.fnn_gemm_a8w8(null, null, null, null, null, 0, 256, 4096, 4096, 4096, 256, 0, 0, 0, null) == 0
+    assert hip_lib.fnn_gemm_a8w8(null, null, null, null, null, 8, 0, 4096, 4096, 4096, 0, 0, 0, 0, null) == 0
+    assert hip_lib.fnn_gemm_a8w8(null, null, null, null, null, 8, 256, 4096, 4096, 4096, 256, 0, 0, 0, null) == -1
+    assert hip_lib.fnn_gemm_a16w8(null, null, null, null, null, null, 0, 256, 4096, 4096, 4096, 256, 0,
+                                  0, 0, 0, 0, 0, null) == 0
