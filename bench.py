@@ -30,8 +30,18 @@ PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA, published (5.0 POP/s)
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published (8 TB/s)
 
 
-def _events_ms(fn, iters, torch):
-    """Average duration of fn() over `iters` back-to-back calls, HIP events on the current stream."""
+def _events_ms(fn, iters, torch, preroll_s=0.04):
+    """Average duration of fn() over `iters` back-to-back calls, HIP events on the current stream.
+    The calls are preceded by an untimed pre-roll of the same call: host-side input generation between the
+    measurements leaves the device idle long enough for its clocks to drop, and a hundred launches of a
+    20 us kernel would otherwise be over before they have come back."""
+    t0 = time.perf_counter()
+    k = 0
+    while time.perf_counter() - t0 < preroll_s:
+        for _ in range(20):
+            fn(k)
+            k += 1
+        torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
