@@ -752,3 +752,38 @@ def test_empty_inputs_through_the_operators():
     y = flashnn_amd.LayerNorm(4096).to(DEV)(torch.empty(0, 4096, dtype=torch.float16, device=DEV))
     assert y.shape == (0, 4096)
     torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------ randomly drawn shapes
+@pytest.mark.parametrize("seed", range(40))
+def test_random_shapes_against_the_oracle(seed):
+    """Shapes, types and options drawn at random (fixed seeds) around the edges of the kernels' fast paths:
+    row counts either side of 16/32/64, channel counts that are and are not multiples of 32, K with every
+    kind of tail.  A8W8 bit-exact, weight-only within the stated tolerance."""
+    import random
+    rnd = random.Random(1000 + seed)
+    M = rnd.choice([1, 2, 5, 16, 17, 31, 32, 33, 40, 48, 63, 64, 65, 100, 129, 200, 260, 300, 513])
+    N = rnd.choice([16, 32, 48, 64, 80, 96, 144, 256, 272, 512, 528, 1024, 1040, 1920, 4096, 4112])
+    K = rnd.choice([32, 64, 96, 128, 160, 512, 544, 576, 608, 1024, 1056, 1088, 1120, 1152, 2048, 2080, 4096, 4128,
+                    1000, 72])
+    out_ty = rnd.choice([torch.float16, torch.bfloat16])
+    g = torch.Generator().manual_seed(seed)
+    a, b = _rand_i8((M, K), 2 * seed), _rand_i8((N, K), 2 * seed + 1)
+    ar = (torch.rand(M, generator=g) * 0.05).to(rnd.choice([torch.float16, torch.bfloat16, torch.float32]))
+    ac = (torch.rand(N, generator=g) * 0.05).to(rnd.choice([torch.float16, torch.bfloat16, torch.float32]))
+    out = flashnn_amd.GemmA8W8(out_ty)(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV))
+    want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.numpy(), b.numpy()), O.to_np(ar), O.to_np(ac), _tag(out_ty))
+    assert np.array_equal(out.float().cpu().numpy(), want), f"a8w8 M={M} N={N} K={K} {out_ty}"
+
+    bits = rnd.choice([8, 4])
+    M = rnd.choice([1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 48, 64, 65, 70, 100, 130])
+    N = rnd.choice([16, 32, 64, 96, 128, 144, 256, 512, 528, 1024, 2048, 2064, 4096])
+    K = rnd.choice([128, 256, 512, 1024, 1152, 2048, 4096, 1056, 1088, 1120, 640, 384])
+    group = rnd.choice([0, 0, 128, 128, 64, 32])
+    if group and K % group:
+        group = 0
+    act_ty = rnd.choice([torch.float16, torch.bfloat16])
+    scale_ty = rnd.choice([act_ty, act_ty, torch.float32]) if group == 0 else act_ty
+    case = _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp=rnd.random() < 0.6,
+                      with_bias=rnd.random() < 0.4, seed=seed)
+    _wo_check(*case, group, bits, act_ty)
