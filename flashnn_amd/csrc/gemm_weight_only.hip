@@ -506,17 +506,28 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     // Fill LDS in batches: all loads of a batch are issued before the first store, so a batch
     // costs one memory latency (a load-store loop would pay it once per element).
     constexpr int NT = kDecWaves * 64;
+    const int chunks = p.K / 8;   // 16-byte pieces per activation row
+    // the first batch of activations is asked for before the scale tables are filled, so that the two
+    // fills cost one memory latency between them, not one each (a decode launch is a handful of latencies)
+    v4u v_first[4];
+    {
+        const v4u* src = (const v4u*)p.act;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v_first[u] = src[min(u * NT + (int)threadIdx.x, chunks - 1)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
     if (p.scale_dtype == FNN_F16) fill_scales_lds<FNN_F16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
     else fill_scales_lds<FNN_BF16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
     {
-        const int chunks = p.K / 8;   // 16-byte pieces per activation row
         for (int m = 0; m < p.M; ++m) {
             const v4u* src = (const v4u*)((const uint16_t*)p.act + (int64_t)m * p.lda);
             v4u* dst = (v4u*)(a_lds + m * a_stride);
             for (int c0 = 0; c0 < chunks; c0 += 4 * NT) {
                 v4u v[4];
+                const bool first = m == 0 && c0 == 0;   // uniform
 #pragma unroll
-                for (int u = 0; u < 4; ++u) v[u] = src[min(c0 + u * NT + (int)threadIdx.x, chunks - 1)];
+                for (int u = 0; u < 4; ++u)
+                    v[u] = first ? v_first[u] : src[min(c0 + u * NT + (int)threadIdx.x, chunks - 1)];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int c = c0 + u * NT + threadIdx.x;
