@@ -93,20 +93,16 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     const int wm = wave & 1;
     const int wn = wave >> 1;
 
-    // Scales of the tile go to LDS as fp32, so that the epilogue needs no global loads.  They are asked
-    // for right behind the first copies of the ring (called from the prologues below): asked for first, their
-    // latency stood alone in front of every tile, about a microsecond and a half before the first copy was
-    // even issued.  The wait for them also waits for those copies, which the first barrier needs anyway.
-    auto stage_scales = [&]() {
-        if constexpr (MODE != OUT_I32) {
-            for (int e = threadIdx.x; e < BM + BN; e += 256) {
-                const bool is_row = e < BM;
-                const int idx = is_row ? min(m0 + e, p.M - 1) : min(n0 + e - BM, p.N - 1);
-                const float v = load_as_f32(is_row ? p.arow : p.acol, idx, is_row ? p.arow_dtype : p.acol_dtype);
-                if (is_row) sc_row[e] = v; else sc_col[e - BM] = v;
-            }
+    // Scales of the tile go to LDS as fp32 before anything else is in flight; the epilogue then
+    // needs no global loads.
+    if constexpr (MODE != OUT_I32) {
+        for (int e = threadIdx.x; e < BM + BN; e += 256) {
+            const bool is_row = e < BM;
+            const int idx = is_row ? min(m0 + e, p.M - 1) : min(n0 + e - BM, p.N - 1);
+            const float v = load_as_f32(is_row ? p.arow : p.acol, idx, is_row ? p.arow_dtype : p.acol_dtype);
+            if (is_row) sc_row[e] = v; else sc_col[e - BM] = v;
         }
-    };
+    }
 
     // copy plan: load j of this wave fills rows (j*NWAVES + wave)*8 .. +7; lane L writes slot (L & 7)
     // of row (L >> 3) of that group, which holds logical chunk (L & 7) ^ ((row >> 1) & 7)
@@ -253,7 +249,6 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         copy_b(sb0, 0);
         copy_a(sa0, 0);
         copy_b(sb1, 1);
-        stage_scales();
         wait_barrierB(true);
         read_frags(sa0, sb0, 0);
         copy_a(sa1, 1);
@@ -306,7 +301,6 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         copy_b(sb0, 0);
         copy_a(sa1, 1);
         copy_b(sb1, 1);
-        stage_scales();
         wait_barrier3(true);
         read_frags(sa0, sb0, 0);
         int j = 0;
