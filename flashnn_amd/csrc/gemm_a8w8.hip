@@ -482,6 +482,25 @@ static TileChoice choose_tile(int64_t M, int64_t N) {
     return c;
 }
 
+// With 256x192 tiles, the number of 192-wide tile columns to give a first launch when the rest is better done
+// by a second launch of 256x128 tiles, or 0.  A round of 256 workgroups takes one tile time however few of
+// them exist, so a last round that is mostly empty is expensive; the columns are then cut where the first
+// launch ends on a full round.  Costs in 256x192 tile times: a 256x128 tile takes 128/192/0.85 of one, the
+// second launch about 0.08 (its launch gap and start-up).
+static int split_columns_192(int64_t M, int64_t N) {
+    const int64_t tm = (M + 255) / 256, c = (N + 191) / 192;
+    const double single = (double)((tm * c + 255) / 256);
+    double best = single - 0.1;      // worth a second launch only from a tenth of a round
+    int best_c1 = 0;
+    for (int64_t c1 = c - 1; c1 >= 1 && c1 >= c - 64; --c1) {
+        const int64_t rem = N - 192 * c1;
+        const int64_t r1 = (tm * c1 + 255) / 256, r2 = (tm * ((rem + 127) / 128) + 255) / 256;
+        const double cost = (double)r1 + (double)r2 * (128.0 / 192.0 / 0.85) + 0.08;
+        if (cost < best) { best = cost; best_c1 = (int)c1; }
+    }
+    return best_c1;
+}
+
 template <int BM, int BN, int MODE>
 static void launch_mfma(A8W8Args& p, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -506,7 +525,24 @@ static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
     }
     TileChoice c = choose_tile(p.M, p.N);
     if (force_bm > 0) c = {force_bm, force_bn};
-    if (c.bm == 256 && c.bn == 192) launch_mfma<256, 192, MODE>(p, st);
+    if (c.bm == 256 && c.bn == 192) {
+        const int c1 = force_bm == 0 ? split_columns_192(p.M, p.N) : 0;
+        if (c1 > 0) {
+            // columns [0, 192 c1) in 192-wide tiles, the rest in 128-wide ones
+            A8W8Args q = p;
+            q.N = 192 * c1;
+            launch_mfma<256, 192, MODE>(q, st);
+            const int64_t n_off = q.N;
+            q = p;
+            q.N = p.N - (int)n_off;
+            q.b = p.b + n_off * p.ldb;
+            q.out = (char*)p.out + n_off * (MODE == OUT_I32 ? 4 : 2);
+            if (p.acol) q.acol = (const char*)p.acol + n_off * (p.acol_dtype == FNN_F32 ? 4 : 2);
+            launch_mfma<256, 128, MODE>(q, st);
+        } else {
+            launch_mfma<256, 192, MODE>(p, st);
+        }
+    }
     else if (c.bm == 256 && c.bn == 128) launch_mfma<256, 128, MODE>(p, st);
     else if (c.bm == 64 && c.bn == 128) launch_mfma<64, 128, MODE>(p, st);
     else launch_mfma<128, 128, MODE>(p, st);
