@@ -7,7 +7,8 @@
 //     copied global -> LDS with direct-to-LDS 16-byte loads (no VGPR staging) into one of
 //     two static LDS stages while the MFMAs of the previous slab run;
 //   * both operands are K-contiguous, so a lane's 16-byte LDS read is directly one
-//     v_mfma_i32_32x32x32_i8 operand.  The 16-byte chunks of each 128-byte LDS row are
+//     v_mfma_i32_16x16x64_i8 operand (with random operands the device sustains a fifth more of
+//     these than of the 32x32x32 shape: 4.0 against 3.35 POP/s).  The 16-byte chunks of each 128-byte LDS row are
 //     XOR-swizzled with (row & 7) so that the 8 lanes served together hit 8 distinct
 //     bank groups.  The swizzle is applied on the global side of the copy (the LDS side
 //     of a direct-to-LDS load is linear in the lane id);
@@ -39,16 +40,13 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
 
 // ------------------------------------------------------------------ main MFMA kernel
-// K % 128 == 0, K >= 512.  K is walked in slabs of 128 bytes: every row piece a copy fetches
+// K % 32 == 0, K >= 512.  K is walked in slabs of 128 bytes: every row piece a copy fetches
 // is one full 128-byte line, which is what the L2 -> LDS path needs to run at speed (64-byte
-// pieces reach little more than half the rate).  The LDS holds a ring of three stages for the a-rows
-// (copied two slabs ahead, a third per k-step) and, for the 256x192 tile, two for the b-rows (one slab
-// ahead): 3*BM + 2*BN rows of 128 bytes = 144 KB.  The smaller tiles have room for a third b-stage
-// and copy the b-rows two slabs ahead as well (3 to 20 % faster).  There is one barrier per slab, at
-// the start of its LAST k-step: by then every fragment of the slab is in registers, so both of
-// its stages are free and are re-armed right after the barrier, and the barrier publishes the
-// next slab, whose first fragments are read under the last MFMAs of the current one.
-// Fragments are double-buffered in registers; LDS reads and MFMAs alternate one to one.
+// pieces reach little more than half the rate).  The LDS holds a ring of stages per operand.  The
+// 256x192 tile has three for the b-rows (the weights, streamed from HBM, copied two slabs ahead) and
+// two for the a-rows (L2 hits after their first use, copied one slab ahead): 2*BM + 3*BN rows of 128
+// bytes = 136 KB.  The smaller tiles have room for three stages of both and copy both two slabs ahead
+// (3 to 20 % faster).  There is one barrier per slab; the loop around it is described where it is written.
 // Chunk c (16 bytes) of LDS row r is stored at slot c ^ ((r >> 1) & 7).  A 16-byte LDS read serves
 // 16 lanes (16 consecutive rows, same chunk) per cycle out of 64 banks = 256 bytes; two rows fill
 // that period, so rows of equal parity must land in 8 different slots.  (r & 7 instead gives
@@ -59,7 +57,9 @@ template <int BM, int BN, int MODE>
 __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     constexpr int NWAVES = 4;
     constexpr int WTM = BM / 2, WTN = BN / 2;
-    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int FM = WTM / 16, FN = WTN / 16;   // 16x16 fragments per wave tile
+    constexpr int HN = FN / 2;
+    static_assert(WTM % 16 == 0 && WTN % 32 == 0, "wave tile must split into 16-row fragments, the weight rows in two halves");
     constexpr int NLA = BM / (8 * NWAVES);   // a wave-load covers 8 rows of 128 bytes
     constexpr int NLB = BN / (8 * NWAVES);
     static_assert(BM % (8 * NWAVES) == 0 && BN % (8 * NWAVES) == 0, "tile rows must split evenly");
@@ -148,52 +148,65 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
                                                  (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
 
-    // read plan: lane reads row (lane & 31) of a fragment, logical chunk 2*ks + (lane >> 5)
-    const int frow = lane & 31;
-    const int hsel = lane >> 5;
-    int rd_off[4];
+    // read plan: a fragment is 16 rows x 64 bytes of K; lane reads row (lane & 15), logical chunk
+    // 4*kq + (lane >> 4) of chunk kq (0 or 1) of the slab
+    const int frow = lane & 15;
+    const int csel = lane >> 4;
+    int rd_off[2];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) rd_off[ks] = frow * BK + (((2 * ks + hsel) ^ ((frow >> 1) & 7)) * 16);
+    for (int kq = 0; kq < 2; ++kq) rd_off[kq] = frow * BK + (((4 * kq + csel) ^ ((frow >> 1) & 7)) * 16);
     const int a_base = wm * WTM * BK;
     const int b_base = wn * WTN * BK;
 
-    v16i acc[FN][FM];
+    v4i acc[FN][FM];
 #pragma unroll
     for (int i = 0; i < FN; ++i)
 #pragma unroll
-        for (int j = 0; j < FM; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+        for (int j = 0; j < FM; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-    v4i wf[2][FN], af[2][FM];   // fragment double buffer, indexed by k-step parity
-    auto read_frags = [&](const char* sa, const char* sb, int ks) {
+    // Fragments of both 64-byte chunks of a slab live in registers, indexed by chunk.  The NRD reads of
+    // a chunk are issued in two parts, in the order the MFMAs need them: first half of the weight
+    // fragments, the activation fragments, second half of the weight fragments.
+    v4i wf[2][FN], af[2][FM];
+    constexpr int NRD = FN + FM, NRA = (NRD + 1) / 2;
+    auto read_part = [&](const char* sa, const char* sb, int kq, int part) {
 #pragma unroll
-        for (int i = 0; i < FN; ++i) wf[ks & 1][i] = *(const v4i*)(sb + b_base + i * 32 * BK + rd_off[ks]);
-#pragma unroll
-        for (int j = 0; j < FM; ++j) af[ks & 1][j] = *(const v4i*)(sa + a_base + j * 32 * BK + rd_off[ks]);
+        for (int r = 0; r < NRD; ++r) {
+            if ((r >= NRA) != (part == 1)) continue;
+            if (r < HN) wf[kq][r] = *(const v4i*)(sb + b_base + r * 16 * BK + rd_off[kq]);
+            else if (r < HN + FM) af[kq][r - HN] = *(const v4i*)(sa + a_base + (r - HN) * 16 * BK + rd_off[kq]);
+            else wf[kq][r - FM] = *(const v4i*)(sb + b_base + (r - FM) * 16 * BK + rd_off[kq]);
+        }
     };
-    auto mfmas = [&](int par) {
+    // one phase of MFMAs: half h of the weight fragments of chunk kq against all activation fragments
+    auto mfmas = [&](int kq, int h) {
 #pragma unroll
-        for (int i = 0; i < FN; ++i)
+        for (int i = h * HN; i < (h + 1) * HN; ++i)
 #pragma unroll
             for (int j = 0; j < FM; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[par][i], af[par][j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[kq][i], af[kq][j], acc[i][j], 0, 0, 0);
     };
-    // ask the scheduler for: MFMA, 2 LDS reads, MFMA, 2 LDS reads, ... then the remaining MFMAs.
-    // The reads of the next k-step are all issued under the first few MFMAs, which leaves their
-    // latency the rest of the k-step (8 MFMAs = 256 cycles) to elapse.
-    auto interleave = [&]() {
-        constexpr int NRD = FN + FM;
+    // ask the scheduler for: 2 MFMAs, 1 LDS read, 2 MFMAs, 1 LDS read, ... then the remaining MFMAs, so
+    // that the reads of a phase are spread over its first half and have its second half to return
+    auto interleave = [&](int part) {
+        constexpr int NM = HN * FM;
+        constexpr int R0 = NRA, R1 = NRD - NRA;
+        constexpr int PER = NM >= 2 * R0 ? 2 : 1;
+        if (part == 0) {
 #pragma unroll
-        for (int q = 0; q < NRD / 2; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            for (int q = 0; q < R0; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            if constexpr (NM - PER * R0 > 0) __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * R0, 0);
+        } else {
+#pragma unroll
+            for (int q = 0; q < R1; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            if constexpr (NM - PER * R1 > 0) __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * R1, 0);
         }
-        if constexpr (NRD % 2 == 1) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, FN * FM - (NRD + 1) / 2, 0);
     };
     // Wait until at most `newer` of this wave's copies are outstanding and its LDS reads have
     // returned, then cross the workgroup barrier.  A bare s_barrier: __syncthreads() would add a
@@ -207,121 +220,145 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         asm volatile("" ::: "memory");
     };
 
-    // K = 128 * (KT - 1) + 32 * last_steps: the last slab may hold fewer than four k-steps
+    // K = 128 * (KT - 1) + 32 * last_steps: the last slab may hold fewer than 128 bytes per row
     const int KT = (p.K + BK - 1) / BK;
     const int last_steps = (p.K - (KT - 1) * BK) / 32;
     const int tail_fix = lchunk * 16 >= last_steps * 32 ? -(lchunk * 16) : 0;
-    // the slabs 0 .. KT-2 run through the ring; the last one has no successor to prefetch and is
-    // worked off after the loops, from whichever stages it landed in
-    auto last_slab = [&](const char* sa, const char* sb) {
+    // The last slab, in stages (ca, cb), after its barrier; chunk 1 of the slab before it is in registers.
+    // Where K ends in the middle of a 64-byte chunk, the lanes that hold its second half feed zeros
+    // as weights (the bytes they read exist, but belong to no product).
+    auto mask_half = [&](int kq) {
+        if (csel >= 2) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            if (ks < last_steps) {
-                if (ks + 1 < last_steps) read_frags(sa, sb, ks + 1);
-                mfmas(ks & 1);
-            }
+            for (int i = 0; i < FN; ++i) wf[kq][i] = v4i{0, 0, 0, 0};
         }
     };
-    // One slab = four k-steps; slab j lives in (sa, sb), slab j+1 in (nsa, nsb).  Copies of slab j+2
-    // are issued in three parts during k-steps 0..2 into the stage freed at the previous barrier
-    // (issued in one burst they block the wave's MFMAs behind them).  The barrier at the start of the
-    // last k-step publishes slab j+1, whose first fragments are read under the last MFMAs of slab j.
+    auto last_iter = [&](const char* ca, const char* cb) {
+        read_part(ca, cb, 0, 0);
+        mfmas(1, 0);
+        read_part(ca, cb, 0, 1);
+        mfmas(1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (last_steps == 1) mask_half(0);
+        if (last_steps >= 3) {
+            read_part(ca, cb, 1, 0);
+            read_part(ca, cb, 1, 1);
+        }
+        mfmas(0, 0);
+        mfmas(0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (last_steps >= 3) {
+            if (last_steps == 3) mask_half(1);
+            mfmas(1, 0);
+            mfmas(1, 1);
+        }
+    };
+    // A slab is two 64-byte chunks of K; a chunk's MFMAs run in two phases (one half of the weight
+    // fragments each), so an iteration has four phases of HN*FM MFMAs.  Iteration i starts with the one
+    // barrier: it publishes slab i and frees the stages of slab i-1, every read of which was issued
+    // in the previous iteration.  Phases A and B multiply chunk 1 of slab i-1 (in registers) while chunk 0
+    // of slab i is read; phases C and D multiply that chunk 0 while chunk 1 is read.  The reads are so
+    // spread evenly: (FN+FM)/2 per phase.  The freed stages take the slab two ahead, copied in parts
+    // over the phases (issued in one burst the copies block the wave's MFMAs behind them).
+#define FNN_PHASE(ca, cb, kq, part, copies, mq, mh)  \
+    read_part(ca, cb, kq, part);                      \
+    copies;                                           \
+    mfmas(mq, mh);                                    \
+    interleave(part);                                 \
+    __builtin_amdgcn_sched_barrier(0);
     if constexpr (BDEEP) {
+        // a-rows in two stages: slab i+1 goes into the a-stage of slab i-1, in one burst after the barrier
+        // (it must be complete at the next one); b-rows in three: slab i+2 follows in three parts, and only
+        // those parts may be in flight at the next barrier
         auto wait_barrierB = [&](bool keep) { wait_barrier_n(keep, std::integral_constant<int, NLB>{}); };
-        auto slabB = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fb, int j, bool steady) {
-            const bool more = steady || j + 2 < KT;
-            const int fix = !steady && j + 2 == KT - 1 ? tail_fix : 0;
-#pragma unroll
-            for (int ks = 0; ks < 3; ++ks) {
-                read_frags(sa, sb, ks + 1);
-                if (more) copy_b_part(fb, j + 2, ks, fix);
-                mfmas(ks & 1);
-                interleave();
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            wait_barrierB(more);
-            read_frags(nsa, nsb, 0);
-            if (more) copy_a(sa, j + 2, fix);
-            mfmas(1);
-            interleave();
-            __builtin_amdgcn_sched_barrier(0);
+        auto iterB = [&](const char* ca, const char* cb, char* fa, char* fb, int i, bool steady) {
+            const bool more = steady || i + 2 < KT;
+            const int fix_a = !steady && i + 1 == KT - 1 ? tail_fix : 0;
+            const int fix_b = !steady && i + 2 == KT - 1 ? tail_fix : 0;
+            wait_barrierB(true);
+            FNN_PHASE(ca, cb, 0, 0, copy_a(fa, i + 1, fix_a), 1, 0)
+            FNN_PHASE(ca, cb, 0, 1, if (more) copy_b_part(fb, i + 2, 0, fix_b), 1, 1)
+            FNN_PHASE(ca, cb, 1, 0, if (more) copy_b_part(fb, i + 2, 1, fix_b), 0, 0)
+            FNN_PHASE(ca, cb, 1, 1, if (more) copy_b_part(fb, i + 2, 2, fix_b), 0, 1)
         };
         copy_b(sb0, 0);
         copy_a(sa0, 0);
         copy_b(sb1, 1);
         wait_barrierB(true);
-        read_frags(sa0, sb0, 0);
+        read_part(sa0, sb0, 0, 0);
+        read_part(sa0, sb0, 0, 1);
         copy_a(sa1, 1);
-        int j = 0;
+        copy_b_part(sb2, 2, 0);
+        FNN_PHASE(sa0, sb0, 1, 0, copy_b_part(sb2, 2, 1), 0, 0)
+        FNN_PHASE(sa0, sb0, 1, 1, copy_b_part(sb2, 2, 2), 0, 1)
+        int i = 1;
         // (the steady loop stops one slab earlier when the last slab is partial: its copies need the fix)
-        for (; j + 8 + (last_steps < 4) <= KT; j += 6) {
-            slabB(sa0, sb0, sa1, sb1, sb2, j, true);
-            slabB(sa1, sb1, sa0, sb2, sb0, j + 1, true);
-            slabB(sa0, sb2, sa1, sb0, sb1, j + 2, true);
-            slabB(sa1, sb0, sa0, sb1, sb2, j + 3, true);
-            slabB(sa0, sb1, sa1, sb2, sb0, j + 4, true);
-            slabB(sa1, sb2, sa0, sb0, sb1, j + 5, true);
+        for (; i + 8 + (last_steps < 4) <= KT; i += 6) {
+            iterB(sa1, sb1, sa0, sb0, i, true);
+            iterB(sa0, sb2, sa1, sb1, i + 1, true);
+            iterB(sa1, sb0, sa0, sb2, i + 2, true);
+            iterB(sa0, sb1, sa1, sb0, i + 3, true);
+            iterB(sa1, sb2, sa0, sb1, i + 4, true);
+            iterB(sa0, sb0, sa1, sb2, i + 5, true);
         }
-        for (; j < KT - 1; j += 6) {
-            slabB(sa0, sb0, sa1, sb1, sb2, j, false);
-            if (j + 2 < KT) slabB(sa1, sb1, sa0, sb2, sb0, j + 1, false);
-            if (j + 3 < KT) slabB(sa0, sb2, sa1, sb0, sb1, j + 2, false);
-            if (j + 4 < KT) slabB(sa1, sb0, sa0, sb1, sb2, j + 3, false);
-            if (j + 5 < KT) slabB(sa0, sb1, sa1, sb2, sb0, j + 4, false);
-            if (j + 6 < KT) slabB(sa1, sb2, sa0, sb0, sb1, j + 5, false);
+        for (; i < KT - 1; i += 6) {
+            iterB(sa1, sb1, sa0, sb0, i, false);
+            if (i + 1 < KT - 1) iterB(sa0, sb2, sa1, sb1, i + 1, false);
+            if (i + 2 < KT - 1) iterB(sa1, sb0, sa0, sb2, i + 2, false);
+            if (i + 3 < KT - 1) iterB(sa0, sb1, sa1, sb0, i + 3, false);
+            if (i + 4 < KT - 1) iterB(sa1, sb2, sa0, sb1, i + 4, false);
+            if (i + 5 < KT - 1) iterB(sa0, sb0, sa1, sb2, i + 5, false);
         }
+        wait_barrierB(false);
         const int lb = (KT - 1) % 3;
-        last_slab((KT - 1) & 1 ? sa1 : sa0, lb == 0 ? sb0 : lb == 1 ? sb1 : sb2);
+        last_iter((KT - 1) & 1 ? sa1 : sa0, lb == 0 ? sb0 : lb == 1 ? sb1 : sb2);
     } else {
-        // three stages each: a(j+2) and b(j+2) are both copied in parts during k-steps 0..2 of slab j,
-        // into the stages freed at the previous barrier; at the barrier only they may be in flight
+        // three stages each: slab i+2 of both operands goes into the stages of slab i-1 in three parts
+        // during phases A..C; at the next barrier only those parts may be in flight
         auto wait_barrier3 = [&](bool keep) { wait_barrier_n(keep, std::integral_constant<int, NLA + NLB>{}); };
-        auto slab3 = [&](char* sa, char* sb, const char* nsa, const char* nsb, char* fa, char* fb, int j,
-                         bool steady) {
-            const bool more = steady || j + 2 < KT;
-            const int fix = !steady && j + 2 == KT - 1 ? tail_fix : 0;
-#pragma unroll
-            for (int ks = 0; ks < 3; ++ks) {
-                read_frags(sa, sb, ks + 1);
-                if (more) {
-                    copy_a_part(fa, j + 2, ks, fix);
-                    copy_b_part(fb, j + 2, ks, fix);
-                }
-                mfmas(ks & 1);
-                interleave();
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            wait_barrier3(more);
-            read_frags(nsa, nsb, 0);
-            mfmas(1);
-            interleave();
-            __builtin_amdgcn_sched_barrier(0);
+        auto iter3 = [&](const char* ca, const char* cb, char* fa, char* fb, int i, bool steady) {
+            const bool more = steady || i + 2 < KT;
+            const int fix = !steady && i + 2 == KT - 1 ? tail_fix : 0;
+            wait_barrier3(true);
+            FNN_PHASE(ca, cb, 0, 0, if (more) { copy_a_part(fa, i + 2, 0, fix); copy_b_part(fb, i + 2, 0, fix); }, 1, 0)
+            FNN_PHASE(ca, cb, 0, 1, if (more) { copy_a_part(fa, i + 2, 1, fix); copy_b_part(fb, i + 2, 1, fix); }, 1, 1)
+            FNN_PHASE(ca, cb, 1, 0, if (more) { copy_a_part(fa, i + 2, 2, fix); copy_b_part(fb, i + 2, 2, fix); }, 0, 0)
+            FNN_PHASE(ca, cb, 1, 1, , 0, 1)
         };
         copy_a(sa0, 0);
         copy_b(sb0, 0);
         copy_a(sa1, 1);
         copy_b(sb1, 1);
         wait_barrier3(true);
-        read_frags(sa0, sb0, 0);
-        int j = 0;
-        for (; j + 5 + (last_steps < 4) <= KT; j += 3) {
-            slab3(sa0, sb0, sa1, sb1, sa2, sb2, j, true);
-            slab3(sa1, sb1, sa2, sb2, sa0, sb0, j + 1, true);
-            slab3(sa2, sb2, sa0, sb0, sa1, sb1, j + 2, true);
+        read_part(sa0, sb0, 0, 0);
+        read_part(sa0, sb0, 0, 1);
+        copy_a_part(sa2, 2, 0);
+        copy_b_part(sb2, 2, 0);
+        copy_a_part(sa2, 2, 1);
+        copy_b_part(sb2, 2, 1);
+        FNN_PHASE(sa0, sb0, 1, 0, { copy_a_part(sa2, 2, 2); copy_b_part(sb2, 2, 2); }, 0, 0)
+        FNN_PHASE(sa0, sb0, 1, 1, , 0, 1)
+        int i = 1;
+        for (; i + 5 + (last_steps < 4) <= KT; i += 3) {
+            iter3(sa1, sb1, sa0, sb0, i, true);
+            iter3(sa2, sb2, sa1, sb1, i + 1, true);
+            iter3(sa0, sb0, sa2, sb2, i + 2, true);
         }
-        for (; j < KT - 1; j += 3) {
-            slab3(sa0, sb0, sa1, sb1, sa2, sb2, j, false);
-            if (j + 2 < KT) slab3(sa1, sb1, sa2, sb2, sa0, sb0, j + 1, false);
-            if (j + 3 < KT) slab3(sa2, sb2, sa0, sb0, sa1, sb1, j + 2, false);
+        for (; i < KT - 1; i += 3) {
+            iter3(sa1, sb1, sa0, sb0, i, false);
+            if (i + 1 < KT - 1) iter3(sa2, sb2, sa1, sb1, i + 1, false);
+            if (i + 2 < KT - 1) iter3(sa0, sb0, sa2, sb2, i + 2, false);
         }
+        wait_barrier3(false);
         const int ls = (KT - 1) % 3;
-        last_slab(ls == 0 ? sa0 : ls == 1 ? sa1 : sa2, ls == 0 ? sb0 : ls == 1 ? sb1 : sb2);
+        last_iter(ls == 0 ? sa0 : ls == 1 ? sa1 : sa2, ls == 0 ? sb0 : ls == 1 ? sb1 : sb2);
     }
+#undef FNN_PHASE
 
     // ---- epilogue ----
-    // acc[i][j][r]: n = wn0 + i*32 + 8*(r/4) + 4*(lane>>5) + (r&3),  m = wm0 + j*32 + (lane&31).
-    // A lane owns 4 consecutive n of ONE row, so storing straight from registers would touch 32
-    // rows per instruction with 16 bytes each.  Instead every wave transposes its sub-tile through
+    // acc[i][j][r]: n = wn0 + i*16 + 4*(lane>>4) + r,  m = wm0 + j*16 + (lane&15).
+    // A lane owns 4 consecutive n of ONE row, so storing straight from registers would touch 16
+    // rows per instruction with 8 bytes each.  Instead every wave transposes its sub-tile through
     // LDS (one ring stage per wave, free now) 64 rows at a time and writes whole rows:
     // 16 bytes per lane, consecutive lanes on consecutive addresses.
     const int wm0 = m0 + wm * WTM;
@@ -330,30 +367,27 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         const bool vec_ok = (p.ldc & 3) == 0;
 #pragma unroll
         for (int j = 0; j < FM; ++j) {
-            const int m = wm0 + j * 32 + frow;
+            const int m = wm0 + j * 16 + frow;
 #pragma unroll
             for (int i = 0; i < FN; ++i) {
+                const int n = wn0 + i * 16 + 4 * csel;
+                if (m >= p.M || n >= p.N) continue;
+                int32_t* o = (int32_t*)p.out + (int64_t)m * p.ldc + n;
+                if (n + 3 < p.N && vec_ok) {
+                    *(v4i*)o = acc[i][j];
+                } else {
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int n = wn0 + i * 32 + 8 * g + 4 * hsel;
-                    if (m >= p.M || n >= p.N) continue;
-                    int32_t* o = (int32_t*)p.out + (int64_t)m * p.ldc + n;
-                    if (n + 3 < p.N && vec_ok) {
-                        *(v4i*)o = v4i{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
-                                       acc[i][j][4 * g + 3]};
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (n + e < p.N) o[e] = acc[i][j][4 * g + e];
-                    }
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < p.N) o[e] = acc[i][j][e];
                 }
             }
         }
     } else {
         constexpr int TSTRIDE = WTN * 2 + 16;      // bytes per staged row; the pad staggers the banks
         constexpr int PR = WTN * 2 / 16;           // 16-byte pieces per row
-        constexpr int RC = FM >= 2 ? 2 : 1;        // 32-row fragments staged at a time
-        static_assert(RC * 32 * TSTRIDE <= BN * BK && RC * 32 * TSTRIDE <= BM * BK, "transpose buffer must fit a stage");
+        constexpr int RC = FM >= 4 ? 4 : FM;       // 16-row fragments staged at a time
+        static_assert(FM % RC == 0, "staging walks whole groups of fragments");
+        static_assert(RC * 16 * TSTRIDE <= BN * BK && RC * 16 * TSTRIDE <= BM * BK, "transpose buffer must fit a stage");
         char* tbuf = wave == 0 ? sa0 : wave == 1 ? sa1 : wave == 2 ? (BDEEP ? sb1 : sa2) : sb0;
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0x0070);   // all copies and LDS reads of this wave are done
@@ -365,36 +399,33 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
 #pragma unroll
             for (int jj = 0; jj < RC; ++jj) {
                 const int j = jc + jj;
-                const float ar = sc_row[wm * WTM + j * 32 + frow];
+                const float ar = sc_row[wm * WTM + j * 16 + frow];
 #pragma unroll
                 for (int i = 0; i < FN; ++i) {
+                    const int nl = i * 16 + 4 * csel;   // column within the wave tile
+                    const v4f ac = *(const v4f*)&sc_col[wn * WTN + nl];
+                    float v[4];
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int nl = i * 32 + 8 * g + 4 * hsel;   // column within the wave tile
-                        const v4f ac = *(const v4f*)&sc_col[wn * WTN + nl];
-                        float v[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = ((float)acc[i][j][4 * g + e] * ar) * ac[e];
-                        uint32_t lo, hi;
-                        if constexpr (MODE == OUT_BF16) {
-                            lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2bf));
-                            hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2bf));
-                        } else {
-                            lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2h));
-                            hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2h));
-                        }
-                        *(v2u*)(tbuf + (jj * 32 + frow) * TSTRIDE + nl * 2) = v2u{lo, hi};
+                    for (int e = 0; e < 4; ++e) v[e] = ((float)acc[i][j][e] * ar) * ac[e];
+                    uint32_t lo, hi;
+                    if constexpr (MODE == OUT_BF16) {
+                        lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2bf));
+                        hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2bf));
+                    } else {
+                        lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2h));
+                        hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2h));
                     }
+                    *(v2u*)(tbuf + (jj * 16 + frow) * TSTRIDE + nl * 2) = v2u{lo, hi};
                 }
             }
-            // rows jc*32 .. jc*32+63 of the wave tile are staged; write them out row by row
+            // rows jc*16 .. jc*16 + RC*16 - 1 of the wave tile are staged; write them out row by row
 #pragma unroll
-            for (int it = 0; it < (RC * 32 * PR + 63) / 64; ++it) {
+            for (int it = 0; it < (RC * 16 * PR + 63) / 64; ++it) {
                 const int e = it * 64 + lane;
                 const int row = e / PR, c = e % PR;
-                if (e < RC * 32 * PR) {
+                if (e < RC * 16 * PR) {
                     const v4u val = *(const v4u*)(tbuf + row * TSTRIDE + c * 16);
-                    const int m = wm0 + jc * 32 + row;
+                    const int m = wm0 + jc * 16 + row;
                     const int n = wn0 + c * 8;
                     if (m < p.M && n < p.N) {
                         uint16_t* o = (uint16_t*)p.out + (int64_t)m * p.ldc + n;
