@@ -155,7 +155,7 @@ def main():
     sustained = {}
     for label, rnd in (("random_operand_bytes", 1), ("constant_operands", 0)):
         rate = ctypes.c_double(0.0)
-        _lib.check(_lib.load().fnn_debug_mfma_rate(_lib.ptr(sink), rnd, 20000, 40, ctypes.byref(rate),
+        _lib.check(_lib.load().fnn_debug_mfma_rate(_lib.ptr(sink), rnd, 2000, 40, ctypes.byref(rate),
                                                    _lib.current_stream(torch.device(dev))))
         sustained[label] = round(rate.value, 1)
     roofline["mfma_only_sustained"] = dict(sustained, unit="TOP/s")

@@ -501,7 +501,11 @@ struct TileChoice { int bm, bn; };
 // Pick the tile whose last, partly filled round of workgroups costs least on 256 CUs.
 static TileChoice choose_tile(int64_t M, int64_t N) {
     static const struct { int bm, bn; double eff; } cand[] = {
-        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.72}, {64, 128, 0.45}};   // throughput per tile area, measured at K = N = 8192 (at smaller shapes the smaller tiles come closer; a 64x128 tile takes 0.8 of the time of a 128x128 one, so it pays where it doubles the workgroups without adding a round)
+        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.72}, {64, 128, 0.62}};
+    // eff = throughput per tile area relative to the 256x192 tile, measured with every round full.  It
+    // depends on the shape: the 256x128 tile reaches 1.0 at M=2048, K=4096, N=12288, 0.93 at N=22016 and
+    // 0.74 at M=K=N=8192; 128x128 0.71 to 0.76; 64x128 0.64 to 0.67 (a 64x128 tile takes 0.55 to 0.6 of
+    // the time of a 128x128 one, so it pays where it doubles the workgroups without adding a round).
     double best = 1e300;
     TileChoice c{128, 128};
     for (const auto& t : cand) {
