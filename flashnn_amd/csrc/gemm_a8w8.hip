@@ -83,8 +83,15 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     const int xcd = blockIdx.x & 7;
     const int t = xcd * p.tiles_per_xcd + (blockIdx.x >> 3);
     if ((blockIdx.x >> 3) >= p.tiles_per_xcd || t >= p.tiles_m * p.tiles_n) return;
-    const int tile_m = t % p.tiles_m;
-    const int tile_n = t / p.tiles_m;
+    // tiles are numbered in groups of GN tile columns, the column fastest within a group: the 32 workgroups
+    // an XCD runs at a time then cover 8 tile rows x 4 tile columns whatever M is, and fetch
+    // 8*BM + 4*BN operand rows per slab into its L2 instead of tiles_m*BM + BN
+    constexpr int GN = 4;
+    const int grp = t / (GN * p.tiles_m);
+    const int rem = t - grp * (GN * p.tiles_m);
+    const int gw = min(GN, p.tiles_n - grp * GN);
+    const int tile_n = grp * GN + rem % gw;
+    const int tile_m = rem / gw;
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
 
