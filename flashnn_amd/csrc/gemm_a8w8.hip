@@ -1,23 +1,23 @@
 // A8W8 GEMM for gfx950:  acc[m,n] = sum_k a[m,k] * b[n,k]  (int8 x int8 -> int32, exact),
 // out = float(acc) * alpha_row[m] * alpha_col[n]  -> fp16 / bf16   (or the raw int32).
 //
-// Main kernel (K % 128 == 0, 16-byte aligned rows)
+// Main kernel (K % 32 == 0, K >= 512, 16-byte aligned rows)
 //   * one 256-thread workgroup (4 waves, 2x2) per BM x BN output tile, one workgroup per CU;
 //   * K is walked in slabs of 128 bytes.  A slab of the a-rows and b-rows of the tile is
-//     copied global -> LDS with direct-to-LDS 16-byte loads (no VGPR staging) into one of
-//     two static LDS stages while the MFMAs of the previous slab run;
+//     copied global -> LDS with direct-to-LDS 16-byte loads (no VGPR staging) into a ring of
+//     LDS stages, one or two slabs ahead of the MFMAs;
 //   * both operands are K-contiguous, so a lane's 16-byte LDS read is directly one
 //     v_mfma_i32_16x16x64_i8 operand (with random operands the device sustains a fifth more of
-//     these than of the 32x32x32 shape: 4.0 against 3.35 POP/s).  The 16-byte chunks of each 128-byte LDS row are
-//     XOR-swizzled with (row & 7) so that the 8 lanes served together hit 8 distinct
-//     bank groups.  The swizzle is applied on the global side of the copy (the LDS side
+//     these than of the 32x32x32 shape: 4.0 against 3.35 POP/s).  The 16-byte chunks of each
+//     128-byte LDS row are XOR-swizzled with ((row >> 1) & 7) so that the 16 lanes served together
+//     hit distinct banks.  The swizzle is applied on the global side of the copy (the LDS side
 //     of a direct-to-LDS load is linear in the lane id);
 //   * the weight rows feed the MFMA "A" operand and the activation rows the "B"
 //     operand, so a lane ends up with 4 consecutive n for one m: the epilogue scales in
-//     fp32 and writes 8-byte (16-bit out) or 16-byte (int32 out) pieces;
+//     fp32, transposes through LDS and writes whole rows;
 //   * workgroup ids are remapped so that each XCD (ids congruent mod 8 share an L2) works
-//     on a contiguous band of tiles with the m index fastest, which keeps the b-panel and
-//     the whole a-panel slab of the moment resident in that XCD's L2.
+//     on a contiguous band of tiles, numbered so that the workgroups it runs at a time cover
+//     8 tile rows x 4 tile columns and share their operand rows through that XCD's L2.
 //
 // Any other shape takes a small guarded LDS kernel built on v_dot4_i32_i8.
 //

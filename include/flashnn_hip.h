@@ -229,8 +229,10 @@ int fnn_debug_force_a8w8_tile(int bm, int bn);
 
 /*
  * Measurement aid, no counterpart in the reference: the rate, in 1e12 int8 operations per second,
- * at which the current device sustains back-to-back 32x32x32 int8 MFMAs with operands held in
- * registers (two waves per SIMD, no memory traffic).  random_operands != 0 feeds the matrix cores
+ * at which the current device sustains back-to-back 16x16x64 int8 MFMAs with operands held in
+ * registers, in the shape and order of the tiled A8W8 kernel's 256x192 tile (one wave per SIMD, 6 weight
+ * fragments against 8 activation fragments, the weight fragment fixed over the inner loop; no memory
+ * traffic).  random_operands != 0 feeds the matrix cores
  * random bytes, as a GEMM on quantised data does; 0 feeds constants.  The clock follows the power
  * drawn, and that follows the toggling of the operand bits, so the two rates differ; the first is the
  * ceiling an A8W8 GEMM can approach on this device.  Runs 1 + launches kernels of `iters` loop
