@@ -118,6 +118,22 @@ def test_a8w8_partial_last_slab_bit_exact(hip_lib, tile, mnk):
     assert np.array_equal(out.float().cpu().numpy(), O.gemm_a8w8_epilogue_fp32(want, O.to_np(ar), O.to_np(ac), O.F16))
 
 
+@pytest.mark.parametrize("tile,mn", [((64, 128), (720, 773)), ((64, 128), (1100, 300)), ((128, 128), (1290, 650)),
+                                     ((256, 128), (2310, 1100)), ((256, 192), (2400, 1000)), ((256, 192), (2600, 200))])
+def test_a8w8_tile_numbering_many_tile_rows(hip_lib, tile, mn):
+    """More than 8 tile rows and a number of tile columns that is no multiple of 4: the tiles are numbered
+    in groups of 4 tile columns, and the last group is narrower."""
+    M, N = mn
+    K = 512
+    a, b = _rand_i8((M, K), 31), _rand_i8((N, K), 32)
+    assert hip_lib.fnn_debug_force_a8w8_tile(*tile) == 0
+    try:
+        acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+    finally:
+        hip_lib.fnn_debug_force_a8w8_tile(0, 0)
+    assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
+
+
 @pytest.mark.parametrize("mnk", [(5, 7, 100), (130, 70, 1000), (64, 64, 8), (33, 65, 129)])
 def test_a8w8_guarded_kernel_bit_exact(mnk):
     M, N, K = mnk
