@@ -195,7 +195,12 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     };
     // ask the scheduler for: 2 MFMAs, 1 LDS read, 2 MFMAs, 1 LDS read, ... then the remaining MFMAs, so
     // that the reads of a phase are spread over its first half and have its second half to return
-    auto interleave = [&](int part) {
+    // ncopies > 0 also places that many of the phase's copies behind those groups instead of leaving them
+    // to the scheduler, which issues them, with their address arithmetic, ahead of the first MFMA after the
+    // barrier.  Worth 1 to 2 % on the 256x192 tile; the tiles with three stages of both operands ran up to
+    // 1.5 % slower with it and pass 0.
+    auto interleave = [&](int part, auto ncopies) {
+        constexpr int NC = decltype(ncopies)::value;
         constexpr int NM = HN * FM;
         constexpr int R0 = NRA, R1 = NRD - NRA;
         constexpr int PER = NM >= 2 * R0 ? 2 : 1;
@@ -204,6 +209,10 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             for (int q = 0; q < R0; ++q) {
                 __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if constexpr (NC > 0) {
+                    constexpr int VPG = (NC + R0 - 1) / R0;   // copies behind each of the first groups
+                    if (q < (NC + VPG - 1) / VPG) __builtin_amdgcn_sched_group_barrier(0x010, VPG, 0);
+                }
             }
             if constexpr (NM - PER * R0 > 0) __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * R0, 0);
         } else {
@@ -211,6 +220,10 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             for (int q = 0; q < R1; ++q) {
                 __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if constexpr (NC > 0) {
+                    constexpr int VPG = (NC + R1 - 1) / R1;   // copies behind each of the first groups
+                    if (q < (NC + VPG - 1) / VPG) __builtin_amdgcn_sched_group_barrier(0x010, VPG, 0);
+                }
             }
             if constexpr (NM - PER * R1 > 0) __builtin_amdgcn_sched_group_barrier(0x008, NM - PER * R1, 0);
         }
@@ -267,11 +280,11 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     // of slab i is read; phases C and D multiply that chunk 0 while chunk 1 is read.  The reads are so
     // spread evenly: (FN+FM)/2 per phase.  The freed stages take the slab two ahead, copied in parts
     // over the phases (issued in one burst the copies block the wave's MFMAs behind them).
-#define FNN_PHASE(ca, cb, kq, part, copies, mq, mh)  \
+#define FNN_PHASE(ca, cb, kq, part, copies, mq, mh, NC)  \
     read_part(ca, cb, kq, part);                      \
     copies;                                           \
     mfmas(mq, mh);                                    \
-    interleave(part);                                 \
+    interleave(part, std::integral_constant<int, NC>{});  \
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (BDEEP) {
         // a-rows in two stages: slab i+1 goes into the a-stage of slab i-1, in one burst after the barrier
@@ -283,10 +296,10 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             const int fix_a = !steady && i + 1 == KT - 1 ? tail_fix : 0;
             const int fix_b = !steady && i + 2 == KT - 1 ? tail_fix : 0;
             wait_barrierB(true);
-            FNN_PHASE(ca, cb, 0, 0, copy_a(fa, i + 1, fix_a), 1, 0)
-            FNN_PHASE(ca, cb, 0, 1, if (more) copy_b_part(fb, i + 2, 0, fix_b), 1, 1)
-            FNN_PHASE(ca, cb, 1, 0, if (more) copy_b_part(fb, i + 2, 1, fix_b), 0, 0)
-            FNN_PHASE(ca, cb, 1, 1, if (more) copy_b_part(fb, i + 2, 2, fix_b), 0, 1)
+            FNN_PHASE(ca, cb, 0, 0, copy_a(fa, i + 1, fix_a), 1, 0, NLA)
+            FNN_PHASE(ca, cb, 0, 1, if (more) copy_b_part(fb, i + 2, 0, fix_b), 1, 1, (NLB + 2) / 3)
+            FNN_PHASE(ca, cb, 1, 0, if (more) copy_b_part(fb, i + 2, 1, fix_b), 0, 0, (NLB + 2) / 3)
+            FNN_PHASE(ca, cb, 1, 1, if (more) copy_b_part(fb, i + 2, 2, fix_b), 0, 1, (NLB + 2) / 3)
         };
         copy_b(sb0, 0);
         copy_a(sa0, 0);
@@ -296,8 +309,8 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         read_part(sa0, sb0, 0, 1);
         copy_a(sa1, 1);
         copy_b_part(sb2, 2, 0);
-        FNN_PHASE(sa0, sb0, 1, 0, copy_b_part(sb2, 2, 1), 0, 0)
-        FNN_PHASE(sa0, sb0, 1, 1, copy_b_part(sb2, 2, 2), 0, 1)
+        FNN_PHASE(sa0, sb0, 1, 0, copy_b_part(sb2, 2, 1), 0, 0, (NLB + 2) / 3)
+        FNN_PHASE(sa0, sb0, 1, 1, copy_b_part(sb2, 2, 2), 0, 1, (NLB + 2) / 3)
         int i = 1;
         // (the steady loop stops one slab earlier when the last slab is partial: its copies need the fix)
         for (; i + 8 + (last_steps < 4) <= KT; i += 6) {
@@ -327,10 +340,10 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             const bool more = steady || i + 2 < KT;
             const int fix = !steady && i + 2 == KT - 1 ? tail_fix : 0;
             wait_barrier3(true);
-            FNN_PHASE(ca, cb, 0, 0, if (more) { copy_a_part(fa, i + 2, 0, fix); copy_b_part(fb, i + 2, 0, fix); }, 1, 0)
-            FNN_PHASE(ca, cb, 0, 1, if (more) { copy_a_part(fa, i + 2, 1, fix); copy_b_part(fb, i + 2, 1, fix); }, 1, 1)
-            FNN_PHASE(ca, cb, 1, 0, if (more) { copy_a_part(fa, i + 2, 2, fix); copy_b_part(fb, i + 2, 2, fix); }, 0, 0)
-            FNN_PHASE(ca, cb, 1, 1, , 0, 1)
+            FNN_PHASE(ca, cb, 0, 0, if (more) { copy_a_part(fa, i + 2, 0, fix); copy_b_part(fb, i + 2, 0, fix); }, 1, 0, 0)
+            FNN_PHASE(ca, cb, 0, 1, if (more) { copy_a_part(fa, i + 2, 1, fix); copy_b_part(fb, i + 2, 1, fix); }, 1, 1, 0)
+            FNN_PHASE(ca, cb, 1, 0, if (more) { copy_a_part(fa, i + 2, 2, fix); copy_b_part(fb, i + 2, 2, fix); }, 0, 0, 0)
+            FNN_PHASE(ca, cb, 1, 1, , 0, 1, 0)
         };
         copy_a(sa0, 0);
         copy_b(sb0, 0);
@@ -343,8 +356,8 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         copy_b_part(sb2, 2, 0);
         copy_a_part(sa2, 2, 1);
         copy_b_part(sb2, 2, 1);
-        FNN_PHASE(sa0, sb0, 1, 0, { copy_a_part(sa2, 2, 2); copy_b_part(sb2, 2, 2); }, 0, 0)
-        FNN_PHASE(sa0, sb0, 1, 1, , 0, 1)
+        FNN_PHASE(sa0, sb0, 1, 0, { copy_a_part(sa2, 2, 2); copy_b_part(sb2, 2, 2); }, 0, 0, 0)
+        FNN_PHASE(sa0, sb0, 1, 1, , 0, 1, 0)
         int i = 1;
         for (; i + 5 + (last_steps < 4) <= KT; i += 3) {
             iter3(sa1, sb1, sa0, sb0, i, true);
