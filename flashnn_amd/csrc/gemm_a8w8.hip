@@ -146,6 +146,22 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
                                              (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
+    auto copy_a_half = [&](char* stage, int kt, int half, int fix = 0) {
+        const char* slab = (const char*)p.a + (int64_t)kt * BK + fix;
+#pragma unroll
+        for (int j = 0; j < NLA; ++j)
+            if (j * 2 / NLA == half)
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + goa[j]),
+                                                 (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
+    };
+    auto copy_b_half = [&](char* stage, int kt, int half, int fix = 0) {
+        const char* slab = (const char*)p.b + (int64_t)kt * BK + fix;
+#pragma unroll
+        for (int j = 0; j < NLB; ++j)
+            if (j * 2 / NLB == half)
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
+                                                 (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
+    };
     auto copy_b_part = [&](char* stage, int kt, int part, int fix = 0) {
         const char* slab = (const char*)p.b + (int64_t)kt * BK + fix;
 #pragma unroll
@@ -287,19 +303,20 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     interleave(part, std::integral_constant<int, NC>{});  \
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (BDEEP) {
-        // a-rows in two stages: slab i+1 goes into the a-stage of slab i-1, in one burst after the barrier
-        // (it must be complete at the next one); b-rows in three: slab i+2 follows in three parts, and only
-        // those parts may be in flight at the next barrier
+        // a-rows in two stages: slab i+1 goes into the a-stage of slab i-1 during phases A and B (it must be
+        // complete at the next barrier); b-rows in three: slab i+2 follows during phases C and D, and only
+        // its copies may be in flight at the next barrier (vmcnt counts in order, so all a-copies come first).
+        // (All a-copies in phase A and the b-copies over B, C and D: 8192^3 411 -> 402 us, QKV 86.2 -> 85.8 us.)
         auto wait_barrierB = [&](bool keep) { wait_barrier_n(keep, std::integral_constant<int, NLB>{}); };
         auto iterB = [&](const char* ca, const char* cb, char* fa, char* fb, int i, bool steady) {
             const bool more = steady || i + 2 < KT;
             const int fix_a = !steady && i + 1 == KT - 1 ? tail_fix : 0;
             const int fix_b = !steady && i + 2 == KT - 1 ? tail_fix : 0;
             wait_barrierB(true);
-            FNN_PHASE(ca, cb, 0, 0, copy_a(fa, i + 1, fix_a), 1, 0, NLA)
-            FNN_PHASE(ca, cb, 0, 1, if (more) copy_b_part(fb, i + 2, 0, fix_b), 1, 1, (NLB + 2) / 3)
-            FNN_PHASE(ca, cb, 1, 0, if (more) copy_b_part(fb, i + 2, 1, fix_b), 0, 0, (NLB + 2) / 3)
-            FNN_PHASE(ca, cb, 1, 1, if (more) copy_b_part(fb, i + 2, 2, fix_b), 0, 1, (NLB + 2) / 3)
+            FNN_PHASE(ca, cb, 0, 0, copy_a_half(fa, i + 1, 0, fix_a), 1, 0, NLA / 2)
+            FNN_PHASE(ca, cb, 0, 1, copy_a_half(fa, i + 1, 1, fix_a), 1, 1, NLA / 2)
+            FNN_PHASE(ca, cb, 1, 0, if (more) copy_b_half(fb, i + 2, 0, fix_b), 0, 0, NLB / 2)
+            FNN_PHASE(ca, cb, 1, 1, if (more) copy_b_half(fb, i + 2, 1, fix_b), 0, 1, NLB / 2)
         };
         copy_b(sb0, 0);
         copy_a(sa0, 0);
@@ -308,9 +325,8 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         read_part(sa0, sb0, 0, 0);
         read_part(sa0, sb0, 0, 1);
         copy_a(sa1, 1);
-        copy_b_part(sb2, 2, 0);
-        FNN_PHASE(sa0, sb0, 1, 0, copy_b_part(sb2, 2, 1), 0, 0, (NLB + 2) / 3)
-        FNN_PHASE(sa0, sb0, 1, 1, copy_b_part(sb2, 2, 2), 0, 1, (NLB + 2) / 3)
+        FNN_PHASE(sa0, sb0, 1, 0, copy_b_half(sb2, 2, 0), 0, 0, NLB / 2)
+        FNN_PHASE(sa0, sb0, 1, 1, copy_b_half(sb2, 2, 1), 0, 1, NLB / 2)
         int i = 1;
         // (the steady loop stops one slab earlier when the last slab is partial: its copies need the fix)
         for (; i + 8 + (last_steps < 4) <= KT; i += 6) {
