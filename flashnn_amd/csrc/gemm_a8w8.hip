@@ -100,14 +100,21 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     const int wm = wave & 1;
     const int wn = wave >> 1;
 
-    // Scales of the tile go to LDS as fp32 before anything else is in flight; the epilogue then
-    // needs no global loads.
+    // The tile's scales are requested before anything else, as raw words into registers, and nobody waits
+    // for them: they are older than every copy, so they have arrived long before the main loop ends.
+    // They are widened and staged in LDS just before the epilogue, which then needs no global loads.
+    // (Staged at kernel start, their latency came on top of that of the first copies.)
+    constexpr int NSC = (BM + BN + 255) / 256;
+    uint32_t sc_raw[NSC];
     if constexpr (MODE != OUT_I32) {
-        for (int e = threadIdx.x; e < BM + BN; e += 256) {
+#pragma unroll
+        for (int q = 0; q < NSC; ++q) {
+            const int e = threadIdx.x + q * 256;
             const bool is_row = e < BM;
-            const int idx = is_row ? min(m0 + e, p.M - 1) : min(n0 + e - BM, p.N - 1);
-            const float v = load_as_f32(is_row ? p.arow : p.acol, idx, is_row ? p.arow_dtype : p.acol_dtype);
-            if (is_row) sc_row[e] = v; else sc_col[e - BM] = v;
+            const int idx = is_row ? min(m0 + e, p.M - 1) : min(n0 + min(e - BM, BN - 1), p.N - 1);
+            const void* base = is_row ? p.arow : p.acol;
+            sc_raw[q] = (is_row ? p.arow_dtype : p.acol_dtype) == FNN_F32 ? ((const uint32_t*)base)[idx]
+                                                                        : (uint32_t)((const uint16_t*)base)[idx];
         }
     }
 
@@ -430,6 +437,17 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         __builtin_amdgcn_s_waitcnt(0x0070);   // all copies and LDS reads of this wave are done
         __builtin_amdgcn_s_barrier();         // ... and everybody else's: the stages are free
         asm volatile("" ::: "memory");
+#pragma unroll
+        for (int q = 0; q < NSC; ++q) {
+            const int e = threadIdx.x + q * 256;
+            const bool is_row = e < BM;
+            const int dt = is_row ? p.arow_dtype : p.acol_dtype;
+            const float v = dt == FNN_F32 ? __builtin_bit_cast(float, sc_raw[q])
+                                          : dt == FNN_F16 ? f16_bits_to_f32(sc_raw[q]) : bf16_bits_to_f32(sc_raw[q]);
+            if (is_row) sc_row[e] = v;
+            else if (e < BM + BN) sc_col[e - BM] = v;
+        }
+        __syncthreads();
         const bool vec_ok = (p.ldc & 7) == 0;
 #pragma unroll
         for (int jc = 0; jc < FM; jc += RC) {
