@@ -133,12 +133,21 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     // evenly instead of receiving a burst that blocks the wave's issue (and its MFMAs) behind it
     // `fix` moves a lane's 16 bytes back to the start of its row piece: the lanes of the last,
     // partial slab whose chunk lies beyond K fetch bytes that exist (and are never used)
+    // The address of a copy is a scalar base (matrix + slab) plus the lane's 32-bit row offset, which is the
+    // form the copy instruction takes directly; the base is passed through readfirstlane so that it is not
+    // folded into per-lane 64-bit pointers that need vector adds before every copy.
+    auto slab_base = [&](const int8_t* m, int kt) -> const char* {
+        const uint64_t v = (uint64_t)m + (uint64_t)((int64_t)kt * BK);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (const char*)(((uint64_t)hi << 32) | lo);
+    };
     auto copy_a_part = [&](char* stage, int kt, int part, int fix = 0) {
-        const char* slab = (const char*)p.a + (int64_t)kt * BK + fix;
+        const char* slab = slab_base(p.a, kt);
 #pragma unroll
         for (int j = 0; j < NLA; ++j)
             if (j * 3 / NLA == part)
-                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + goa[j]),
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + (uint32_t)(goa[j] + fix)),
                                                  (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
     auto copy_a = [&](char* stage, int kt, int fix = 0) {
@@ -147,34 +156,34 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
         copy_a_part(stage, kt, 2, fix);
     };
     auto copy_b = [&](char* stage, int kt) {
-        const char* slab = (const char*)p.b + (int64_t)kt * BK;
+        const char* slab = slab_base(p.b, kt); const int fix = 0;
 #pragma unroll
         for (int j = 0; j < NLB; ++j)
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + (uint32_t)(gob[j] + fix)),
                                              (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
     auto copy_a_half = [&](char* stage, int kt, int half, int fix = 0) {
-        const char* slab = (const char*)p.a + (int64_t)kt * BK + fix;
+        const char* slab = slab_base(p.a, kt);
 #pragma unroll
         for (int j = 0; j < NLA; ++j)
             if (j * 2 / NLA == half)
-                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + goa[j]),
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + (uint32_t)(goa[j] + fix)),
                                                  (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
     auto copy_b_half = [&](char* stage, int kt, int half, int fix = 0) {
-        const char* slab = (const char*)p.b + (int64_t)kt * BK + fix;
+        const char* slab = slab_base(p.b, kt);
 #pragma unroll
         for (int j = 0; j < NLB; ++j)
             if (j * 2 / NLB == half)
-                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + (uint32_t)(gob[j] + fix)),
                                                  (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
     auto copy_b_part = [&](char* stage, int kt, int part, int fix = 0) {
-        const char* slab = (const char*)p.b + (int64_t)kt * BK + fix;
+        const char* slab = slab_base(p.b, kt);
 #pragma unroll
         for (int j = 0; j < NLB; ++j)
             if (j * 3 / NLB == part)
-                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + gob[j]),
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + (uint32_t)(gob[j] + fix)),
                                                  (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
 
