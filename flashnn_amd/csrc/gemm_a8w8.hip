@@ -129,10 +129,10 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
 #pragma unroll
     for (int j = 0; j < NLB; ++j)
         gob[j] = (uint32_t)min(n0 + (j * NWAVES + wave) * 8 + lrow, p.N - 1) * (uint32_t)p.ldb + lchunk * 16;
-    // the a-copy of a slab is issued in three parts, one per k-step, so that the copy unit is fed
-    // evenly instead of receiving a burst that blocks the wave's issue (and its MFMAs) behind it
-    // `fix` moves a lane's 16 bytes back to the start of its row piece: the lanes of the last,
-    // partial slab whose chunk lies beyond K fetch bytes that exist (and are never used)
+    // The copies of a slab are issued in parts (halves or thirds), one per phase of the loop, so that the
+    // copy unit is fed evenly instead of receiving a burst that blocks the wave's issue (and its MFMAs)
+    // behind it.  `fix` moves a lane's 16 bytes back to the start of its row piece: the lanes of the last,
+    // partial slab whose chunk lies beyond K fetch bytes that exist (and are never used).
     // The address of a copy is a scalar base (matrix + slab) plus the lane's 32-bit row offset, which is the
     // form the copy instruction takes directly; the base is passed through readfirstlane so that it is not
     // folded into per-lane 64-bit pointers that need vector adds before every copy.
