@@ -53,6 +53,19 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // two-way conflicts: measured 8 instead of 4 cycles per read.)  The swizzle is applied on the
 // global side of the copy; the LDS side of a direct-to-LDS load is linear in the lane id.
 
+// An LDS stage that exists only in some instantiations (a zero-length array is not allowed).
+template <bool HAS, int BYTES>
+struct OptionalStage {
+    static __device__ __forceinline__ char* get() {
+        __shared__ __attribute__((aligned(1024))) char buf[BYTES];
+        return buf;
+    }
+};
+template <int BYTES>
+struct OptionalStage<false, BYTES> {
+    static __device__ __forceinline__ char* get() { return nullptr; }
+};
+
 template <int BM, int BN, int MODE>
 __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     constexpr int NWAVES = 4;
@@ -68,8 +81,11 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     __shared__ __attribute__((aligned(1024))) char sa1[BM * BK];
     // tiles too large for three stages of both operands give the third stage to the b-rows (the
     // weights, streamed from HBM) and copy the a-rows (L2 hits after their first use) one slab ahead
-    constexpr bool BDEEP = 3 * (BM + BN) * BK + 4 * (BM + BN) + 1024 > 160 * 1024;
-    __shared__ __attribute__((aligned(1024))) char sa2[BDEEP ? 16 : BM * BK];
+    // The 128x128 tile takes the same arrangement although three stages of both would fit: with two
+    // a-stages it needs exactly 80 KB, and two workgroups share a CU - each one's prologue, epilogue and
+    // barrier waits then run under the other's MFMAs.
+    constexpr bool BDEEP = 3 * (BM + BN) * BK + 4 * (BM + BN) + 1024 > 160 * 1024 || (BM == 128 && BN == 128);
+    char* const sa2 = OptionalStage<!BDEEP, BM * BK>::get();   // no third a-stage, and no LDS for it, where BDEEP
     __shared__ __attribute__((aligned(1024))) char sb0[BN * BK];
     __shared__ __attribute__((aligned(1024))) char sb1[BN * BK];
     // a third b-stage where the tile leaves room for it (3 * (BM + BN) rows <= 160 KB): the b-rows are
@@ -77,8 +93,11 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     // to land, which is about the loaded L2 latency
     constexpr int NSB = 3 * (BM + BN) * BK + 4 * (BM + BN) + 1024 <= 160 * 1024 ? 3 : 2;
     __shared__ __attribute__((aligned(1024))) char sb2[NSB == 3 || BDEEP ? BN * BK : 16];
-    __shared__ __attribute__((aligned(16))) float sc_row[BM];   // alpha_row of the tile's rows, fp32
-    __shared__ __attribute__((aligned(16))) float sc_col[BN];   // alpha_col of the tile's columns
+    // alpha_row of the tile's rows and alpha_col of its columns as fp32: staged only before the epilogue, in
+    // the third b-stage, which is free by then and which the epilogue's transposition does not use
+    static_assert(NSB == 3 || BDEEP, "the scales live in the third b-stage");
+    float* const sc_row = (float*)sb2;
+    float* const sc_col = sc_row + BM;
 
     const int xcd = blockIdx.x & 7;
     const int t = xcd * p.tiles_per_xcd + (blockIdx.x >> 3);
@@ -562,31 +581,12 @@ __global__ __launch_bounds__(256) void gemm_a8w8_any_kernel(const A8W8Args p) {
 // ------------------------------------------------------------------------ dispatch
 struct TileChoice { int bm, bn; };
 
-// Pick the tile whose last, partly filled round of workgroups costs least on 256 CUs.
-static TileChoice choose_tile(int64_t M, int64_t N) {
-    static const struct { int bm, bn; double eff; } cand[] = {
-        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.72}, {64, 128, 0.62}};
-    // eff = throughput per tile area relative to the 256x192 tile, measured with every round full.  It
-    // depends on the shape: the 256x128 tile reaches 1.0 at M=2048, K=4096, N=12288, 0.93 at N=22016 and
-    // 0.74 at M=K=N=8192; 128x128 0.71 to 0.76; 64x128 0.64 to 0.67 (a 64x128 tile takes 0.55 to 0.6 of
-    // the time of a 128x128 one, so it pays where it doubles the workgroups without adding a round).
-    double best = 1e300;
-    TileChoice c{128, 128};
-    for (const auto& t : cand) {
-        const int64_t tiles = ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
-        const int64_t rounds = (tiles + 255) / 256;
-        const double cost = (double)rounds * t.bm * t.bn / t.eff;
-        if (cost < best) { best = cost; c = {t.bm, t.bn}; }
-    }
-    return c;
-}
-
 // With 256x192 tiles, the number of 192-wide tile columns to give a first launch when the rest is better done
 // by a second launch of 256x128 tiles, or 0.  A round of 256 workgroups takes one tile time however few of
 // them exist, so a last round that is mostly empty is expensive; the columns are then cut where the first
 // launch ends on a full round.  Costs in 256x192 tile times: a 256x128 tile takes 128/192/0.85 of one, the
 // second launch about 0.08 (its launch gap and start-up).
-static int split_columns_192(int64_t M, int64_t N) {
+static int split_columns_192(int64_t M, int64_t N, double* cost_out = nullptr) {
     const int64_t tm = (M + 255) / 256, c = (N + 191) / 192;
     const double single = (double)((tm * c + 255) / 256);
     double best = single - 0.1;      // worth a second launch only from a tenth of a round
@@ -597,7 +597,40 @@ static int split_columns_192(int64_t M, int64_t N) {
         const double cost = (double)r1 + (double)r2 * (128.0 / 192.0 / 0.85) + 0.08;
         if (cost < best) { best = cost; best_c1 = (int)c1; }
     }
+    if (cost_out) *cost_out = best_c1 > 0 ? best : single;   // in 256x192 tile times
     return best_c1;
+}
+
+// Pick the tile whose rounds of workgroups cost least on 256 CUs.
+static TileChoice choose_tile(int64_t M, int64_t N) {
+    static const struct { int bm, bn; double eff; } cand[] = {
+        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.82}, {64, 128, 0.55}};
+    // eff = throughput per tile area relative to the 256x192 tile, measured with every round full.  It
+    // depends on the shape: the 256x128 tile reaches 1.0 at M=2048, K=4096, N=12288, 0.93 at N=22016 and
+    // 0.74 at M=K=N=8192; 128x128 0.85 with two workgroups on every CU (0.71 to 0.76 with one); 64x128 0.64
+    // to 0.67 in full rounds.  The 128x128 tile runs two workgroups per CU, so a round of it holds 512 tiles; a
+    // last round of at most 256 leaves every workgroup a CU of its own and takes 0.64 of a shared one (41.7
+    // against 65.1 us at K = N = 8192).  The two small tiles are priced a little below their full-round
+    // figures (0.82, 0.55): that puts the ties seen on the box on the right side (M=768 N=35584 and M=2112
+    // N=13312 stay with 256x192, 116 against 122 us and 118 against 121; M=320 N=17792 and M=576 N=17792 move
+    // from 64x128 to 128x128, 43 -> 36.5 us and 64.5 -> 57 us).
+    double best = 1e300;
+    TileChoice c{128, 128};
+    for (const auto& t : cand) {
+        const int64_t tiles = ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
+        double cost;
+        if (t.bm == 128) {
+            const int64_t rem = tiles % 512;
+            cost = ((double)(tiles / 512) + (rem == 0 ? 0.0 : rem <= 256 ? 0.64 : 1.0)) * 2.0 * t.bm * t.bn / t.eff;
+        } else if (t.bn == 192) {
+            split_columns_192(M, N, &cost);   // with the ragged last round split off where that pays
+            cost *= 256.0 * 192.0;
+        } else {
+            cost = (double)((tiles + 255) / 256) * t.bm * t.bn / t.eff;
+        }
+        if (cost < best) { best = cost; c = {t.bm, t.bn}; }
+    }
+    return c;
 }
 
 template <int BM, int BN, int MODE>
