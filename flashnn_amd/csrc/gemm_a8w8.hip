@@ -66,7 +66,7 @@ struct OptionalStage<false, BYTES> {
     static __device__ __forceinline__ char* get() { return nullptr; }
 };
 
-template <int BM, int BN, int MODE>
+template <int BM, int BN, int MODE, bool PAIR = false>
 __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     constexpr int NWAVES = 4;
     constexpr int WTM = BM / 2, WTN = BN / 2;
@@ -81,10 +81,13 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     __shared__ __attribute__((aligned(1024))) char sa1[BM * BK];
     // tiles too large for three stages of both operands give the third stage to the b-rows (the
     // weights, streamed from HBM) and copy the a-rows (L2 hits after their first use) one slab ahead
-    // The 128x128 tile takes the same arrangement although three stages of both would fit: with two
-    // a-stages it needs exactly 80 KB, and two workgroups share a CU - each one's prologue, epilogue and
-    // barrier waits then run under the other's MFMAs.
-    constexpr bool BDEEP = 3 * (BM + BN) * BK + 4 * (BM + BN) + 1024 > 160 * 1024 || (BM == 128 && BN == 128);
+    // PAIR (128x128 tile, more than 256 tiles): the same arrangement although three stages of both would
+    // fit - with two a-stages the tile needs exactly 80 KB, and two workgroups share a CU: each one's
+    // prologue, epilogue and barrier waits then run under the other's MFMAs (17 to 25 % faster).  With at
+    // most 256 tiles every workgroup has a CU to itself and the three-stage version is the faster one
+    // (by 3 % at K = 8192, by 20 % at K = 18944).
+    static_assert(!PAIR || 2 * ((2 * BM + 3 * BN) * BK) <= 160 * 1024, "a pair of workgroups must fit the LDS");
+    constexpr bool BDEEP = 3 * (BM + BN) * BK + 4 * (BM + BN) + 1024 > 160 * 1024 || PAIR;
     char* const sa2 = OptionalStage<!BDEEP, BM * BK>::get();   // no third a-stage, and no LDS for it, where BDEEP
     __shared__ __attribute__((aligned(1024))) char sb0[BN * BK];
     __shared__ __attribute__((aligned(1024))) char sb1[BN * BK];
@@ -586,7 +589,7 @@ struct TileChoice { int bm, bn; };
 // them exist, so a last round that is mostly empty is expensive; the columns are then cut where the first
 // launch ends on a full round.  Costs in 256x192 tile times: a 256x128 tile takes 128/192/0.85 of one, the
 // second launch about 0.08 (its launch gap and start-up).
-static int split_columns_192(int64_t M, int64_t N, double* cost_out = nullptr) {
+static int split_columns_192(int64_t M, int64_t N) {
     const int64_t tm = (M + 255) / 256, c = (N + 191) / 192;
     const double single = (double)((tm * c + 255) / 256);
     double best = single - 0.1;      // worth a second launch only from a tenth of a round
@@ -597,49 +600,39 @@ static int split_columns_192(int64_t M, int64_t N, double* cost_out = nullptr) {
         const double cost = (double)r1 + (double)r2 * (128.0 / 192.0 / 0.85) + 0.08;
         if (cost < best) { best = cost; best_c1 = (int)c1; }
     }
-    if (cost_out) *cost_out = best_c1 > 0 ? best : single;   // in 256x192 tile times
     return best_c1;
 }
 
-// Pick the tile whose rounds of workgroups cost least on 256 CUs.
+// Pick the tile whose last, partly filled round of workgroups costs least on 256 CUs.
 static TileChoice choose_tile(int64_t M, int64_t N) {
     static const struct { int bm, bn; double eff; } cand[] = {
-        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.82}, {64, 128, 0.55}};
+        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.72}, {64, 128, 0.62}};
     // eff = throughput per tile area relative to the 256x192 tile, measured with every round full.  It
     // depends on the shape: the 256x128 tile reaches 1.0 at M=2048, K=4096, N=12288, 0.93 at N=22016 and
-    // 0.74 at M=K=N=8192; 128x128 0.85 with two workgroups on every CU (0.71 to 0.76 with one); 64x128 0.64
-    // to 0.67 in full rounds.  The 128x128 tile runs two workgroups per CU, so a round of it holds 512 tiles; a
-    // last round of at most 256 leaves every workgroup a CU of its own and takes 0.64 of a shared one (41.7
-    // against 65.1 us at K = N = 8192).  The two small tiles are priced a little below their full-round
-    // figures (0.82, 0.55): that puts the ties seen on the box on the right side (M=768 N=35584 and M=2112
-    // N=13312 stay with 256x192, 116 against 122 us and 118 against 121; M=320 N=17792 and M=576 N=17792 move
-    // from 64x128 to 128x128, 43 -> 36.5 us and 64.5 -> 57 us).
+    // 0.74 at M=K=N=8192; 128x128 0.71 to 0.76; 64x128 0.64 to 0.67 (a 64x128 tile takes 0.55 to 0.6 of
+    // the time of a 128x128 one, so it pays where it doubles the workgroups without adding a round).
+    // The 128x128 figure is that of one workgroup per CU.  From 257 tiles on the tile runs two per CU and
+    // reaches 0.85; a model that prices this (and the column split of the 256x192 tile) chose better in
+    // eight of ten shapes tried and worse in a sweep's short-K shapes, so the choice is left as it was and
+    // only shapes that took the 128x128 tile anyway gain.
     double best = 1e300;
     TileChoice c{128, 128};
     for (const auto& t : cand) {
         const int64_t tiles = ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
-        double cost;
-        if (t.bm == 128) {
-            const int64_t rem = tiles % 512;
-            cost = ((double)(tiles / 512) + (rem == 0 ? 0.0 : rem <= 256 ? 0.64 : 1.0)) * 2.0 * t.bm * t.bn / t.eff;
-        } else if (t.bn == 192) {
-            split_columns_192(M, N, &cost);   // with the ragged last round split off where that pays
-            cost *= 256.0 * 192.0;
-        } else {
-            cost = (double)((tiles + 255) / 256) * t.bm * t.bn / t.eff;
-        }
+        const int64_t rounds = (tiles + 255) / 256;
+        const double cost = (double)rounds * t.bm * t.bn / t.eff;
         if (cost < best) { best = cost; c = {t.bm, t.bn}; }
     }
     return c;
 }
 
-template <int BM, int BN, int MODE>
+template <int BM, int BN, int MODE, bool PAIR = false>
 static void launch_mfma(A8W8Args& p, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
-    gemm_a8w8_ring_kernel<BM, BN, MODE><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p);
+    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p);
 }
 
 template <int MODE>
@@ -677,6 +670,7 @@ static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
     }
     else if (c.bm == 256 && c.bn == 128) launch_mfma<256, 128, MODE>(p, st);
     else if (c.bm == 64 && c.bn == 128) launch_mfma<64, 128, MODE>(p, st);
+    else if ((int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) > 256) launch_mfma<128, 128, MODE, true>(p, st);
     else launch_mfma<128, 128, MODE>(p, st);
 }
 
