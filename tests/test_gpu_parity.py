@@ -134,6 +134,28 @@ def test_a8w8_tile_numbering_many_tile_rows(hip_lib, tile, mn):
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
 
 
+@pytest.mark.parametrize("mnk", [(2080, 2060, 512), (2200, 2100, 1184), (700, 6200, 640)])
+def test_a8w8_128x128_pairs_bit_exact(hip_lib, mnk):
+    """More than 256 tiles of 128x128: the launcher takes the version of the tile that fits two workgroups
+    on a CU (two a-stages, scales staged in the third b-stage before the epilogue).  Accumulators and the
+    scaled 16-bit output, K a multiple of 128 and not."""
+    M, N, K = mnk
+    assert ((M + 127) // 128) * ((N + 127) // 128) > 256
+    a, b = _rand_i8((M, K), 41), _rand_i8((N, K), 42)
+    assert hip_lib.fnn_debug_force_a8w8_tile(128, 128) == 0
+    try:
+        acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+        g = torch.Generator().manual_seed(43)
+        ar = (torch.rand(M, 1, generator=g) * 0.05).half()
+        ac = (torch.rand(1, N, generator=g) * 0.05).half()
+        out = flashnn_amd.GemmA8W8(torch.bfloat16)(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV))
+    finally:
+        hip_lib.fnn_debug_force_a8w8_tile(0, 0)
+    want = O.gemm_a8w8_acc(a.numpy(), b.numpy())
+    assert np.array_equal(acc, want)
+    assert np.array_equal(out.float().cpu().numpy(), O.gemm_a8w8_epilogue_fp32(want, O.to_np(ar), O.to_np(ac), O.BF16))
+
+
 @pytest.mark.parametrize("mnk", [(5, 7, 100), (130, 70, 1000), (64, 64, 8), (33, 65, 129)])
 def test_a8w8_guarded_kernel_bit_exact(mnk):
     M, N, K = mnk
