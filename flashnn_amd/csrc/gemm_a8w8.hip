@@ -611,10 +611,7 @@ static TileChoice choose_tile(int64_t M, int64_t N) {
     // depends on the shape: the 256x128 tile reaches 1.0 at M=2048, K=4096, N=12288, 0.93 at N=22016 and
     // 0.74 at M=K=N=8192; 128x128 0.71 to 0.76; 64x128 0.64 to 0.67 (a 64x128 tile takes 0.55 to 0.6 of
     // the time of a 128x128 one, so it pays where it doubles the workgroups without adding a round).
-    // The 128x128 figure is that of one workgroup per CU.  From 257 tiles on the tile runs two per CU and
-    // reaches 0.85; a model that prices this (and the column split of the 256x192 tile) chose better in
-    // eight of ten shapes tried and worse in a sweep's short-K shapes, so the choice is left as it was and
-    // only shapes that took the 128x128 tile anyway gain.
+    // The 128x128 figure is that of one workgroup per CU; the pairs are priced below.
     double best = 1e300;
     TileChoice c{128, 128};
     for (const auto& t : cand) {
@@ -622,6 +619,16 @@ static TileChoice choose_tile(int64_t M, int64_t N) {
         const int64_t rounds = (tiles + 255) / 256;
         const double cost = (double)rounds * t.bm * t.bn / t.eff;
         if (cost < best) { best = cost; c = {t.bm, t.bn}; }
+    }
+    // The 128x128 tile in pairs (two workgroups per CU from 257 tiles on: a round holds 512 of them at 0.85,
+    // a last round of at most 256 leaves every workgroup a CU of its own and takes 0.64 of a shared one)
+    // replaces a smaller or narrower tile where it is cheaper.  It never replaces the 256x192 tile: the two
+    // shapes where this pricing did so were slower on the box (116 -> 122 us, 118 -> 121 us).
+    const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
+    if (t128 > 256 && !(c.bm == 256 && c.bn == 192)) {
+        const int64_t rem = t128 % 512;
+        const double pair = ((double)(t128 / 512) + (rem == 0 ? 0.0 : rem <= 256 ? 0.64 : 1.0)) * 2.0 * 128 * 128 / 0.85;
+        if (pair < best) c = {128, 128};
     }
     return c;
 }
