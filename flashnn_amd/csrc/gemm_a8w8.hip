@@ -2,7 +2,8 @@
 // out = float(acc) * alpha_row[m] * alpha_col[n]  -> fp16 / bf16   (or the raw int32).
 //
 // Main kernel (K % 32 == 0, K >= 512, 16-byte aligned rows)
-//   * one 256-thread workgroup (4 waves, 2x2) per BM x BN output tile, one workgroup per CU;
+//   * one 256-thread workgroup (4 waves, 2x2) per BM x BN output tile; one workgroup per CU for the
+//     256-row tiles, two for the 64x128 tile and for the pair version of the 128x128 tile;
 //   * K is walked in slabs of 128 bytes.  A slab of the a-rows and b-rows of the tile is
 //     copied global -> LDS with direct-to-LDS 16-byte loads (no VGPR staging) into a ring of
 //     LDS stages, one or two slabs ahead of the MFMAs;
