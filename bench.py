@@ -153,10 +153,15 @@ def main():
     import ctypes
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     sustained = {}
+    probe = ctypes.CDLL(os.path.join(ROOT, "flashnn_amd", "benchmarks", "libfnn_probe.so"))
+    probe.fnn_probe_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                          ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
     for label, rnd in (("random_operand_bytes", 1), ("constant_operands", 0)):
         rate = ctypes.c_double(0.0)
-        _lib.check(_lib.load().fnn_debug_mfma_rate(_lib.ptr(sink), rnd, 2000, 40, ctypes.byref(rate),
-                                                   _lib.current_stream(torch.device(dev))))
+        rc = probe.fnn_probe_mfma_rate(_lib.ptr(sink), rnd, 2000, 40, ctypes.byref(rate),
+                                       _lib.current_stream(torch.device(dev)))
+        if rc != 0:
+            sys.exit(f"bench.py: the MFMA rate probe failed with hipError {rc}")
         sustained[label] = round(rate.value, 1)
     roofline["mfma_only_sustained"] = dict(sustained, unit="TOP/s")
     roofline["frac_of_sustained_random"] = round(gemm_tops / sustained["random_operand_bytes"], 4)

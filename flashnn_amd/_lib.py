@@ -23,14 +23,13 @@ _SIGNATURES = {
     "fnn_layernorm": [_ptr, _ptr, _ptr, _ptr, _f32, _i64, _i64, _i64, _i64, _int, _int, _ptr],
     "fnn_layernorm_dquant": [_ptr, _ptr, _ptr, _ptr, _ptr, _f32, _i64, _i64, _i64, _i64, _int, _int, _ptr],
     "fnn_gemm_a8w8": [_ptr] * 5 + [_i64] * 6 + [_int] * 3 + [_ptr],
-    "fnn_gemm_a8w8_tiled": [_ptr] * 5 + [_i64] * 6 + [_int] * 5 + [_ptr],
+    "fnn_gemm_a8w8_tiled": [_ptr] * 5 + [_i64] * 6 + [_int] * 6 + [_ptr],
     "fnn_gemm_a8w8_i32": [_ptr] * 3 + [_i64] * 6 + [_ptr],
+    "fnn_gemm_a8w8_i32_tiled": [_ptr] * 3 + [_i64] * 6 + [_int] * 3 + [_ptr],
     "fnn_gemm_a16w8": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],
     "fnn_gemm_a16w4": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],
     "fnn_fused_moe_a8w8": [_ptr] * 9 + [_i64] * 9 + [_int] * 7 + [_ptr],
     "fnn_fused_moe_a16w4": [_ptr] * 9 + [_i64] * 14 + [_int] * 8 + [_ptr],
-    "fnn_debug_force_a8w8_tile": [_int, _int],
-    "fnn_debug_mfma_rate": [_ptr, _int, _int, _int, ctypes.POINTER(ctypes.c_double), _ptr],
 }
 _RESTYPE = {"fnn_last_error": ctypes.c_char_p}
 

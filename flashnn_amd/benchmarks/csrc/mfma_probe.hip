@@ -4,11 +4,19 @@
 // the rate is measured for operands of random bytes (what a GEMM on quantised data feeds them) and
 // for constant operands (which reach the datasheet rate).  The A8W8 kernels are judged against the
 // datasheet peak; this number says how much of the gap any kernel can close.
+//
+// Built into libfnn_probe.so, a library of its own that only bench.py loads: it creates events and waits
+// for them, which the product library never does.
+//   int fnn_probe_mfma_rate(void* sink, int random_operands, int iters, int launches, double* tops,
+//                           void* stream);
+// returns 0, or a hipError_t; sink: 4 bytes of device memory (never written); *tops: 1e12 int8
+// operations per second over `launches` kernels of `iters` loop iterations on `stream`.
 #include <hip/hip_runtime.h>
-
-#include "fnn_common.h"
+#include <stdint.h>
 
 namespace fnn {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
     x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
@@ -58,36 +66,31 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(int* __restrict__ sink, 
 
 }  // namespace fnn
 
-extern "C" int fnn_debug_mfma_rate(void* sink, int random_operands, int iters, int launches,
+extern "C" int fnn_probe_mfma_rate(void* sink, int random_operands, int iters, int launches,
                                    double* tops, void* stream) {
     using namespace fnn;
-    if (!sink || !tops || iters <= 0 || launches <= 0) {
-        set_error("fnn_debug_mfma_rate: bad argument");
-        return FNN_ERR_ARG;
-    }
+    if (!sink || !tops || iters <= 0 || launches <= 0) return (int)hipErrorInvalidValue;
     hipStream_t st = (hipStream_t)stream;
     int dev = 0, cus = 0;
     hipEvent_t e0 = nullptr, e1 = nullptr;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
-        set_error("fnn_debug_mfma_rate: %s", hipGetErrorString(hipGetLastError()));
-        return FNN_ERR_HIP;
-    }
+    hipError_t err = hipGetDevice(&dev);
+    if (err == hipSuccess) err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (err == hipSuccess) err = hipEventCreate(&e0);
+    if (err == hipSuccess) err = hipEventCreate(&e1);
+    if (err != hipSuccess) return (int)err;
     const int wgs = cus;   // one wave per SIMD, as in the tiled kernel; the 48 MFMAs of an iteration are independent
     mfma_rate_kernel<<<wgs, 256, 0, st>>>((int*)sink, random_operands, iters);   // warm-up
     (void)hipEventRecord(e0, st);
     for (int l = 0; l < launches; ++l) mfma_rate_kernel<<<wgs, 256, 0, st>>>((int*)sink, random_operands, iters);
     (void)hipEventRecord(e1, st);
     float ms = 0.f;
-    const hipError_t err = hipEventSynchronize(e1) == hipSuccess ? hipEventElapsedTime(&ms, e0, e1) : hipGetLastError();
+    err = hipEventSynchronize(e1);
+    if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
-    if (err != hipSuccess || ms <= 0.f) {
-        set_error("fnn_debug_mfma_rate: %s", hipGetErrorString(err));
-        return FNN_ERR_HIP;
-    }
+    if (err != hipSuccess) return (int)err;
+    if (ms <= 0.f) return (int)hipErrorUnknown;
     // 16x16x64 MFMA = 2 * 16 * 16 * 64 operations; 4 waves per workgroup, 48 MFMAs per iteration
     *tops = (double)wgs * 4 * 48 * (double)iters * launches * 32768.0 / ((double)ms * 1e-3) * 1e-12;
-    return FNN_OK;
+    return 0;
 }

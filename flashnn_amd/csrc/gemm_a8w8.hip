@@ -67,10 +67,12 @@ struct OptionalStage<false, BYTES> {
     static __device__ __forceinline__ char* get() { return nullptr; }
 };
 
-template <int BM, int BN, int MODE, bool PAIR = false>
-__global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
-    constexpr int NWAVES = 4;
-    constexpr int WTM = BM / 2, WTN = BN / 2;
+template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2>
+__global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Args p) {
+    // WGM x 2 waves.  WGM = 4 puts two waves on every SIMD (at most 256 registers each): one can issue
+    // MFMAs while the other waits for LDS fragments, a copy or the barrier.
+    constexpr int NWAVES = WGM * 2, NT = NWAVES * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / 2;
     constexpr int FM = WTM / 16, FN = WTN / 16;   // 16x16 fragments per wave tile
     constexpr int HN = FN / 2;
     static_assert(WTM % 16 == 0 && WTN % 32 == 0, "wave tile must split into 16-row fragments, the weight rows in two halves");
@@ -120,19 +122,19 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wm = wave & 1;
-    const int wn = wave >> 1;
+    const int wm = wave % WGM;
+    const int wn = wave / WGM;
 
     // The tile's scales are requested before anything else, as raw words into registers, and nobody waits
     // for them: they are older than every copy, so they have arrived long before the main loop ends.
     // They are widened and staged in LDS just before the epilogue, which then needs no global loads.
     // (Staged at kernel start, their latency came on top of that of the first copies.)
-    constexpr int NSC = (BM + BN + 255) / 256;
+    constexpr int NSC = (BM + BN + NT - 1) / NT;
     uint32_t sc_raw[NSC];
     if constexpr (MODE != OUT_I32) {
 #pragma unroll
         for (int q = 0; q < NSC; ++q) {
-            const int e = threadIdx.x + q * 256;
+            const int e = threadIdx.x + q * NT;
             const bool is_row = e < BM;
             const int idx = is_row ? min(m0 + e, p.M - 1) : min(n0 + min(e - BM, BN - 1), p.N - 1);
             const void* base = is_row ? p.arow : p.acol;
@@ -459,19 +461,20 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             }
         }
     } else {
-        constexpr int TSTRIDE = WTN * 2 + 16;      // bytes per staged row; the pad staggers the banks
-        constexpr int PR = WTN * 2 / 16;           // 16-byte pieces per row
-        constexpr int RC = FM >= 4 ? 4 : FM;       // 16-row fragments staged at a time
-        static_assert(FM % RC == 0, "staging walks whole groups of fragments");
-        static_assert(RC * 16 * TSTRIDE <= BN * BK && RC * 16 * TSTRIDE <= BM * BK, "transpose buffer must fit a stage");
-        char* tbuf = wave == 0 ? sa0 : wave == 1 ? sa1 : wave == 2 ? (BDEEP ? sb1 : sa2) : sb0;
+        // A lane holds 4 consecutive n of one row m per fragment: 8 bytes.  v_permlane16_swap exchanges the
+        // odd 16-lane rows of one register with the even rows of another; applied to the packed halves
+        // of two neighbouring weight fragments it leaves every lane with 8 consecutive n (16 bytes) of one
+        // of the two, so that a store instruction writes 64 contiguous bytes of each of its 16 rows and
+        // the three instructions of a fragment row the wave's whole 192-byte (WTN * 2) piece of them.  No
+        // LDS transposition, no barrier between the waves.
+        static_assert(FN % 2 == 0, "weight fragments are stored in pairs");
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0x0070);   // all copies and LDS reads of this wave are done
         __builtin_amdgcn_s_barrier();         // ... and everybody else's: the stages are free
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int q = 0; q < NSC; ++q) {
-            const int e = threadIdx.x + q * 256;
+            const int e = threadIdx.x + q * NT;
             const bool is_row = e < BM;
             const int dt = is_row ? p.arow_dtype : p.acol_dtype;
             const float v = dt == FNN_F32 ? __builtin_bit_cast(float, sc_raw[q])
@@ -480,53 +483,58 @@ __global__ __launch_bounds__(256) void gemm_a8w8_ring_kernel(const A8W8Args p) {
             else if (e < BM + BN) sc_col[e - BM] = v;
         }
         __syncthreads();
-        const bool vec_ok = (p.ldc & 7) == 0;
+        const int nsel = (csel & 1) * 16 + (csel >> 1) * 8;   // column of this lane's 16 bytes within a fragment pair
+        v4f ac[FN];
 #pragma unroll
-        for (int jc = 0; jc < FM; jc += RC) {
+        for (int i = 0; i < FN; ++i) ac[i] = *(const v4f*)&sc_col[wn * WTN + i * 16 + 4 * csel];
+        // a tile that lies wholly inside the matrix stores without bounds checks (a uniform choice)
+        const bool inside = m0 + BM <= p.M && n0 + BN <= p.N && (p.ldc & 7) == 0;
+        auto store_rows = [&](auto guarded) {
+            constexpr bool G = decltype(guarded)::value;
+            uint16_t* const obase = (uint16_t*)p.out + (int64_t)(wm0 + frow) * p.ldc + wn0 + nsel;
 #pragma unroll
-            for (int jj = 0; jj < RC; ++jj) {
-                const int j = jc + jj;
+            for (int j = 0; j < FM; ++j) {
                 const float ar = sc_row[wm * WTM + j * 16 + frow];
+                const int m = wm0 + j * 16 + frow;
 #pragma unroll
-                for (int i = 0; i < FN; ++i) {
-                    const int nl = i * 16 + 4 * csel;   // column within the wave tile
-                    const v4f ac = *(const v4f*)&sc_col[wn * WTN + nl];
-                    float v[4];
+                for (int i = 0; i < FN; i += 2) {
+                    uint32_t lo[2], hi[2];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = ((float)acc[i][j][e] * ar) * ac[e];
-                    uint32_t lo, hi;
-                    if constexpr (MODE == OUT_BF16) {
-                        lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2bf));
-                        hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2bf));
-                    } else {
-                        lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2h));
-                        hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2h));
-                    }
-                    *(v2u*)(tbuf + (jj * 16 + frow) * TSTRIDE + nl * 2) = v2u{lo, hi};
-                }
-            }
-            // rows jc*16 .. jc*16 + RC*16 - 1 of the wave tile are staged; write them out row by row
+                    for (int h = 0; h < 2; ++h) {
+                        float v[4];
 #pragma unroll
-            for (int it = 0; it < (RC * 16 * PR + 63) / 64; ++it) {
-                const int e = it * 64 + lane;
-                const int row = e / PR, c = e % PR;
-                if (e < RC * 16 * PR) {
-                    const v4u val = *(const v4u*)(tbuf + row * TSTRIDE + c * 16);
-                    const int m = wm0 + jc * 16 + row;
-                    const int n = wn0 + c * 8;
-                    if (m < p.M && n < p.N) {
-                        uint16_t* o = (uint16_t*)p.out + (int64_t)m * p.ldc + n;
-                        if (n + 7 < p.N && vec_ok) {
-                            __builtin_nontemporal_store(val, (v4u*)o);
+                        for (int e = 0; e < 4; ++e) v[e] = ((float)acc[i + h][j][e] * ar) * ac[i + h][e];
+                        if constexpr (MODE == OUT_BF16) {
+                            lo[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2bf));
+                            hi[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2bf));
                         } else {
+                            lo[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2h));
+                            hi[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2h));
+                        }
+                    }
+                    const v2u sl = __builtin_amdgcn_permlane16_swap(lo[0], lo[1], false, false);
+                    const v2u sh = __builtin_amdgcn_permlane16_swap(hi[0], hi[1], false, false);
+                    const v4u val = v4u{sl[0], sh[0], sl[1], sh[1]};
+                    if constexpr (!G) {
+                        __builtin_nontemporal_store(val, (v4u*)(obase + (int64_t)(j * 16) * p.ldc + i * 16));
+                    } else {
+                        const int n = wn0 + i * 16 + nsel;
+                        if (m < p.M && n < p.N) {
+                            uint16_t* o = (uint16_t*)p.out + (int64_t)m * p.ldc + n;
+                            if (n + 7 < p.N && (p.ldc & 7) == 0) {
+                                __builtin_nontemporal_store(val, (v4u*)o);
+                            } else {
 #pragma unroll
-                            for (int q = 0; q < 8; ++q)
-                                if (n + q < p.N) o[q] = (uint16_t)(val[q >> 1] >> (16 * (q & 1)));
+                                for (int q = 0; q < 8; ++q)
+                                    if (n + q < p.N) o[q] = (uint16_t)(val[q >> 1] >> (16 * (q & 1)));
+                            }
                         }
                     }
                 }
             }
-        }
+        };
+        if (inside) store_rows(std::false_type{});
+        else store_rows(std::true_type{});
     }
 }
 
@@ -634,52 +642,74 @@ static TileChoice choose_tile(int64_t M, int64_t N) {
     return c;
 }
 
-template <int BM, int BN, int MODE, bool PAIR = false>
+template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2>
 static void launch_mfma(A8W8Args& p, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
-    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p);
+    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, WGM><<<dim3(p.tiles_per_xcd * 8), dim3(WGM * 128), 0, st>>>(p);
+}
+
+// The tiles that exist: (rows, columns, waves per workgroup).
+static bool valid_tile(int bm, int bn, int waves) {
+    if (bm == 0 && bn == 0) return waves == 0;
+    if (waves == 0 || waves == 4)
+        return (bm == 256 && (bn == 192 || bn == 128)) || (bm == 128 && bn == 128) || (bm == 64 && bn == 128);
+    if (waves == 8) return bm == 256 && (bn == 256 || bn == 192 || bn == 128);
+    return false;
 }
 
 template <int MODE>
-static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn) {
+static void launch_tile(A8W8Args& p, hipStream_t st, int bm, int bn, int waves) {
+    if (waves == 8) {
+        if (bn == 256) launch_mfma<256, 256, MODE, false, 4>(p, st);
+        else if (bn == 192) launch_mfma<256, 192, MODE, false, 4>(p, st);
+        else launch_mfma<256, 128, MODE, false, 4>(p, st);
+    }
+    else if (bm == 256 && bn == 192) launch_mfma<256, 192, MODE>(p, st);
+    else if (bm == 256 && bn == 128) launch_mfma<256, 128, MODE>(p, st);
+    else if (bm == 64 && bn == 128) launch_mfma<64, 128, MODE>(p, st);
+    else if ((int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) > 256) launch_mfma<128, 128, MODE, true>(p, st);
+    else launch_mfma<128, 128, MODE>(p, st);
+}
+
+template <int MODE>
+static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn, int force_waves) {
     // the MFMA kernel walks K in slabs of 128 bytes and addresses rows with 32-bit offsets
     const bool fast = p.K % 32 == 0 && p.K >= 512 && p.lda % 16 == 0 && p.ldb % 16 == 0 &&
                       ((uintptr_t)p.a % 16) == 0 && ((uintptr_t)p.b % 16) == 0 &&
                       ((uintptr_t)p.out % 16) == 0 && (int64_t)p.M * p.lda < (1LL << 31) &&
                       (int64_t)p.N * p.ldb < (1LL << 31);
-    // few activation rows: stream the weights once (unless a test forces a tile of the tiled kernel)
+    // few activation rows: stream the weights once (unless the caller names a tile of the tiled kernel)
     if (force_bm == 0 && p.M <= 64 && launch_a8w8_skinny(p, MODE, st)) return;
     if (!fast) {
         gemm_a8w8_any_kernel<MODE><<<dim3((p.N + 63) / 64, (p.M + 63) / 64), dim3(256), 0, st>>>(p);
         return;
     }
-    TileChoice c = choose_tile(p.M, p.N);
-    if (force_bm > 0) c = {force_bm, force_bn};
+    if (force_bm > 0) {
+        launch_tile<MODE>(p, st, force_bm, force_bn, force_waves);
+        return;
+    }
+    const TileChoice c = choose_tile(p.M, p.N);
     if (c.bm == 256 && c.bn == 192) {
-        const int c1 = force_bm == 0 ? split_columns_192(p.M, p.N) : 0;
+        const int c1 = split_columns_192(p.M, p.N);
         if (c1 > 0) {
             // columns [0, 192 c1) in 192-wide tiles, the rest in 128-wide ones
             A8W8Args q = p;
             q.N = 192 * c1;
-            launch_mfma<256, 192, MODE>(q, st);
+            launch_tile<MODE>(q, st, 256, 192, 0);
             const int64_t n_off = q.N;
             q = p;
             q.N = p.N - (int)n_off;
             q.b = p.b + n_off * p.ldb;
             q.out = (char*)p.out + n_off * (MODE == OUT_I32 ? 4 : 2);
             if (p.acol) q.acol = (const char*)p.acol + n_off * (p.acol_dtype == FNN_F32 ? 4 : 2);
-            launch_mfma<256, 128, MODE>(q, st);
-        } else {
-            launch_mfma<256, 192, MODE>(p, st);
+            launch_tile<MODE>(q, st, 256, 128, 0);
+            return;
         }
     }
-    else if (c.bm == 256 && c.bn == 128) launch_mfma<256, 128, MODE>(p, st);
-    else if (c.bm == 64 && c.bn == 128) launch_mfma<64, 128, MODE>(p, st);
-    else if ((int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) > 256) launch_mfma<128, 128, MODE, true>(p, st);
-    else launch_mfma<128, 128, MODE>(p, st);
+    launch_tile<MODE>(p, st, c.bm, c.bn, 0);
 }
 
 static int check_args(const char* fn, const void* out, const void* a, const void* b, int64_t M,
@@ -702,39 +732,43 @@ static int check_args(const char* fn, const void* out, const void* a, const void
 
 using namespace fnn;
 
-static bool valid_tile(int bm, int bn);
-
-// Test hook: force a tile shape (bm, bn) for the next calls on any thread; (0, 0) = automatic.
-static int g_force_bm = 0, g_force_bn = 0;
-extern "C" int fnn_debug_force_a8w8_tile(int bm, int bn) {
-    if (!valid_tile(bm, bn)) { set_error("fnn_debug_force_a8w8_tile: no such tile %dx%d", bm, bn); return FNN_ERR_ARG; }
-    g_force_bm = bm;
-    g_force_bn = bn;
-    return FNN_OK;
-}
-
-static bool valid_tile(int bm, int bn) {
-    return (bm == 0 && bn == 0) || (bm == 256 && (bn == 192 || bn == 128)) || (bm == 128 && bn == 128) ||
-           (bm == 64 && bn == 128);
-}
-
 static int gemm_a8w8_entry(const char* fn, void* out, const void* a, const void* b, const void* alpha_row,
                            const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                            int64_t ldc, int out_dtype, int alpha_row_dtype, int alpha_col_dtype, int tile_m,
-                           int tile_n, void* stream) {
+                           int tile_n, int waves, void* stream) {
     int rc = check_args(fn, out, a, b, M, N, K, lda, ldb, ldc);
     if (rc != FNN_OK) return rc;
     if (M != 0 && N != 0 && (!alpha_row || !alpha_col)) { set_error("%s: null scale pointer", fn); return FNN_ERR_ARG; }
     if (!is16(out_dtype)) { set_error("%s: Output type must be float16 or bfloat16", fn); return FNN_ERR_UNSUPPORTED; }
     if (!isflt(alpha_row_dtype) || !isflt(alpha_col_dtype)) { set_error("%s: bad scale type", fn); return FNN_ERR_UNSUPPORTED; }
-    if (!valid_tile(tile_m, tile_n)) { set_error("%s: no such tile %dx%d", fn, tile_m, tile_n); return FNN_ERR_ARG; }
+    if (!valid_tile(tile_m, tile_n, waves)) {
+        set_error("%s: no such tile %dx%d with %d waves", fn, tile_m, tile_n, waves);
+        return FNN_ERR_ARG;
+    }
     if (M == 0 || N == 0) return FNN_OK;
     A8W8Args p{};
     p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = out; p.arow = alpha_row; p.acol = alpha_col;
     p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
     p.out_dtype = out_dtype; p.arow_dtype = alpha_row_dtype; p.acol_dtype = alpha_col_dtype;
-    if (out_dtype == FNN_F16) dispatch<OUT_F16>(p, (hipStream_t)stream, tile_m, tile_n);
-    else dispatch<OUT_BF16>(p, (hipStream_t)stream, tile_m, tile_n);
+    if (out_dtype == FNN_F16) dispatch<OUT_F16>(p, (hipStream_t)stream, tile_m, tile_n, waves);
+    else dispatch<OUT_BF16>(p, (hipStream_t)stream, tile_m, tile_n, waves);
+    return check_launch(fn);
+}
+
+static int gemm_a8w8_i32_entry(const char* fn, int32_t* acc, const void* a, const void* b, int64_t M, int64_t N,
+                               int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int tile_m, int tile_n,
+                               int waves, void* stream) {
+    int rc = check_args(fn, acc, a, b, M, N, K, lda, ldb, ldc);
+    if (rc != FNN_OK) return rc;
+    if (!valid_tile(tile_m, tile_n, waves)) {
+        set_error("%s: no such tile %dx%d with %d waves", fn, tile_m, tile_n, waves);
+        return FNN_ERR_ARG;
+    }
+    if (M == 0 || N == 0) return FNN_OK;
+    A8W8Args p{};
+    p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = acc;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    dispatch<OUT_I32>(p, (hipStream_t)stream, tile_m, tile_n, waves);
     return check_launch(fn);
 }
 
@@ -743,27 +777,27 @@ extern "C" int fnn_gemm_a8w8(void* out, const void* a, const void* b, const void
                              int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
                              int alpha_col_dtype, void* stream) {
     return gemm_a8w8_entry("fnn_gemm_a8w8", out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc, out_dtype,
-                           alpha_row_dtype, alpha_col_dtype, g_force_bm, g_force_bn, stream);
+                           alpha_row_dtype, alpha_col_dtype, 0, 0, 0, stream);
 }
 
 extern "C" int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, const void* alpha_row,
                                    const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
                                    int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
-                                   int alpha_col_dtype, int tile_m, int tile_n, void* stream) {
+                                   int alpha_col_dtype, int tile_m, int tile_n, int waves, void* stream) {
     return gemm_a8w8_entry("fnn_gemm_a8w8_tiled", out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc, out_dtype,
-                           alpha_row_dtype, alpha_col_dtype, tile_m, tile_n, stream);
+                           alpha_row_dtype, alpha_col_dtype, tile_m, tile_n, waves, stream);
 }
 
 extern "C" int fnn_gemm_a8w8_i32(int32_t* acc, const void* a, const void* b, int64_t M, int64_t N,
                                  int64_t K, int64_t lda, int64_t ldb, int64_t ldc, void* stream) {
-    int rc = check_args("fnn_gemm_a8w8_i32", acc, a, b, M, N, K, lda, ldb, ldc);
-    if (rc != FNN_OK) return rc;
-    if (M == 0 || N == 0) return FNN_OK;
-    A8W8Args p{};
-    p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = acc;
-    p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
-    dispatch<OUT_I32>(p, (hipStream_t)stream, g_force_bm, g_force_bn);
-    return check_launch("fnn_gemm_a8w8_i32");
+    return gemm_a8w8_i32_entry("fnn_gemm_a8w8_i32", acc, a, b, M, N, K, lda, ldb, ldc, 0, 0, 0, stream);
+}
+
+extern "C" int fnn_gemm_a8w8_i32_tiled(int32_t* acc, const void* a, const void* b, int64_t M, int64_t N,
+                                       int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int tile_m, int tile_n,
+                                       int waves, void* stream) {
+    return gemm_a8w8_i32_entry("fnn_gemm_a8w8_i32_tiled", acc, a, b, M, N, K, lda, ldb, ldc, tile_m, tile_n, waves,
+                               stream);
 }
 
 extern "C" int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const void* alpha_row,

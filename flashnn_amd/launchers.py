@@ -120,11 +120,13 @@ def _flat_scale(t, n, what):
     return t if t.is_contiguous() else t.contiguous()
 
 
-def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col):
+def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col, tile=None):
     """Replaces triton_gemm_a8w8_forward (flashnn/triton_kernels/gemm_a8w8.py:182-221).
 
     Unlike the Triton launcher the scale type need not equal the output type: fp16, bf16 and
-    fp32 scales are accepted in any combination."""
+    fp32 scales are accepted in any combination.  `tile` = (rows, columns, waves) names a tile of
+    the MFMA kernel and bypasses the tuned-configuration lookup (not part of the reference's
+    signature; the results are the same bits for every tile)."""
     assert a.dtype == torch.int8 and b.dtype == torch.int8, "Matrix A/B must be int8 type"
     assert a.is_contiguous(), "Matrix A must be contiguous"
     assert out.dtype == torch.float16 or out.dtype == torch.bfloat16, \
@@ -146,19 +148,22 @@ def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col):
     stream = _lib.current_stream(a.device)
     # shape-keyed tuned tile, named as the reference names the launch (gemm_a8w8.py:199)
     method_name = f"gemm_a8w8_{M}_{N}_{K}"
-    tile = tuned_configs.CACHE.lookup(method_name)
+    if tile is None:
+        tile = tuned_configs.CACHE.lookup(method_name)
     if tile is None and get_autotune_triton_kernels():
         tile = tuned_configs.tune(method_name, tuned_configs.A8W8_CANDIDATES,
-                                  lambda t: _lib.check(lib.fnn_gemm_a8w8_tiled(*args, t[0], t[1], stream)))
-    if tile is None or tile == (0, 0):
+                                  lambda t: _lib.check(lib.fnn_gemm_a8w8_tiled(*args, *t, stream)))
+    if tile is None or tile[0] == 0:
         _lib.check(lib.fnn_gemm_a8w8(*args, stream))
     else:
-        _lib.check(lib.fnn_gemm_a8w8_tiled(*args, tile[0], tile[1], stream))
+        _lib.check(lib.fnn_gemm_a8w8_tiled(*args, *tile, stream))
     return out
 
 
-def hip_gemm_a8w8_int32(a, b):
-    """Raw int32 accumulators of the A8W8 contraction (no reference launcher; parity hook)."""
+def hip_gemm_a8w8_int32(a, b, tile=(0, 0, 0)):
+    """Raw int32 accumulators of the A8W8 contraction (no reference launcher; parity hook).
+    `tile` = (rows, columns, waves) names a tile of the MFMA kernel; (0, 0, 0) leaves the choice to the
+    library."""
     assert a.dtype == torch.int8 and b.dtype == torch.int8, "Matrix A/B must be int8 type"
     assert a.is_contiguous() and b.is_contiguous() and a.shape[1] == b.shape[1]
     _lib.require_gpu(a, b)
@@ -166,8 +171,8 @@ def hip_gemm_a8w8_int32(a, b):
     M, K = a.shape
     N = b.shape[0]
     acc = torch.empty((M, N), dtype=torch.int32, device=a.device)
-    _lib.check(lib.fnn_gemm_a8w8_i32(_lib.ptr(acc), _lib.ptr(a), _lib.ptr(b), M, N, K, K, K, N,
-                                     _lib.current_stream(a.device)))
+    _lib.check(lib.fnn_gemm_a8w8_i32_tiled(_lib.ptr(acc), _lib.ptr(a), _lib.ptr(b), M, N, K, K, K, N, *tile,
+                                           _lib.current_stream(a.device)))
     return acc
 
 

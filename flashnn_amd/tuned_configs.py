@@ -10,7 +10,8 @@ processes, the recorded configuration is used without timing anything.  With tun
 recorded configurations are still honoured; shapes without one take the library's static choice.
 
 File format (the reference's, triton_utils.py:38-57): {method_name: [kwargs, launch_options]} with
-kwargs = {"BLOCK_M": .., "BLOCK_N": ..} ((0, 0) = the library's own choice) and launch_options = {}.
+kwargs = {"BLOCK_M": .., "BLOCK_N": ..} ((0, 0) = the library's own choice) and launch_options =
+{"num_warps": 4 or 8} (absent = the tile's default), the reference's own option names (gemm_a8w8.py:17-50).
 The file lives at $FLASHNN_AMD_TUNED_CONFIGS or flashnn_amd/configs/hip_autotune_best_configs.json.
 FORECE_RE_TUNE_TRITON_KERNELS (the reference's spelling, triton_utils.py:22-24) lists method-name
 prefixes, separated by ';', that are tuned again even if recorded.
@@ -21,8 +22,10 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 JSON_FILENAME = "hip_autotune_best_configs.json"
 
-# candidate output tiles of the A8W8 MFMA kernel; (0, 0) = static choice (which may be a few-row kernel)
-A8W8_CANDIDATES = [(0, 0), (256, 192), (256, 128), (128, 128), (64, 128)]
+# candidate (rows, columns, waves) of the A8W8 MFMA kernel; (0, 0, 0) = static choice (which may be a
+# few-row kernel); waves = 0 is the tile's default (four)
+A8W8_CANDIDATES = [(0, 0, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0),
+                   (256, 256, 8), (256, 192, 8), (256, 128, 8)]
 
 
 def json_file_path():
@@ -38,12 +41,13 @@ def force_re_tune(method_name):
 
 
 def serialize_best_config(tile):
-    return [{"BLOCK_M": int(tile[0]), "BLOCK_N": int(tile[1])}, {}]
+    waves = int(tile[2]) if len(tile) > 2 else 0
+    return [{"BLOCK_M": int(tile[0]), "BLOCK_N": int(tile[1])}, {"num_warps": waves} if waves else {}]
 
 
 def deserialize_best_config(entry):
-    kwargs = entry[0]
-    return int(kwargs["BLOCK_M"]), int(kwargs["BLOCK_N"])
+    kwargs, options = entry[0], entry[1] if len(entry) > 1 else {}
+    return int(kwargs["BLOCK_M"]), int(kwargs["BLOCK_N"]), int(options.get("num_warps", 0))
 
 
 class TunedConfigs:

@@ -149,17 +149,25 @@ int fnn_layernorm_dquant(void* q, void* scale, const void* x, const void* gamma,
                          int gb_dtype, void* stream);
 
 /*
- * fnn_gemm_a8w8 with the output tile of the MFMA kernel chosen by the caller: (tile_m, tile_n) one of
- * 256x192, 256x128, 128x128, 64x128, or (0, 0) for the library's own choice.  A forced tile also bypasses the
- * few-row kernels.  This is what a shape-keyed tuned-configuration cache calls - the role that
- * compile_and_cache_kernels and its JSON file play in the reference
- * (flashnn/triton_kernels/triton_utils.py:84-151; method name "gemm_a8w8_M_N_K", gemm_a8w8.py:199).
+ * fnn_gemm_a8w8 with the output tile of the MFMA kernel chosen by the caller: (tile_m, tile_n, waves) with
+ * waves = 4 (or 0: the tile's default) and the tile one of 256x192, 256x128, 128x128, 64x128, or waves = 8
+ * (two wavefronts on every SIMD) and the tile one of 256x256, 256x192, 256x128; (0, 0, 0) is the library's
+ * own choice.  A named tile also bypasses the few-row kernels.  This is what a shape-keyed
+ * tuned-configuration cache calls - the role that compile_and_cache_kernels and its JSON file play in the
+ * reference (flashnn/triton_kernels/triton_utils.py:84-151; method name "gemm_a8w8_M_N_K",
+ * gemm_a8w8.py:199; `waves` is the num_warps of its launch options, gemm_a8w8.py:17-50).
  * Results are bit-identical for every tile.
  */
 int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, const void* alpha_row,
                         const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
                         int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
-                        int alpha_col_dtype, int tile_m, int tile_n, void* stream);
+                        int alpha_col_dtype, int tile_m, int tile_n, int waves, void* stream);
+
+/* fnn_gemm_a8w8_i32 through a named tile (same tiles as fnn_gemm_a8w8_tiled): lets a test check the integer
+ * result of every tile bit for bit.  No counterpart in the reference API. */
+int fnn_gemm_a8w8_i32_tiled(int32_t* acc, const void* a, const void* b, int64_t M, int64_t N, int64_t K,
+                            int64_t lda, int64_t ldb, int64_t ldc, int tile_m, int tile_n, int waves,
+                            void* stream);
 
 /*
  * Replaces fused_moe_a8w8_forward(A, B, C, alpha_row_ptr, alpha_col_ptr, topk_weights, topk_ids,
@@ -218,27 +226,6 @@ int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const void* scale
                         int64_t stride_scale_k, int64_t stride_zp_be, int64_t stride_zp_n,
                         int64_t stride_zp_k, int group, int mul_routed_weight, int top_k, int block_m,
                         int act_dtype, int scale_dtype, int zp_dtype, int topk_weights_dtype,
-                        void* stream);
-
-/*
- * Test hook, no counterpart in the reference: force the output tile (bm x bn) of the MFMA
- * A8W8 kernel for subsequent calls, so that every tile shape can be checked on small
- * problems; (0, 0) restores the automatic choice.  Valid tiles: 256x192, 256x128, 128x128, 64x128.  Process-wide and not synchronised: for tests only.
- */
-int fnn_debug_force_a8w8_tile(int bm, int bn);
-
-/*
- * Measurement aid, no counterpart in the reference: the rate, in 1e12 int8 operations per second,
- * at which the current device sustains back-to-back 16x16x64 int8 MFMAs with operands held in
- * registers, in the shape and order of the tiled A8W8 kernel's 256x192 tile (one wave per SIMD, 6 weight
- * fragments against 8 activation fragments, the weight fragment fixed over the inner loop; no memory
- * traffic).  random_operands != 0 feeds the matrix cores
- * random bytes, as a GEMM on quantised data does; 0 feeds constants.  The clock follows the power
- * drawn, and that follows the toggling of the operand bits, so the two rates differ; the first is the
- * ceiling an A8W8 GEMM can approach on this device.  Runs 1 + launches kernels of `iters` loop
- * iterations on `stream` and waits for them.  sink: 4 bytes of device memory (never written).
- */
-int fnn_debug_mfma_rate(void* sink, int random_operands, int iters, int launches, double* tops,
                         void* stream);
 
 #ifdef __cplusplus

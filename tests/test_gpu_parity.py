@@ -82,75 +82,72 @@ def _rand_i8(shape, seed, lo=-128, hi=128):
     return torch.randint(lo, hi, shape, generator=g, dtype=torch.int8)
 
 
-@pytest.mark.parametrize("tile", [(0, 0), (256, 192), (256, 128), (128, 128), (64, 128)])
+# every tile of the MFMA kernel: (rows, columns, waves); (0, 0, 0) = the library's own choice
+TILES = [(0, 0, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0), (256, 256, 8), (256, 192, 8),
+         (256, 128, 8)]
+
+
+def _scaled(out_ty, a, b, ar, ac, tile):
+    out = torch.empty((a.shape[0], b.shape[0]), dtype=out_ty, device=a.device)
+    return launchers.hip_gemm_a8w8_forward(out, a, b, ar, ac, tile=tile)
+
+
+@pytest.mark.parametrize("tile", TILES)
 @pytest.mark.parametrize("mnk", [(128, 128, 128), (300, 200, 512), (512, 768, 1024), (16, 4096, 4096),
                                  (257, 129, 640), (64, 320, 1152), (130, 100, 2048)])
-def test_a8w8_accumulators_bit_exact(hip_lib, tile, mnk):
+def test_a8w8_accumulators_bit_exact(tile, mnk):
     M, N, K = mnk
     a, b = _rand_i8((M, K), 1), _rand_i8((N, K), 2)
-    assert hip_lib.fnn_debug_force_a8w8_tile(*tile) == 0
-    try:
-        acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
-    finally:
-        hip_lib.fnn_debug_force_a8w8_tile(0, 0)
+    acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV), tile).cpu().numpy()
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
 
 
-@pytest.mark.parametrize("tile", [(0, 0), (256, 192), (256, 128), (128, 128), (64, 128)])
+@pytest.mark.parametrize("tile", TILES)
 @pytest.mark.parametrize("mnk", [(300, 200, 544), (257, 385, 576), (64, 320, 608), (130, 100, 1056),
                                  (10, 1920, 1760), (40, 260, 7392), (520, 390, 8896)])
-def test_a8w8_partial_last_slab_bit_exact(hip_lib, tile, mnk):
+def test_a8w8_partial_last_slab_bit_exact(tile, mnk):
     """K a multiple of 32 but not of 128 (the FFN shapes of models sharded over 4 or 8 GPUs): the
     last 128-byte slab holds one to three k-steps; few-row problems take the tiled kernel too."""
     M, N, K = mnk
     a, b = _rand_i8((M, K), 21), _rand_i8((N, K), 22)
-    assert hip_lib.fnn_debug_force_a8w8_tile(*tile) == 0
-    try:
-        acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
-        g = torch.Generator().manual_seed(23)
-        ar = (torch.rand(M, 1, generator=g) * 0.05).half()
-        ac = (torch.rand(1, N, generator=g) * 0.05).half()
-        out = flashnn_amd.GemmA8W8(torch.float16)(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV))
-    finally:
-        hip_lib.fnn_debug_force_a8w8_tile(0, 0)
+    acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV), tile).cpu().numpy()
+    g = torch.Generator().manual_seed(23)
+    ar = (torch.rand(M, 1, generator=g) * 0.05).half()
+    ac = (torch.rand(1, N, generator=g) * 0.05).half()
+    out = _scaled(torch.float16, a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV), tile if tile[0] else None)
     want = O.gemm_a8w8_acc(a.numpy(), b.numpy())
     assert np.array_equal(acc, want)
     assert np.array_equal(out.float().cpu().numpy(), O.gemm_a8w8_epilogue_fp32(want, O.to_np(ar), O.to_np(ac), O.F16))
 
 
-@pytest.mark.parametrize("tile,mn", [((64, 128), (720, 773)), ((64, 128), (1100, 300)), ((128, 128), (1290, 650)),
-                                     ((256, 128), (2310, 1100)), ((256, 192), (2400, 1000)), ((256, 192), (2600, 200))])
-def test_a8w8_tile_numbering_many_tile_rows(hip_lib, tile, mn):
+@pytest.mark.parametrize("tile,mn", [((64, 128, 0), (720, 773)), ((64, 128, 0), (1100, 300)),
+                                     ((128, 128, 0), (1290, 650)), ((256, 128, 0), (2310, 1100)),
+                                     ((256, 192, 0), (2400, 1000)), ((256, 192, 0), (2600, 200)),
+                                     ((256, 192, 8), (2400, 1000)), ((256, 256, 8), (2600, 1300)),
+                                     ((256, 128, 8), (2310, 1100))])
+def test_a8w8_tile_numbering_many_tile_rows(tile, mn):
     """More than 8 tile rows and a number of tile columns that is no multiple of 4: the tiles are numbered
     in groups of 4 tile columns, and the last group is narrower."""
     M, N = mn
     K = 512
     a, b = _rand_i8((M, K), 31), _rand_i8((N, K), 32)
-    assert hip_lib.fnn_debug_force_a8w8_tile(*tile) == 0
-    try:
-        acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
-    finally:
-        hip_lib.fnn_debug_force_a8w8_tile(0, 0)
+    acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV), tile).cpu().numpy()
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
 
 
 @pytest.mark.parametrize("mnk", [(2080, 2060, 512), (2200, 2100, 1184), (700, 6200, 640)])
-def test_a8w8_128x128_pairs_bit_exact(hip_lib, mnk):
+def test_a8w8_128x128_pairs_bit_exact(mnk):
     """More than 256 tiles of 128x128: the launcher takes the version of the tile that fits two workgroups
     on a CU (two a-stages, scales staged in the third b-stage before the epilogue).  Accumulators and the
     scaled 16-bit output, K a multiple of 128 and not."""
     M, N, K = mnk
     assert ((M + 127) // 128) * ((N + 127) // 128) > 256
     a, b = _rand_i8((M, K), 41), _rand_i8((N, K), 42)
-    assert hip_lib.fnn_debug_force_a8w8_tile(128, 128) == 0
-    try:
-        acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
-        g = torch.Generator().manual_seed(43)
-        ar = (torch.rand(M, 1, generator=g) * 0.05).half()
-        ac = (torch.rand(1, N, generator=g) * 0.05).half()
-        out = flashnn_amd.GemmA8W8(torch.bfloat16)(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV))
-    finally:
-        hip_lib.fnn_debug_force_a8w8_tile(0, 0)
+    acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV), (128, 128, 0)).cpu().numpy()
+    g = torch.Generator().manual_seed(43)
+    ar = (torch.rand(M, 1, generator=g) * 0.05).half()
+    ac = (torch.rand(1, N, generator=g) * 0.05).half()
+    out = _scaled(torch.bfloat16, a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV), (128, 128, 0))
     want = O.gemm_a8w8_acc(a.numpy(), b.numpy())
     assert np.array_equal(acc, want)
     assert np.array_equal(out.float().cpu().numpy(), O.gemm_a8w8_epilogue_fp32(want, O.to_np(ar), O.to_np(ac), O.BF16))

@@ -154,29 +154,34 @@ def test_tuned_config_file_format_and_lookup(tmp_path, monkeypatch):
     monkeypatch.delenv("FORECE_RE_TUNE_TRITON_KERNELS", raising=False)
     cache = TC.TunedConfigs()
     assert cache.lookup("gemm_a8w8_2048_12288_4096") is None
-    cache.record("gemm_a8w8_2048_12288_4096", (256, 192))
-    cache.record("gemm_a8w8_16_4096_4096", (0, 0))
+    cache.record("gemm_a8w8_2048_12288_4096", (256, 192, 8))
+    cache.record("gemm_a8w8_16_4096_4096", (0, 0, 0))
     data = json.load(open(path))
-    assert data == {"gemm_a8w8_2048_12288_4096": [{"BLOCK_M": 256, "BLOCK_N": 192}, {}],
+    assert data == {"gemm_a8w8_2048_12288_4096": [{"BLOCK_M": 256, "BLOCK_N": 192}, {"num_warps": 8}],
                     "gemm_a8w8_16_4096_4096": [{"BLOCK_M": 0, "BLOCK_N": 0}, {}]}
     # a fresh view (another process) reads the file back
     other = TC.TunedConfigs()
-    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 192) and other.lookup("gemm_a8w8_1_1_1") is None
+    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 192, 8) and other.lookup("gemm_a8w8_1_1_1") is None
     # forced re-tune by method-name prefix, once per process
     monkeypatch.setenv("FORECE_RE_TUNE_TRITON_KERNELS", "gemm_a8w8_2048;fuse_moe")
     assert TC.force_re_tune("gemm_a8w8_2048_12288_4096") and not TC.force_re_tune("gemm_a8w8_16_4096_4096")
-    assert other.lookup("gemm_a8w8_2048_12288_4096") is None and other.lookup("gemm_a8w8_16_4096_4096") == (0, 0)
-    other.record("gemm_a8w8_2048_12288_4096", (256, 128))
-    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 128)
+    assert other.lookup("gemm_a8w8_2048_12288_4096") is None and other.lookup("gemm_a8w8_16_4096_4096") == (0, 0, 0)
+    other.record("gemm_a8w8_2048_12288_4096", (256, 128, 0))
+    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 128, 0)
     assert TC.serialize_best_config((128, 128)) == [{"BLOCK_M": 128, "BLOCK_N": 128}, {}]
-    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 192}, {}]) == (256, 192)
+    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 192}, {}]) == (256, 192, 0)
+    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 256}, {"num_warps": 8}]) == (256, 256, 8)
 
 
 def test_tiled_entry_rejects_unknown_tiles(hip_lib):
     one = ctypes.c_void_p(16)
     null = ctypes.c_void_p(0)
-    rc = hip_lib.fnn_gemm_a8w8_tiled(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 0, 0, 0, 64, 64, null)
+    rc = hip_lib.fnn_gemm_a8w8_tiled(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 0, 0, 0, 64, 64, 0, null)
     assert rc == -1 and b"no such tile 64x64" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a8w8_tiled(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 0, 0, 0, 128, 128, 8, null)
+    assert rc == -1 and b"no such tile 128x128 with 8 waves" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a8w8_i32_tiled(one, one, one, 4, 4, 128, 128, 128, 4, 256, 256, 4, null)
+    assert rc == -1 and b"no such tile 256x256 with 4 waves" in hip_lib.fnn_last_error()
 
 
 def test_empty_calls_need_no_addresses(hip_lib):
