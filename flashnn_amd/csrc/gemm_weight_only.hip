@@ -447,8 +447,12 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_kernel(const Wo
 //   * sign flip, nibble mask and exponent insertion are one 3-input bit operation;
 //   * the wave index is made scalar so the K loop is scalar control flow, the weight
 //     address is a scalar base plus a per-lane 32-bit offset.
-template <int WBITS, int ADT, bool G128, int MP, int CH, bool FULL>
+// REFQ (1, or 2 with zero points; fp16 activations, per-channel fp16 scales and zero points): every weight is dequantised and rounded
+// to fp16 as the reference's torch path does before the dot product (ref_dq_f16), and the scale tables, the
+// MFMAs against ones and the fold are not needed.
+template <int WBITS, int ADT, bool G128, int MP, int CH, bool FULL, int REFQ = 0>
 __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(const WoArgs p) {
+    static_assert(!REFQ || (ADT == FNN_F16 && !G128), "reference rounding: fp16, per-channel");
     typedef MfmaT<ADT> MT;
     constexpr int NH = WBITS == 4 ? 2 : 1;
     constexpr int NC = 8 * NH;
@@ -496,10 +500,28 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
         const char* base = w_tile + (int64_t)min(step, s_end - 1) * 128;   // scalar
         return __builtin_nontemporal_load((const v4u*)(base + w_off));
     };
+    // REFQ: the scale and zero point of this lane's weight row (two channels per row with int4 weights),
+    // requested ahead of the weights: loads return in order, and the first conversion needs them
+    uint32_t rq_sb[NH], rq_zb[NH];
+    if constexpr (REFQ) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h) {
+            const int n = min(n0 + j7 * NH + h, p.N - 1);
+            rq_sb[h] = ((const uint16_t*)p.scale)[n];
+            rq_zb[h] = REFQ == 2 ? ((const uint16_t*)p.zp)[n] : 0u;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
     v4u wq[UN];
     if (s_begin < s_end) {
 #pragma unroll
         for (int i = 0; i < UN; ++i) wq[i] = load_w(s_begin + i);
+    }
+    v2h rq_s[NH], rq_z[NH];
+    const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
+    if constexpr (REFQ) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h) { rq_s[h] = pair_of_f16_bits(rq_sb[h]); rq_z[h] = pair_of_f16_bits(rq_zb[h]); }
     }
 
     for (int e = threadIdx.x; e < ZERO_BYTES / 4; e += kDecWaves * 64) ((uint32_t*)smem)[e] = 0;
@@ -516,8 +538,10 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
         for (int u = 0; u < 4; ++u) v_first[u] = src[min(u * NT + (int)threadIdx.x, chunks - 1)];
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (p.scale_dtype == FNN_F16) fill_scales_lds<FNN_F16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
-    else fill_scales_lds<FNN_BF16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
+    if constexpr (!REFQ) {
+        if (p.scale_dtype == FNN_F16) fill_scales_lds<FNN_F16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
+        else fill_scales_lds<FNN_BF16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
+    }
     {
         for (int m = 0; m < p.M; ++m) {
             const v4u* src = (const v4u*)((const uint16_t*)p.act + (int64_t)m * p.lda);
@@ -559,6 +583,11 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     const v4f zero4 = v4f{0, 0, 0, 0};
 
     auto fold = [&](uint32_t addr) {
+        if constexpr (REFQ) {
+#pragma unroll
+            for (int h = 0; h < NH; ++h) outv[h] = accg[h];
+            return;
+        }
         float sv[NH * 4], zv[NH * 4];
 #pragma unroll
         for (int q = 0; q < NH; ++q) {
@@ -598,20 +627,30 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
                     // refill the queue slot only after its old value is dead, so that both live
                     // in the same registers
                     if (i + UN < CH) wq[i % UN] = load_w(step + UN);
+                    if constexpr (REFQ) {
+                        e0 = ref_dq_f16<REFQ == 2>(e0, rq_c, rq_z[0], rq_s[0]);
+                        e1 = ref_dq_f16<REFQ == 2>(e1, rq_c, rq_z[0], rq_s[0]);
+                        o0 = ref_dq_f16<REFQ == 2>(o0, rq_c, rq_z[NH - 1], rq_s[NH - 1]);
+                        o1 = ref_dq_f16<REFQ == 2>(o1, rq_c, rq_z[NH - 1], rq_s[NH - 1]);
+                    }
                     accg[0] = MT::mma(e0, a0, first ? zero4 : accg[0]);
                     accg[1] = MT::mma(o0, a0, first ? zero4 : accg[1]);
-                    asum = MT::mma(ones, a0, first ? zero4 : asum);
+                    if constexpr (!REFQ) asum = MT::mma(ones, a0, first ? zero4 : asum);
                     accg[0] = MT::mma(e1, a1, accg[0]);
                     accg[1] = MT::mma(o1, a1, accg[1]);
-                    asum = MT::mma(ones, a1, asum);
+                    if constexpr (!REFQ) asum = MT::mma(ones, a1, asum);
                 } else {
                     v4u s0, s1;
                     convert_w8<ADT>(w, s0, s1);
                     if (i + UN < CH) wq[i % UN] = load_w(step + UN);
+                    if constexpr (REFQ) {
+                        s0 = ref_dq_f16<REFQ == 2>(s0, rq_c, rq_z[0], rq_s[0]);
+                        s1 = ref_dq_f16<REFQ == 2>(s1, rq_c, rq_z[0], rq_s[0]);
+                    }
                     accg[0] = MT::mma(s0, a0, first ? zero4 : accg[0]);
-                    asum = MT::mma(ones, a0, first ? zero4 : asum);
+                    if constexpr (!REFQ) asum = MT::mma(ones, a0, first ? zero4 : asum);
                     accg[0] = MT::mma(s1, a1, accg[0]);
-                    asum = MT::mma(ones, a1, asum);
+                    if constexpr (!REFQ) asum = MT::mma(ones, a1, asum);
                 }
                 if constexpr (G128) {
                     if (i % GS == GS - 1 || (!FULL && step + 1 == s_end))
@@ -1004,13 +1043,22 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
         const int steps = p.K / 128;
         const bool full16 = steps % (kDecWaves * 16) == 0, full8 = steps % (kDecWaves * 8) == 0;
         const size_t smem = fixed + act_bytes + 16 * 256 + 32;
-#define FNN_DEC(G, MPV)                                                                              \
+        if (smem > 64 * 1024) return false;   // beyond what a launch may ask for without raising the kernel's limit
+#define FNN_DEC(G, MPV, ...)                                                                         \
     do {                                                                                             \
-        if (full16) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, true><<<grid, block, smem, st>>>(p); \
-        else if (full8) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 8, true><<<grid, block, smem, st>>>(p); \
-        else gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, false><<<grid, block, smem, st>>>(p);  \
+        if (full16) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, true, ##__VA_ARGS__><<<grid, block, smem, st>>>(p); \
+        else if (full8) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 8, true, ##__VA_ARGS__><<<grid, block, smem, st>>>(p); \
+        else gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, false, ##__VA_ARGS__><<<grid, block, smem, st>>>(p);  \
     } while (0)
-        if (p.group == 0) FNN_DEC(false, 8);
+        // fp16 activations with per-channel fp16 scales: the reference's own per-weight rounding
+        bool refq = false;
+        if constexpr (ADT == FNN_F16) {
+            refq = p.group == 0 && p.scale_dtype == FNN_F16;
+            if (refq && p.zp) FNN_DEC(false, 8, 2);
+            else if (refq) FNN_DEC(false, 8, 1);
+        }
+        if (refq) {}
+        else if (p.group == 0) FNN_DEC(false, 8);
         else if (p.M == 1) FNN_DEC(true, 1);
         else if (p.M == 2) FNN_DEC(true, 2);
         else if (p.M <= 4) FNN_DEC(true, 4);
@@ -1019,6 +1067,7 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
         return true;
     }
     const size_t smem = fixed + (act_lds ? act_bytes : 0);
+    if (smem > 64 * 1024) return false;
     if (p.group > 0) {
         if (act_lds) gemm_wo_decode_kernel<WBITS, ADT, true, true><<<grid, block, smem, st>>>(p);
         else gemm_wo_decode_kernel<WBITS, ADT, true, false><<<grid, block, smem, st>>>(p);

@@ -42,8 +42,12 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // D: slabs of weights in flight per wave (8 loads per lane in flight stream faster than 16: measured
 // 19.8 against 21.7 us for 117 MB in a load-only model).  NTL: non-temporal weight loads, for a
 // single pass over the weights.
-template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL, bool MOE = false>
+// REFQ (1, or 2 with zero points; fp16 activations, per-channel fp16 scales and zero points): every weight is dequantised and rounded to
+// fp16 as the reference's torch path does before the dot product (ref_dq_f16 in wo_common.h); the MFMAs
+// against ones and the fold at the end are then not needed.
+template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL, bool MOE = false, int REFQ = 0>
 __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, const int passes, const MoeArgs q) {
+    static_assert(!REFQ || (ADT == FNN_F16 && !G128 && !MOE), "reference rounding: fp16, per-channel");
     // Gathered form with group tables: the reference's mixture-of-experts launcher lays them out
     // [expert][channel][group] (flashnn/triton_kernels/fused_moe_a16w4.py:336-344), the transpose of the
     // [group][channel] tables above, so 16-byte loads of 8 neighbouring channels do not exist.  The
@@ -113,14 +117,19 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     // full 128-byte line per row (16 rows x 64 bytes per load, the MFMA operand's own shape, streams
     // a quarter slower from HBM).  A wave-private 2 KB staging area in LDS turns the two loads
     // into the operand layout: row i at i*128, its 16-byte chunk c at slot c ^ ((i >> 1) & 7).
+    // An address is a wave-uniform 64-bit base (matrix, tile, slab: scalar arithmetic) plus the lane's 32-bit
+    // offset, the form the load instruction takes directly: no 64-bit vector adds per load.
     const int wr8 = lane >> 3, wc8 = lane & 7;
-    const char* wptr = (const char*)p.qw + (MOE ? (int64_t)expert * q.stride_be : 0) + (int64_t)(row0 + wr8) * p.ldw +
-                       wc8 * 16 + (int64_t)sl0 * 128;
+    const char* const wbase = (const char*)p.qw + (MOE ? (int64_t)expert * q.stride_be : 0) + (int64_t)row0 * p.ldw +
+                              (int64_t)sl0 * 128;
     const int64_t w_half = 8 * p.ldw;
-    const int wfix = wc8 * 16 >= tail_k ? -(wc8 * 16) : 0;
+    const uint32_t woff = (uint32_t)wr8 * (uint32_t)p.ldw + wc8 * 16;
+    const uint32_t woff_tail = wc8 * 16 >= tail_k ? woff - wc8 * 16 : woff;
     auto load_w = [&](int jj, int half) -> v4u {
         const int j = min(jj, nsl - 1);
-        const v4u* src = (const v4u*)(wptr + (int64_t)j * 128 + half * w_half + (part_tail && j == nsl - 1 ? wfix : 0));
+        const char* base = wbase + (int64_t)j * 128 + half * w_half;               // scalar
+        const uint32_t off = part_tail && j == nsl - 1 ? woff_tail : woff;          // uniform choice
+        const v4u* src = (const v4u*)(base + off);
         return NTL ? __builtin_nontemporal_load(src) : *src;
     };
     char* const wmine = wst + wave * 2048;
@@ -137,20 +146,21 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     constexpr int NCP = MB * 4 / RT;            // copies per wave and slab
     const int t = rt * 64 + lane;
     const int tokq = t >> 4;
-    const char* act_part = (const char*)p.act + (int64_t)sl0 * 256;
-    int64_t goff[NCP];
-    int afix[NCP];
+    // (rows of a pass lie within 64 rows of its first one, so their offsets fit 32 bits; gathered rows do not)
+    typedef typename std::conditional<MOE, int64_t, uint32_t>::type aoff_t;
+    const char* act_part = (const char*)p.act + (int64_t)sl0 * 256 + (MOE ? 0 : (int64_t)m_base * p.lda * 2);
+    aoff_t goff[NCP], goff_tail[NCP];
 #pragma unroll
     for (int i = 0; i < NCP; ++i) {
         const int tok = i * (4 * RT) + tokq;
         const int chunk = (t & 15) ^ (tok & 15);
-        afix[i] = chunk * 8 >= tail_k ? -(chunk * 16) : 0;
         if constexpr (MOE) {
             const int id = token_of(tok);
             goff[i] = (int64_t)(id < q.num_valid ? id / q.top_k : 0) * p.lda * 2 + chunk * 16;
         } else {
-            goff[i] = (int64_t)min(m_base + tok, p.M - 1) * p.lda * 2 + chunk * 16;
+            goff[i] = (uint32_t)min(tok, p.M - 1 - m_base) * (uint32_t)(p.lda * 2) + chunk * 16;
         }
+        goff_tail[i] = chunk * 8 >= tail_k ? goff[i] - chunk * 16 : goff[i];
     }
     auto copy_act = [&](char* stage, int jj) {
         const int j = min(jj, nsl - 1);
@@ -158,7 +168,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         const bool last = part_tail && j == nsl - 1;
 #pragma unroll
         for (int i = 0; i < NCP; ++i)
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + goff[i] + (last ? afix[i] : 0)),
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + (last ? goff_tail[i] : goff[i])),
                                              (lds_ptr_t)(stage + ks * SLAB + (i * RT * 64 + rt * 64) * 16), 16, 0, 0);
     };
     // ---- activation fragment reads: lane (li, lg) reads chunks 8 s + 2 lg + h of row 16 mb + li
@@ -171,15 +181,28 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     // ---- group tables: NCL consecutive channels per lane
     typedef typename std::conditional<NH == 2, v4u, v2u>::type tab_t;
     const int n0 = NH * (row0 + 4 * lg);
-    const uint16_t* sptr = (const uint16_t*)p.scale + (int64_t)sl0 * p.N + n0;
-    const uint16_t* zptr = (p.zp ? (const uint16_t*)p.zp : (const uint16_t*)p.scale) + (int64_t)sl0 * p.N + n0;
+    const uint16_t* sptr = (const uint16_t*)p.scale + (int64_t)sl0 * p.N + NH * row0;             // scalar
+    const uint16_t* zptr = (p.zp ? (const uint16_t*)p.zp : (const uint16_t*)p.scale) + (int64_t)sl0 * p.N + NH * row0;
+    const uint32_t tab_off = NH * 4 * lg * 2;                                                        // bytes
     const bool has_zp = p.zp != nullptr;
     // without zero points the second table load reads the scales again and is multiplied away
     const float zmul = has_zp ? 1.f : 0.f;
     auto load_tab = [&](const uint16_t* base, int jj) -> tab_t {
         const int j = min(jj, nsl - 1);
-        return *(const tab_t*)(base + (int64_t)j * p.N);
+        return *(const tab_t*)((const char*)(base + (int64_t)j * p.N) + tab_off);
     };
+
+    // REFQ: the scale and zero point of the weight row this lane feeds to the MFMAs (row li of the tile)
+    v2h rq_s[NH], rq_z[NH];
+    const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
+    if constexpr (REFQ) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h) {
+            const int n = NH * (row0 + li) + h;
+            rq_s[h] = pair_of_f16_bits(((const uint16_t*)p.scale)[n]);
+            rq_z[h] = pair_of_f16_bits(p.zp ? ((const uint16_t*)p.zp)[n] : 0u);
+        }
+    }
 
     v4f outv[MB][NH], accg[MB][NH], asum[MB];
 #pragma unroll
@@ -250,6 +273,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
                 bf[s][mb][1] = *(const v4u*)(stage + rd[s][1] + mb * 4096);
             }
         if (last) {   // partial slab: fragment (s, h) of this lane holds k = 8 * (8 s + 2 lg + h) .. + 7
+            asm volatile("" ::: "memory");   // a branch, taken once per wave, not sixteen selects in every slab
 #pragma unroll
             for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -263,29 +287,44 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
             v4u e[2][2], o[2][2];
             convert_w4_nat<ADT>(w0, e[0][0], e[0][1], o[0][0], o[0][1]);
             convert_w4_nat<ADT>(w1, e[1][0], e[1][1], o[1][0], o[1][1]);
+            if constexpr (REFQ) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        e[s][h] = ref_dq_f16<REFQ == 2>(e[s][h], rq_c, rq_z[0], rq_s[0]);
+                        o[s][h] = ref_dq_f16<REFQ == 2>(o[s][h], rq_c, rq_z[NH - 1], rq_s[NH - 1]);
+                    }
+            }
 #pragma unroll
             for (int s = 0; s < 2; ++s)
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
                     accg[mb][0] = MT::mma(e[s][0], bf[s][mb][0], accg[mb][0]);
                     accg[mb][1] = MT::mma(o[s][0], bf[s][mb][0], accg[mb][1]);
-                    asum[mb] = MT::mma(ones, bf[s][mb][0], asum[mb]);
+                    if constexpr (!REFQ) asum[mb] = MT::mma(ones, bf[s][mb][0], asum[mb]);
                     accg[mb][0] = MT::mma(e[s][1], bf[s][mb][1], accg[mb][0]);
                     accg[mb][1] = MT::mma(o[s][1], bf[s][mb][1], accg[mb][1]);
-                    asum[mb] = MT::mma(ones, bf[s][mb][1], asum[mb]);
+                    if constexpr (!REFQ) asum[mb] = MT::mma(ones, bf[s][mb][1], asum[mb]);
                 }
         } else {
             v4u c[2][2];
             convert_w8<ADT>(w0, c[0][0], c[0][1]);
             convert_w8<ADT>(w1, c[1][0], c[1][1]);
+            if constexpr (REFQ) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) c[s][h] = ref_dq_f16<REFQ == 2>(c[s][h], rq_c, rq_z[0], rq_s[0]);
+            }
 #pragma unroll
             for (int s = 0; s < 2; ++s)
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
                     accg[mb][0] = MT::mma(c[s][0], bf[s][mb][0], accg[mb][0]);
-                    asum[mb] = MT::mma(ones, bf[s][mb][0], asum[mb]);
+                    if constexpr (!REFQ) asum[mb] = MT::mma(ones, bf[s][mb][0], asum[mb]);
                     accg[mb][0] = MT::mma(c[s][1], bf[s][mb][1], accg[mb][0]);
-                    asum[mb] = MT::mma(ones, bf[s][mb][1], asum[mb]);
+                    if constexpr (!REFQ) asum[mb] = MT::mma(ones, bf[s][mb][1], asum[mb]);
                 }
         }
     };
@@ -370,7 +409,12 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
 #undef FNN_PANEL_ITER
 
     // ---- per-channel scales: one fold at the end
-    if constexpr (!G128) {
+    if constexpr (REFQ) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int h = 0; h < NH; ++h) outv[mb][h] = accg[mb][h];
+    } else if constexpr (!G128) {
         float sc[NCL], zc[NCL];
 #pragma unroll
         for (int c = 0; c < NCL; ++c) {
@@ -503,10 +547,24 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);
     p.m_base = 0;
+    // fp16 activations with per-channel fp16 scales (and zero points): the reference's own per-weight rounding
+    constexpr bool CAN_REFQ = ADT == FNN_F16;
+    const bool refq = CAN_REFQ && p.group == 0 && p.scale_dtype == FNN_F16 && (!p.zp || p.zp_dtype == FNN_F16);
+#define FNN_PANEL3(G, SDTV, MBV, RTV, NTLV)                                                              \
+    do {                                                                                                 \
+        if constexpr (CAN_REFQ && !G) {                                                                  \
+            if (refq) {                                                                                  \
+                if (p.zp) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, NTLV, false, 2><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{}); \
+                else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, NTLV, false, 1><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{}); \
+                break;                                                                                   \
+            }                                                                                            \
+        }                                                                                                \
+        gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, NTLV><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{}); \
+    } while (0)
 #define FNN_PANEL2(G, SDTV, MBV, RTV)                                                                    \
     do {                                                                                                 \
-        if (passes == 1) gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, true><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{}); \
-        else gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, false><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{});         \
+        if (passes == 1) FNN_PANEL3(G, SDTV, MBV, RTV, true);                                            \
+        else FNN_PANEL3(G, SDTV, MBV, RTV, false);                                                       \
     } while (0)
 #define FNN_PANEL(G, SDTV)                                   \
     do {                                                     \
@@ -529,6 +587,7 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     }
 #undef FNN_PANEL
 #undef FNN_PANEL2
+#undef FNN_PANEL3
     return true;
 }
 

@@ -91,6 +91,31 @@ __device__ __forceinline__ void convert_w4(const v4u w, v4u& e0, v4u& e1, v4u& o
     o1 = v4u{o[4], o[5], o[6], o[7]};
 }
 
+// The reference's per-weight dequantisation for fp16 scales (flashnn/quant_gemm.py:14-17, 168): the weight
+// minus its zero point, rounded to fp16, times the scale, rounded to fp16 again; the dot product then runs
+// over these rounded weights.  x holds two weights as coff + q (the exponent-trick conversion, exact), so
+// the first subtraction is exact and the other two operations round exactly as torch rounds them.
+// Used where activations and scales are both fp16: the result then differs from the reference's only by
+// the order of the fp32 additions.
+// ZP = false: no zero points were given; the reference then subtracts zeros, which changes nothing.
+template <bool ZP>
+__device__ __forceinline__ uint32_t ref_dq_f16(uint32_t x, const v2h coff, const v2h zp, const v2h s) {
+#pragma clang fp contract(off)
+    v2h v = __builtin_bit_cast(v2h, x) - coff;
+    if constexpr (ZP) v = v - zp;
+    v = v * s;
+    return __builtin_bit_cast(uint32_t, v);
+}
+template <bool ZP>
+__device__ __forceinline__ v4u ref_dq_f16(v4u x, const v2h coff, const v2h zp, const v2h s) {
+    return v4u{ref_dq_f16<ZP>(x[0], coff, zp, s), ref_dq_f16<ZP>(x[1], coff, zp, s), ref_dq_f16<ZP>(x[2], coff, zp, s),
+               ref_dq_f16<ZP>(x[3], coff, zp, s)};
+}
+// an fp16 bit pattern in both halves of a packed pair
+__device__ __forceinline__ v2h pair_of_f16_bits(uint32_t h) {
+    return __builtin_bit_cast(v2h, (h & 0xFFFFu) * 0x10001u);
+}
+
 // reorder 8 consecutive 16-bit values to (0,2)(1,3)(4,6)(5,7)
 __device__ __forceinline__ v4u perm_act_w4(const v4u a) {
     return v4u{__builtin_amdgcn_perm(a[1], a[0], 0x05040100u), __builtin_amdgcn_perm(a[1], a[0], 0x07060302u),

@@ -34,3 +34,15 @@ def oracle_c():
     lib.fnn_oracle_a8w8_epilogue.argtypes = [p, p, p, p, i64, i64]
     lib.fnn_oracle_a8w8_epilogue.restype = None
     return lib
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Weight-only cases in which some outputs left rtol/atol 1e-2 of the reference-rounding oracle (they
+    passed because each such output is closer to the float64 value than the oracle's): name and count."""
+    mod = sys.modules.get("test_gpu_parity") or sys.modules.get("tests.test_gpu_parity")
+    breaches = getattr(mod, "WO_BREACHES", None)
+    if breaches:
+        terminalreporter.write_line(f"weight-only outputs beyond rtol/atol 1e-2 of the oracle in {len(breaches)} cases "
+                                    "(each at least as close to float64 as the oracle):")
+        for case, nbad, total in breaches:
+            terminalreporter.write_line(f"  {case}: {nbad} of {total}")

@@ -413,7 +413,17 @@ def _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp, with_bias, seed)
     return act, w, qw, scale, zp, bias
 
 
-def _wo_check(act, w, qw, scale, zp, bias, group, bits, out_ty):
+WO_BREACHES = []   # (test id, outputs beyond the stated tolerance, outputs) of the cases that had any
+
+
+def _wo_check(act, w, qw, scale, zp, bias, group, bits, out_ty, strict=False):
+    """The stated tolerance, unscaled: |got - oracle| <= 1e-2 + 1e-2 |oracle|, the oracle being the reference's
+    torch path with its per-weight rounding of the dequantised weights to the scale type (fp16 for group
+    tables).  Where activations and per-channel scales are both fp16 the kernels round the same way and
+    `strict` demands that no output leaves the tolerance.  Elsewhere the kernels scale in fp32, which the
+    reference's rounding can leave by more than the tolerance on outputs near zero of long dot products;
+    such an output must then be at least as close to the float64 value as the oracle's is, and the count is
+    reported."""
     d = lambda t: None if t is None else t.to(DEV)
     out = flashnn_amd.GemmWeightOnly(out_ty)(d(act), d(qw), d(scale), d(bias), d(zp))
     assert out.dtype == out_ty and out.shape == (act.shape[0], w.shape[0])
@@ -422,16 +432,18 @@ def _wo_check(act, w, qw, scale, zp, bias, group, bits, out_ty):
     want = O.weight_only_gemm(n(act), w.numpy(), n(scale), n(zp), n(bias), _tag(scale.dtype), _tag(out_ty),
                               group, bits == 4)
     exact = O.weight_only_gemm_f64(n(act), w.numpy(), n(scale), n(zp), n(bias), group)
-    # within the stated tolerance of the reference's torch path.  The reference rounds every
-    # dequantised weight to fp16 (bf16 with bf16 scales), which alone moves an output by about
-    # 2^-11 (2^-8) of the output's spread; where the stress inputs make that spread much larger
-    # than 1 the absolute tolerance is taken relative to it.
+    bad = np.abs(got - want) > ATOL + RTOL * np.abs(want)
+    if bad.any():
+        import os
+        case = os.environ.get("PYTEST_CURRENT_TEST", "?").split(" ")[0]
+        WO_BREACHES.append((case, int(bad.sum()), bad.size))
+        assert not strict, f"{int(bad.sum())} outputs beyond the stated tolerance on a reference-rounding path"
+        assert (np.abs(got[bad] - exact[bad]) <= np.abs(want[bad] - exact[bad])).all()
+    # ... and as close to the mathematical value as one output rounding (and fp32 accumulation) allows
     spread = max(1.0, float(np.sqrt(np.mean(want.astype(np.float64) ** 2))))
-    atol = (ATOL if scale.dtype != torch.bfloat16 else 5e-2) * spread
-    np.testing.assert_allclose(got, want, rtol=RTOL, atol=atol)
-    # ... and at least as close to the mathematical value as one output rounding allows
     ulp = 2.0 ** -9 if out_ty == torch.float16 else 2.0 ** -6
-    assert (np.abs(got - exact) <= np.abs(exact) * ulp + 2e-3 * spread).all()
+    slack = (2e-3 if not strict else 8e-3) * spread   # the reference's rounding itself moves an output by about 2^-11 |w| sqrt(K)
+    assert (np.abs(got - exact) <= np.abs(exact) * ulp + slack).all()
 
 
 @pytest.mark.parametrize("bits", [8, 4])
@@ -546,7 +558,8 @@ def test_a16w8_decode_config(M, kn):
     act = workloads.activations(M, K, torch.float16, seed=31)
     w, s32 = workloads.int8_weights(N, K, seed=32)
     scale = s32.half()
-    _wo_check(act, w, w, scale, None, None, 0, 8, torch.float16)
+    # fp16 activations, per-channel fp16 scales: the kernels round every weight as the reference does
+    _wo_check(act, w, w, scale, None, None, 0, 8, torch.float16, strict=True)
 
 
 @pytest.mark.parametrize("M", [1, 4, 16, 64, 256])
