@@ -950,6 +950,287 @@ __global__ __launch_bounds__(kGemvMaxWaves * 64) void gemm_wo_gemv_kernel(const 
     }
 }
 
+// ------------------------------------------------ GEMV kernel, flattened: eight equal chunks per CU
+// One wave per tile leaves a CU with as many waves as it has tiles - seven at N = 28672 int4 channels, on
+// four SIMDs: three SIMDs carry two streams and one carries one, and the kernel ends when the doubled-up
+// ones do.  Here the wpw tiles of a workgroup times the K/128 steps of a tile are one sequence of
+// wpw * steps steps, cut into eight equal, contiguous chunks, one per wave: two waves on every SIMD, each
+// with the same number of bytes to stream.  A chunk is at most one tile long, so it covers the end of one
+// tile and the beginning of the next; the two partial results are kept apart, written to LDS, and the
+// parts of every tile are added in ascending K order by one wave (a fixed order: the result does not
+// depend on timing).  Chunks, tiles and the 8-step blocks of the group slots all begin at multiples of
+// eight steps (checked on the host), so a block never straddles two tiles.  Group size 128, M <= 4.
+//
+// Start-up is a matter of how many cache lines the CU has to ask for before the first weights arrive.  The
+// scale and zero-point tables are [K/128][N]: the 16 channels of one tile are 32 bytes of each row, so a
+// wave fetching its own tile's tables asks for one line per group and table (the wpw tiles of a workgroup
+// for the same lines again).  The workgroup's tiles are neighbours, so it fetches the tables of all of
+// them together instead, wpw * 32 contiguous bytes per row, with all its threads, into one shared LDS
+// table: an eighth of the requests.
+//
+// A wave executes about one instruction every 2 ns here, so what stands between the kernel's start and its
+// first loads is kept short: where a chunk begins (tile and step) and which chunks make up a tile are
+// worked out on the host and passed as packed 4-bit fields, the weight loads are issued first, and the
+// tables are fetched by 16 lanes per row, which needs no division.  fp16 tables only.
+struct GemvFlatPlan {
+    uint32_t tA;      // 4 bits per wave: the tile (of the workgroup) its chunk begins in
+    uint32_t sA8;     // 4 bits per wave: the step it begins at, in units of 8
+    uint32_t len8;    // 4 bits per wave: the length of its chunk, in units of 8 steps
+    uint32_t wfirst;  // 4 bits per tile: the first chunk that overlaps it
+    uint32_t wlast;   // 4 bits per tile: the last one
+};
+
+template <int WBITS, int ADT, int MP>
+__global__ __launch_bounds__(512) void gemm_wo_gemv_flat_kernel(const WoArgs p, const int wpw, const GemvFlatPlan plan) {
+    typedef MfmaT<ADT> MT;
+    constexpr int NH = WBITS == 4 ? 2 : 1;
+    constexpr int NC = 8 * NH;
+    constexpr int GS = 8 / MP;
+    constexpr int UN = 8;
+    constexpr int NW = 8;
+    constexpr int nt = NW * 64;
+    constexpr float c_off = WBITS == 4 ? (ADT == FNN_F16 ? 1024.f + 8.f : 128.f + 8.f)
+                                       : (ADT == FNN_F16 ? 1024.f + 128.f : 128.f);
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int li = lane & 15;
+    const int lg = lane >> 4;
+    const int half = li >> 3;
+    const int j7 = li & 7;
+
+    const int steps = p.K / 128;
+    const int chunk = ((plan.len8 >> (4 * wave)) & 15) * 8;   // steps of this wave, a multiple of 8, at most `steps`
+    const int tA = (plan.tA >> (4 * wave)) & 15;   // the chunk begins in tile tA of the workgroup, at step sA
+    const int sA = ((plan.sA8 >> (4 * wave)) & 15) * 8;
+    const int len1 = min(chunk, steps - sA);       // steps in tile tA; the other chunk - len1 are in tile tA + 1
+    // workgroups id, id + 8, id + 16 .. share an XCD and its L2: they take neighbouring tiles, whose table rows
+    // share cache lines (a tile's 32 bytes of a table row are a quarter of a line)
+    const int per_xcd = gridDim.x >> 3;            // the grid is a multiple of 8 (host-checked)
+    const int tile0 = ((blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3)) * wpw;
+
+    // LDS: [32 B of zeros][activations M x (K+32)][per wave: 2 x (scale, zoff) of 8 groups x NC f32][parts 8 x 2 x PART f32]
+    constexpr int PART = NH * 4 * 64;              // floats of one partial result
+    constexpr int TBLK = 8 * NC;                   // floats of one table of one block of eight groups
+    const int a_stride = p.K + 32;
+    uint16_t* a_lds = (uint16_t*)(smem + 32);
+    float* const tabs = (float*)(smem + 32 + (size_t)p.M * a_stride * 2);
+    float* const my_tab = tabs + wave * (4 * TBLK);            // [parity][scale | zoff][8 groups][NC]
+    float* const parts = tabs + NW * 4 * TBLK;
+
+    const uint32_t w_off = (uint32_t)j7 * (uint32_t)p.ldw + lg * 32 + half * 16;
+    const char* const wA = (const char*)p.qw + (int64_t)(tile0 + tA) * 8 * p.ldw + (int64_t)sA * 128;
+    const char* const wB = (const char*)p.qw + (int64_t)(tile0 + tA + 1) * 8 * p.ldw - (int64_t)len1 * 128;
+    auto load_w = [&](int f) -> v4u {
+        const int g = min(f, chunk - 1);
+        const char* base = (g < len1 ? wA : wB) + (int64_t)g * 128;   // scalar
+        return __builtin_nontemporal_load((const v4u*)(base + w_off));
+    };
+    // ---- tables: the scales and zero points of a block of eight steps (eight groups x the tile's NC
+    // channels: 2 x 16-byte pieces per group and table) are fetched one block ahead by 16 lanes of the wave,
+    // converted, and passed to the fold through a wave-private LDS area - no staging of whole tables at the
+    // start (a burst of small scattered requests in front of the weight stream), no barrier.
+    const bool has_zp = p.zp != nullptr;
+    const uint16_t* zp_src = has_zp ? (const uint16_t*)p.zp : (const uint16_t*)p.scale;
+    const float zmul = has_zp ? 1.f : 0.f;
+    const uint32_t tab_lane = (uint32_t)((lane / (NC / 8)) & 7) * (uint32_t)p.N * 2 + (lane % (NC / 8)) * 16;   // bytes: group row, piece
+    auto load_tabs = [&](int sb, v4u& sv, v4u& zv) {   // block of steps sb .. sb + 7 of the chunk (clamped)
+        const int b = min(sb, chunk - 8);
+        const int tile = tile0 + tA + (b < len1 ? 0 : 1);
+        const int grp = b < len1 ? sA + b : b - len1;
+        const int64_t off = ((int64_t)grp * p.N + (int64_t)tile * NC) * 2;        // scalar, bytes
+        sv = *(const v4u*)((const char*)p.scale + off + tab_lane);
+        zv = *(const v4u*)((const char*)zp_src + off + tab_lane);
+    };
+    auto stage_tabs = [&](int parity, const v4u sv, const v4u zv) {
+        {
+            float sc[8], zo[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t sb = (sv[j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
+                const uint32_t zb = (zv[j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
+                sc[j] = f16_bits_to_f32(sb);
+                zo[j] = sc[j] * (c_off + zmul * f16_bits_to_f32(zb));
+            }
+            if (lane < 8 * (NC / 8)) {             // 8 groups x NC / 8 pieces
+                float* sd = my_tab + parity * 2 * TBLK + (lane / (NC / 8)) * NC + (lane % (NC / 8)) * 8;
+                float* zd = sd + TBLK;
+                *(v4f*)sd = v4f{sc[0], sc[1], sc[2], sc[3]};
+                *(v4f*)(sd + 4) = v4f{sc[4], sc[5], sc[6], sc[7]};
+                *(v4f*)zd = v4f{zo[0], zo[1], zo[2], zo[3]};
+                *(v4f*)(zd + 4) = v4f{zo[4], zo[5], zo[6], zo[7]};
+            }
+        }
+    };
+    // ---- start-up: every load is issued before the first wait, in the order in which the data is needed
+    // (loads return in order): the activations, which every wave needs at its first step and which come from
+    // the L2; the tables of the first block; the first UN weight pieces.  One bare barrier (a __syncthreads()
+    // would wait for every load in flight) publishes the activations.
+    constexpr int AB = 4;
+    const int chunks = p.K / 8;
+    constexpr int MROWS = MP < 4 ? MP : 4;
+    v4u av[MROWS][AB];
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+        const v4u* src = (const v4u*)((const uint16_t*)p.act + (int64_t)min(m, p.M - 1) * p.lda);
+#pragma unroll
+        for (int u = 0; u < AB; ++u) {
+            if (u * nt < chunks) av[m][u] = src[min(u * nt + (int)threadIdx.x, chunks - 1)];
+            else av[m][u] = v4u{0, 0, 0, 0};
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    v4u tsv, tzv;
+    load_tabs(0, tsv, tzv);
+    __builtin_amdgcn_sched_barrier(0);
+    v4u wq[UN];
+#pragma unroll
+    for (int i = 0; i < UN; ++i) wq[i] = load_w(i);
+    __builtin_amdgcn_sched_barrier(0);
+
+    if (threadIdx.x < 8) ((uint32_t*)smem)[threadIdx.x] = 0;
+#pragma unroll
+    for (int m = 0; m < MROWS; ++m) {
+        v4u* dst = (v4u*)(a_lds + m * a_stride);
+#pragma unroll
+        for (int u = 0; u < AB; ++u) {
+            const int c = u * nt + threadIdx.x;
+            if (m < p.M && c < chunks) dst[c] = WBITS == 4 ? perm_act_w4(av[m][u]) : av[m][u];
+        }
+    }
+    // (K <= AB * 512 * 8 = 16384 is checked on the host: the staged batches hold a whole row)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);            // lgkmcnt(0): this wave's LDS writes are done
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    const int m_col = j7 % MP;
+    const int gslot = j7 / MP;
+    const bool col_valid = m_col < p.M;
+    bool use[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) use[i] = col_valid && (i % GS) == gslot;
+    const int koff = lg * 32 + half * 16;
+    const uint32_t a_base = (uint32_t)((const char*)(a_lds + m_col * a_stride + koff) - smem);
+    uint32_t a_real = a_base + sA * 256;
+    // table entry of (group slot, this lane's channels) in the wave's area of the current block
+    constexpr uint32_t rowb = NC * 4;              // bytes of a table row
+    const uint32_t sz_lane = (uint32_t)((const char*)(my_tab + NH * 4 * (lg & 1)) - smem) + gslot * rowb;
+    constexpr uint32_t z_delta = TBLK * 4;
+
+    v4f outv[NH], outA[NH], accg[NH], asum;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) { outv[h] = v4f{0, 0, 0, 0}; outA[h] = v4f{0, 0, 0, 0}; accg[h] = v4f{0, 0, 0, 0}; }
+    asum = v4f{0, 0, 0, 0};
+    const v4f zero4 = v4f{0, 0, 0, 0};
+
+    auto fold = [&](uint32_t addr) {
+        float sv[NH * 4], zv[NH * 4];
+#pragma unroll
+        for (int q = 0; q < NH; ++q) {
+            const v4f a = *(const v4f*)(smem + addr + q * 16);
+            const v4f b = *(const v4f*)(smem + addr + z_delta + q * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { sv[q * 4 + e] = a[e]; zv[q * 4 + e] = b[e]; }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+                outv[h][r] += sv[NH * r + h] * accg[h][r] - zv[NH * r + h] * asum[r];
+    };
+
+    const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+    int parity = 0;
+    for (int sb = 0; sb < chunk; sb += UN) {
+        if (sb == len1) {   // the chunk moves on to the next tile: a new result, K starts over
+#pragma unroll
+            for (int h = 0; h < NH; ++h) { outA[h] = outv[h]; outv[h] = v4f{0, 0, 0, 0}; }
+            a_real = a_base;
+        }
+        // this block's tables go to LDS (the area of the block before last is free: LDS operations of a
+        // wave complete in order), the next block's are requested
+        stage_tabs(parity, tsv, tzv);
+        load_tabs(sb + UN, tsv, tzv);
+        const uint32_t sz_addr = sz_lane + parity * (2 * TBLK * 4);
+        parity ^= 1;
+#pragma unroll
+        for (int i = 0; i < UN; ++i) {
+            const v4u w = wq[i];
+            const uint32_t aa = use[i % 8] ? a_real + i * 256 : 0u;
+            const v4u a0 = *(const v4u*)(smem + aa);
+            const v4u a1 = *(const v4u*)(smem + aa + 16);
+            const bool first = i % GS == 0;
+            if constexpr (WBITS == 4) {
+                v4u e0, e1, o0, o1;
+                convert_w4<ADT>(w, e0, e1, o0, o1);
+                wq[i] = load_w(sb + i + UN);
+                accg[0] = MT::mma(e0, a0, first ? zero4 : accg[0]);
+                accg[1] = MT::mma(o0, a0, first ? zero4 : accg[1]);
+                asum = MT::mma(ones, a0, first ? zero4 : asum);
+                accg[0] = MT::mma(e1, a1, accg[0]);
+                accg[1] = MT::mma(o1, a1, accg[1]);
+                asum = MT::mma(ones, a1, asum);
+            } else {
+                v4u s0, s1;
+                convert_w8<ADT>(w, s0, s1);
+                wq[i] = load_w(sb + i + UN);
+                accg[0] = MT::mma(s0, a0, first ? zero4 : accg[0]);
+                asum = MT::mma(ones, a0, first ? zero4 : asum);
+                accg[0] = MT::mma(s1, a1, accg[0]);
+                asum = MT::mma(ones, a1, asum);
+            }
+            if (i % GS == GS - 1) fold(sz_addr + (i / GS) * GS * rowb);
+            __builtin_amdgcn_sched_barrier(0);   // keep each refill load inside its step
+        }
+        a_real += UN * 256;
+    }
+    if (len1 == chunk) {   // (wave-uniform) the whole chunk lay in tile tA
+#pragma unroll
+        for (int h = 0; h < NH; ++h) { outA[h] = outv[h]; outv[h] = v4f{0, 0, 0, 0}; }
+    }
+
+    // ---- the group-slot columns of a result are added within the wave: column gs * MP + m of a half holds
+    // activation row m, so a butterfly over the lane bits above log2(MP) leaves every lane of a half with
+    // the sum for its m.  Then the two partial results go to LDS, part 0 = tile tA, part 1 = tile tA + 1.
+    float* const mine = parts + (size_t)wave * 2 * PART;
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float a = outA[h][r], b = outv[h][r];
+#pragma unroll
+            for (int o = MP; o < 8; o <<= 1) { a += __shfl_xor(a, o, 64); b += __shfl_xor(b, o, 64); }
+            mine[(h * 4 + r) * 64 + lane] = a;
+            mine[PART + (h * 4 + r) * 64 + lane] = b;
+        }
+    __syncthreads();
+    // ---- wave t adds the parts of tile t in ascending K order and stores it: the chunks that overlap
+    // steps [t * steps, (t + 1) * steps) of the workgroup's sequence, at most three
+    if (wave >= wpw) return;
+    const int t = wave;
+    const int w_first = (plan.wfirst >> (4 * t)) & 15, w_last = (plan.wlast >> (4 * t)) & 15;
+    const int n0 = (tile0 + t) * NC;
+    if (lane < p.M * NC) {
+        const int m = lane / NC, c = lane % NC;
+        const int row = c / NH, h = c % NH;
+        const int r = row & 3;
+        // the two diagonal blocks of the MFMA result: columns 0..7 of lane rows 0..1, columns 8..15 of lane rows 2..3
+        const int lane1 = m + 16 * (row >> 2);
+        const int lane2 = (m + 8) + 16 * ((row + 8) >> 2);
+        float v = 0.f;
+        for (int w = w_first; w <= w_last; ++w) {
+            const int tw = (plan.tA >> (4 * w)) & 15;   // the tile chunk w begins in: part 0 if it is t, else part 1
+            const float* part = parts + (size_t)w * 2 * PART + (tw == t ? 0 : PART);
+            v += part[(h * 4 + r) * 64 + lane1] + part[(h * 4 + r) * 64 + lane2];
+        }
+        const int n = n0 + c;
+        if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+        store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
+    }
+}
+
 // ------------------------------------------------------------------ guarded fallback
 template <int WBITS, int ADT>
 __global__ __launch_bounds__(256) void gemm_wo_any_kernel(const WoArgs p) {
@@ -1020,6 +1301,62 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
         if (need <= 150 * 1024 && (size_t)ngr * 8 * NH * 2 >= (size_t)NH * 4 * 64) {
             const dim3 g2((tiles + wpw - 1) / wpw), b2(wpw * 64);
             const bool full = (p.K / 128) % 8 == 0;
+            // eight equal chunks per workgroup where the tiles do not already make eight waves of equal length
+            {
+                const int steps = p.K / 128;
+                const int chunk = wpw * steps / 8;
+                // zeros, activations, per wave two blocks of two fp32 tables (8 groups x the tile's channels), 16 partial results
+                const size_t need_f = 32 + act_bytes + (size_t)8 * 4 * 8 * 8 * NH * 4 + (size_t)16 * NH * 4 * 64 * 4;
+                const bool flat = wpw < 8 && p.M * 8 * NH <= 64 && wrows % 8 == 0 && tiles % wpw == 0 && steps % 8 == 0 &&
+                                  (wpw * steps) % 64 == 0 && chunk <= steps && steps <= 64 && wpw * NH <= 16 && p.K <= 16384 &&
+                                  p.scale_dtype == FNN_F16 && need_f <= 160 * 1024 && (tiles / wpw) % 8 == 0;
+                if (flat) {
+                    const size_t smem_f = need_f > 84 * 1024 ? need_f : 84 * 1024;
+                    // The four waves a workgroup starts first are served first by their SIMDs and run ahead of the
+                    // four that share those SIMDs; with equal chunks they finish a fifth earlier and the stream
+                    // then runs on half the loads in flight.  Where the arithmetic allows it they get a seventh
+                    // more steps than the others (64 and 48 of 448) and all eight finish together.
+                    int len[8];
+                    for (int w = 0; w < 8; ++w) len[w] = chunk;
+                    if (chunk % 8 == 0 && chunk + 8 <= steps && chunk >= 16) {
+                        for (int w = 0; w < 4; ++w) { len[w] = chunk + 8; len[w + 4] = chunk - 8; }
+                    }
+                    GemvFlatPlan plan{0, 0, 0, 0, 0};
+                    int beg[9];
+                    beg[0] = 0;
+                    for (int w = 0; w < 8; ++w) {
+                        const int ta = beg[w] / steps;
+                        plan.tA |= (uint32_t)ta << (4 * w);
+                        plan.sA8 |= (uint32_t)((beg[w] - ta * steps) / 8) << (4 * w);
+                        plan.len8 |= (uint32_t)(len[w] / 8) << (4 * w);
+                        beg[w + 1] = beg[w] + len[w];
+                    }
+                    for (int t = 0; t < wpw; ++t) {
+                        int wf = 0, wl = 0;
+                        for (int w = 0; w < 8; ++w) {
+                            if (beg[w + 1] <= t * steps) wf = w + 1;
+                            if (beg[w] < (t + 1) * steps) wl = w;
+                        }
+                        plan.wfirst |= (uint32_t)wf << (4 * t);
+                        plan.wlast |= (uint32_t)wl << (4 * t);
+                    }
+#define FNN_GEMV_FLAT(MPV)                                                                                    \
+    do {                                                                                                      \
+        auto kfn = gemm_wo_gemv_flat_kernel<WBITS, ADT, MPV>;                                                  \
+        static bool attr_set = false;                                                                         \
+        if (!attr_set) {                                                                                      \
+            (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            attr_set = true;                                                                                  \
+        }                                                                                                     \
+        kfn<<<g2, dim3(512), smem_f, st>>>(p, wpw, plan);                                                     \
+    } while (0)
+                    if (p.M == 1) FNN_GEMV_FLAT(1);
+                    else if (p.M == 2) FNN_GEMV_FLAT(2);
+                    else FNN_GEMV_FLAT(4);
+#undef FNN_GEMV_FLAT
+                    return true;
+                }
+            }
 #define FNN_GEMV(G, MPV)                                                                                  \
     do {                                                                                                  \
         auto kfn = full ? gemm_wo_gemv_kernel<WBITS, ADT, G, MPV, 8, true>                               \

@@ -587,6 +587,41 @@ def test_a16w4_group128_config(M):
     np.testing.assert_allclose(o1[0].float().cpu().numpy(), col.bfloat16().float().numpy(), rtol=2.0 ** -7, atol=1e-6)
 
 
+@pytest.mark.parametrize("bits,M,N,K", [(4, 1, 24576, 8192), (4, 2, 24576, 8192), (4, 3, 20480, 8192), (4, 4, 28672, 8192),
+                                        (8, 1, 12288, 8192), (4, 2, 28672, 4096), (4, 1, 16384, 8192)])
+def test_weight_only_gemv_equal_chunks(bits, M, N, K):
+    """Up to four rows over many channels with group 128: a workgroup's tiles x K steps are cut into eight
+    equal chunks, one per wave, and a chunk covers the end of one tile and the beginning of the next
+    (5, 6 and 7 tiles per workgroup; 4 tiles: two chunks per tile; K = 4096: the one-wave-per-tile kernel).
+    Bands of channels at the seams against the oracle, zero points and bias on."""
+    g = torch.Generator().manual_seed(500 + M + N)
+    act_ty = torch.bfloat16 if M % 2 else torch.float16
+    act = torch.randn(M, K, generator=g).to(act_ty)
+    lo, hi = (-128, 128) if bits == 8 else (-8, 8)
+    w = torch.randint(lo, hi, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(K // 128, N).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(lo // 2, hi // 2, (K // 128, N), generator=g).half()
+    bias = torch.randn(N, generator=g).to(act_ty)
+    qw = w if bits == 8 else torch.from_numpy(O.pack_int4(w.numpy()))
+    out = flashnn_amd.GemmWeightOnly(act_ty)(act.to(DEV), qw.to(DEV), scale.to(DEV), bias.to(DEV), zp.to(DEV))
+    got = out.float().cpu().numpy()
+    per_tile = 16 if bits == 4 else 8
+    tiles = N // per_tile
+    wpw = -(-tiles // 256)
+    # the first workgroups' tiles (every seam between chunks), one workgroup in the middle, the last one
+    for first in (0, (tiles // wpw // 2) * wpw, tiles - wpw):
+        band = slice(first * per_tile, (first + wpw) * per_tile)
+        want = O.weight_only_gemm(O.to_np(act), w[band].numpy(), O.to_np(scale[:, band]), O.to_np(zp[:, band]),
+                                  O.to_np(bias[band]), O.F16, _tag(act_ty), 128, bits == 4)
+        exact = O.weight_only_gemm_f64(O.to_np(act), w[band].numpy(), O.to_np(scale[:, band]), O.to_np(zp[:, band]),
+                                       O.to_np(bias[band]), 128)
+        bad = np.abs(got[:, band] - want) > ATOL + RTOL * np.abs(want)
+        assert (np.abs(got[:, band][bad] - exact[bad]) <= np.abs(want[bad] - exact[bad])).all()
+        ulp = 2.0 ** -9 if act_ty == torch.float16 else 2.0 ** -6
+        spread = max(1.0, float(np.sqrt(np.mean(want.astype(np.float64) ** 2))))
+        assert (np.abs(got[:, band] - exact) <= np.abs(exact) * ulp + 2e-3 * spread).all()
+
+
 # ------------------------------------------------------- rmsnorm+quant -> A8W8 chain
 @pytest.mark.parametrize("M", [1, 32, 512, 8192])
 def test_rmsnorm_quant_gemm_chain(M):
