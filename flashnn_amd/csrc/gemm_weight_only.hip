@@ -1431,6 +1431,8 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
     // whose waves share the activations through LDS; the other decode kernels for a single row and
     // for the shapes the panel kernel does not take.
     if (p.M <= 4 && (WBITS == 4 || p.M == 1) && launch_decode<WBITS, ADT>(p, st, true)) return;
+    // more than 64 rows: every weight dequantised once per 128 or 256 rows (the panel kernel takes 64 a pass)
+    if (p.M > 64 && launch_wo_tile(p, WBITS, ADT, st)) return;
     if (p.M >= 2 && launch_wo_panel(p, WBITS, ADT, st)) return;
     if (launch_decode<WBITS, ADT>(p, st, false)) return;
     // up to 64 activation rows per pass over the weights

@@ -1,0 +1,380 @@
+// Weight-only GEMM for many activation rows (M > 64): a tiled MFMA kernel, gfx950.
+//
+// With hundreds of activation rows the job is no longer streaming the weights but multiplying: every
+// weight has to be dequantised once per workgroup and used against as many rows as possible.  A
+// 512-thread workgroup (8 waves, 2 along M x 4 along N, two on every SIMD) owns BM activation rows
+// (256 or 128) x 128 output channels and walks K in slabs of 128 (one scale group):
+//   * activations: the slab of the tile's rows (BM x 256 bytes) is copied L2 -> LDS with direct-to-LDS
+//     16-byte loads into a ring of two stages, one slab ahead; 16-byte chunks XOR-swizzled with the row so
+//     that the 16 lanes of a fragment read hit 16 different bank groups;
+//   * weights: the slab of the tile's weight rows (64 packed int4 rows or 128 int8 rows x 128 bytes) goes
+//     the same way into a ring of three stages, two slabs ahead; the slab's scales and zero points (group
+//     size 128) one slab ahead into three stages of their own: nothing waits in registers for HBM, and one
+//     s_waitcnt vmcnt(N) with a compile-time N plus a bare s_barrier publishes a slab (all copies of an
+//     iteration are issued in a fixed order, the weights last: they have two slabs to land and may stay in
+//     flight over the next barrier);
+//   * a wave reads 16 bytes per lane of its weight rows from LDS (16 k of one row), turns them into MFMA
+//     "A" operands with the exponent tricks of wo_common.h (values c + q, exact), reads the activation
+//     fragments ("B" operands) and runs v_mfma_f32_16x16x32_{f16,bf16}: wave tile (BM/2) x 32, 16 or 8
+//     accumulator fragments; an MFMA against ones per activation fragment gives the row sums that remove c
+//     and the zero points;
+//   * at the end of a slab (group size 128) the slab's accumulators are folded into the running output in
+//     fp32: out += s * (acc - (c + zp) * sum_k a_k); with per-channel scales there is one fold at the end;
+//   * bias, rounding, 16-byte (int4: 8 channels) or 8-byte stores.
+// The weights are read from HBM once per 256 rows; tiles of the same channels and different rows follow
+// each other on one XCD and share the weights through its L2.
+//
+// Reference semantics: flashnn/quant_gemm.py:148-206; the Triton kernels this replaces for large M:
+// flashnn/triton_kernels/gemm_a16w4.py:209-333, gemm_a16w8.py:179-272.
+#include <type_traits>
+
+#include "wo_common.h"
+
+namespace fnn {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+template <int WBITS, int ADT, bool G128, int SDT, int BM>
+__global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const int tiles_m, const int tiles) {
+    typedef MfmaT<ADT> MT;
+    static_assert(WBITS == 4 || BM == 128, "three stages of 128 int8 weight rows leave room for 128 activation rows");
+    constexpr int NH = WBITS == 4 ? 2 : 1;          // channels per weight row
+    constexpr int BN = 128;                          // channels per workgroup
+    constexpr int WROWS = BN / NH;                   // weight rows per workgroup
+    constexpr int WGM = 2, WGN = 4;                  // waves along M and N
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;    // wave tile: 128 or 64 rows x 32 channels
+    constexpr int FB = WTM / 16;                     // activation fragments per wave
+    constexpr int NF = WTN / NH / 16;                // 16-row weight fragments per wave (int4: 1, int8: 2)
+    constexpr int NA = NF * NH;                      // A operands per k-step (int4: even and odd channel of the fragment)
+    constexpr float c_off = WBITS == 4 ? (ADT == FNN_F16 ? 1024.f + 8.f : 128.f + 8.f)
+                                       : (ADT == FNN_F16 ? 1024.f + 128.f : 128.f);
+    constexpr int ASTG = BM * 256;                   // bytes of an activation stage
+    constexpr int WSTG = WROWS * 128;                // bytes of a weight stage
+    constexpr int TSTG = 1024;                       // a table stage: scales of 128 channels, then zero points (16-bit)
+    __shared__ __attribute__((aligned(1024))) char sa0[ASTG];
+    __shared__ __attribute__((aligned(1024))) char sa1[ASTG];
+    __shared__ __attribute__((aligned(1024))) char sw0[WSTG];
+    __shared__ __attribute__((aligned(1024))) char sw1[WSTG];
+    __shared__ __attribute__((aligned(1024))) char sw2[WSTG];
+    __shared__ __attribute__((aligned(1024))) char st0[TSTG];
+    __shared__ __attribute__((aligned(1024))) char st1[TSTG];
+    __shared__ __attribute__((aligned(1024))) char st2[TSTG];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int row16 = lane & 15, g = lane >> 4;
+
+    // workgroups id, id + 8, .. share an XCD: the row tiles of one channel tile follow each other there
+    const int per_xcd = gridDim.x >> 3;
+    const int t = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (t >= tiles) return;
+    const int tile_n = t / tiles_m, tile_m = t - tile_n * tiles_m;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int KT = p.K / 128;
+
+    // ---- copies.  A wave instruction writes 1 KB of LDS, linear in the lane id; the swizzle is applied
+    // on the global side.  Activations: instruction i of a wave covers rows (i * 8 + wave) * 4 .. + 3,
+    // lane L row L >> 4, slot L & 15 holding chunk (L & 15) ^ (row & 15).
+    // (row offsets are formed when the copy is issued: eight registers holding them are eight the
+    // accumulators cannot have)
+    constexpr int NCA = BM / 32;
+    const int ar0 = wave * 4 + (lane >> 4);          // the lane's row in instruction 0; instruction i: + 32 i
+    const int ar_max = p.M - 1 - m0;                 // rows beyond M read the last row (and are not stored)
+    const uint32_t a_chunk = (((lane & 15) ^ (ar0 & 15)) << 4);
+    const uint32_t lda2 = (uint32_t)(p.lda * 2);
+    const char* const a_base = (const char*)p.act + (int64_t)m0 * p.lda * 2;
+    auto copy_a = [&](char* stage, int j) {
+        const char* src = a_base + (int64_t)min(j, KT - 1) * 256;        // scalar
+#pragma unroll
+        for (int i = 0; i < NCA; ++i) {
+            const uint32_t off = (uint32_t)min(ar0 + 32 * i, ar_max) * lda2 + a_chunk;
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + off), (lds_ptr_t)(stage + (i * 8 + wave) * 1024), 16, 0, 0);
+        }
+        // (the compiler keeps these offsets in registers where it has them to spare)
+    };
+    // Weights: instruction i of a wave covers weight rows (i * 8 + wave) * 8 .. + 7, lane L row L >> 3, slot
+    // L & 7 holding chunk (L & 7) ^ ((row >> 1) & 7).
+    constexpr int NCW = WROWS / 64;
+    uint32_t gw[NCW];
+#pragma unroll
+    for (int i = 0; i < NCW; ++i) {
+        const int r = (i * 8 + wave) * 8 + (lane >> 3);
+        gw[i] = (uint32_t)r * (uint32_t)p.ldw + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+    }
+    const char* const w_base = (const char*)p.qw + (int64_t)(n0 / NH) * p.ldw;
+    auto copy_w = [&](char* stage, int j) {
+        const char* src = w_base + (int64_t)min(j, KT - 1) * 128;
+#pragma unroll
+        for (int i = 0; i < NCW; ++i)
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + gw[i]), (lds_ptr_t)(stage + (i * 8 + wave) * 1024), 16, 0, 0);
+    };
+    // Tables: 256 bytes of scales and 256 bytes of zero points per slab; every wave issues the same copy
+    // (lanes 0..15 the scales, 16..31 the zero points, the rest a second time), so that all waves count
+    // the same number of loads.
+    constexpr int NCT = G128 ? 1 : 0;
+    const bool has_zp = p.zp != nullptr;
+    const char* const t_src = (lane & 16) && has_zp ? (const char*)p.zp : (const char*)p.scale;
+    const uint32_t gt = (uint32_t)n0 * 2 + (lane & 15) * 16;
+    auto copy_t = [&](char* stage, int j) {
+        if constexpr (G128) {
+            const int64_t off = (int64_t)min(j, KT - 1) * p.N * 2;
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(t_src + off + gt), (lds_ptr_t)stage, 16, 0, 0);
+        }
+    };
+    auto wait_barrier = [&]() {   // everything but the newest weight copies has landed, for every wave
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0070 | (NCW & 15));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // ---- reads
+    // weight fragment f of the wave: rows wn * (64 / NH) + f * 16 + row16; 16 bytes = k 64 h + 16 g .. + 15
+    int w_rd[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) w_rd[h] = (wn * (WTN / NH) + row16) * 128 + (((4 * h + g) ^ ((row16 >> 1) & 7)) << 4);
+    // activation fragment b: rows wm * WTM + b * 16 + row16; k-step (h, q): chunk 8 h + 2 g + q
+    int a_rd[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) a_rd[h][q] = (wm * WTM + row16) * 256 + (((8 * h + 2 * g + q) ^ row16) << 4);
+
+    // G128: outv is the running output and a slab's accumulators live only while one activation fragment is
+    // worked on; per-channel scales: outv accumulates over all of K, asum the activation row sums
+    v4f outv[NA][FB], asum[FB];
+#pragma unroll
+    for (int b = 0; b < FB; ++b) {
+        asum[b] = v4f{0, 0, 0, 0};
+#pragma unroll
+        for (int a = 0; a < NA; ++a) outv[a][b] = v4f{0, 0, 0, 0};
+    }
+    const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+    const v4f zero4 = v4f{0, 0, 0, 0};
+    const float zmul = has_zp ? 1.f : 0.f;
+    typedef typename std::conditional<NH == 2, v4u, v2u>::type tab_t;
+
+    // One slab.  All of the slab's weights are converted first (A operand a of k-step ks; int4: operand
+    // 2 f + (0 even, 1 odd channel) of fragment f, int8: operand = fragment).  Then one activation fragment
+    // at a time: its four k-steps against all operands (five independent MFMA chains, the fifth against
+    // ones for the row sums) and, with group scales, the fold of those accumulators into the running
+    // output, out += s * (acc - (c + zp) * sum a) - vector-ALU work that has the MFMAs of the next
+    // fragment to run under, and accumulators that are dead before the next fragment needs registers.
+    auto slab = [&](const char* sa, const char* sw, const char* stg) {
+        v4u A[4][NA];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+                const v4u w = *(const v4u*)(sw + w_rd[h] + f * 16 * 128);
+                if constexpr (WBITS == 4)
+                    convert_w4_nat<ADT>(w, A[2 * h][2 * f], A[2 * h + 1][2 * f], A[2 * h][2 * f + 1], A[2 * h + 1][2 * f + 1]);
+                else
+                    convert_w8<ADT>(w, A[2 * h][f], A[2 * h + 1][f]);
+            }
+        float sc[NA][4], zc[NA][4];
+        if constexpr (G128) {
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+                const int ch = wn * WTN + f * 16 * NH + g * 4 * NH;   // this lane's 4 rows of fragment f: NH * 4 consecutive channels
+                const tab_t sv = *(const tab_t*)(stg + ch * 2);
+                const tab_t zv = *(const tab_t*)(stg + 256 + ch * 2);
+#pragma unroll
+                for (int o = 0; o < NH; ++o)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int c = NH * r + o;    // channel within the lane's NH * 4
+                        sc[NH * f + o][r] = bits_to_f32<SDT>((sv[c >> 1] >> (16 * (c & 1))) & 0xFFFFu);
+                        zc[NH * f + o][r] = c_off + zmul * bits_to_f32<SDT>((zv[c >> 1] >> (16 * (c & 1))) & 0xFFFFu);
+                    }
+            }
+        }
+        if constexpr (G128) {
+            // software pipeline over the activation fragments: the MFMAs of fragment b are issued between
+            // the fold instructions of fragment b - 1 (one MFMA, then a few vector instructions, and so on),
+            // so that both units work at once within one wave
+            constexpr int NM = 4 * (NA + 1);         // MFMAs per fragment
+            constexpr int NV = NA * 4 * 2;           // fold instructions per fragment
+            constexpr int VPM = (NV + NM - 1) / NM;
+            v4f acc[2][NA], as[2];
+#pragma unroll
+            for (int b = 0; b <= FB; ++b) {
+                if (b < FB) {
+                    v4u B[4];
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) B[ks] = *(const v4u*)(sa + a_rd[ks >> 1][ks & 1] + b * 16 * 256);
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+                        for (int a = 0; a < NA; ++a) acc[b & 1][a] = MT::mma(A[ks][a], B[ks], ks == 0 ? zero4 : acc[b & 1][a]);
+                        as[b & 1] = MT::mma(ones, B[ks], ks == 0 ? zero4 : as[b & 1]);
+                    }
+                }
+                if (b > 0) {
+                    const int pb = b - 1;
+#pragma unroll
+                    for (int a = 0; a < NA; ++a)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            outv[a][pb][r] += sc[a][r] * (acc[pb & 1][a][r] - zc[a][r] * as[pb & 1][r]);
+                }
+                if (b > 0 && b < FB) {
+#pragma unroll
+                    for (int q = 0; q < NM; ++q) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < FB; ++b) {
+                v4u B[4];
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) B[ks] = *(const v4u*)(sa + a_rd[ks >> 1][ks & 1] + b * 16 * 256);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+                    for (int a = 0; a < NA; ++a) outv[a][b] = MT::mma(A[ks][a], B[ks], outv[a][b]);
+                    asum[b] = MT::mma(ones, B[ks], asum[b]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+#define FNN_TILE_ITER(CA, CW, CT, FA, FW, FT, J)                          \
+    do {                                                                  \
+        wait_barrier();                                                   \
+        copy_a(FA, (J) + 1);                                              \
+        copy_t(FT, (J) + 1);                                              \
+        copy_w(FW, (J) + 2);                                              \
+        __builtin_amdgcn_sched_barrier(0);                                \
+        slab(CA, CW, CT);                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                \
+    } while (0)
+
+    // prologue, in the order the loop issues them: slab 0 whole, then the weights of slab 1
+    copy_a(sa0, 0);
+    copy_t(st0, 0);
+    copy_w(sw0, 0);
+    copy_w(sw1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // the stages rotate with periods 2 and 3: six iterations per round
+    int j = 0;
+    for (; j + 6 <= KT; j += 6) {
+        FNN_TILE_ITER(sa0, sw0, st0, sa1, sw2, st1, j);
+        FNN_TILE_ITER(sa1, sw1, st1, sa0, sw0, st2, j + 1);
+        FNN_TILE_ITER(sa0, sw2, st2, sa1, sw1, st0, j + 2);
+        FNN_TILE_ITER(sa1, sw0, st0, sa0, sw2, st1, j + 3);
+        FNN_TILE_ITER(sa0, sw1, st1, sa1, sw0, st2, j + 4);
+        FNN_TILE_ITER(sa1, sw2, st2, sa0, sw1, st0, j + 5);
+    }
+    // the remaining slabs (KT is a multiple of 2: checked on the host, so the activation stages line up)
+    if (j < KT) { FNN_TILE_ITER(sa0, sw0, st0, sa1, sw2, st1, j); }
+    if (j + 1 < KT) { FNN_TILE_ITER(sa1, sw1, st1, sa0, sw0, st2, j + 1); }
+    if (j + 2 < KT) { FNN_TILE_ITER(sa0, sw2, st2, sa1, sw1, st0, j + 2); }
+    if (j + 3 < KT) { FNN_TILE_ITER(sa1, sw0, st0, sa0, sw2, st1, j + 3); }
+#undef FNN_TILE_ITER
+    // ---- per-channel scales: one fold at the end
+    if constexpr (!G128) {
+#pragma unroll
+        for (int a = 0; a < NA; ++a) {
+            float sc[4], zc[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = n0 + wn * WTN + (NH == 2 ? (a >> 1) * 32 + 2 * (4 * g + r) + (a & 1) : a * 16 + 4 * g + r);
+                sc[r] = load_as_f32(p.scale, n, p.scale_dtype);
+                zc[r] = c_off + (has_zp ? load_as_f32(p.zp, n, p.zp_dtype) : 0.f);
+            }
+#pragma unroll
+            for (int b = 0; b < FB; ++b)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) outv[a][b][r] = sc[r] * (outv[a][b][r] - zc[r] * asum[b][r]);
+        }
+    }
+
+    // ---- bias, rounding, store: lane (row16, g) holds, for row m = .. + row16 of fragment b, the channels
+    // int4: n0 + wn * 64 + f * 32 + 8 g .. + 7 (even and odd operands interleaved); int8: .. + f * 16 + 4 g .. + 3
+    const bool out_f16 = p.out_dtype == FNN_F16;
+    const bool vec_out = (p.ldc % 8) == 0 && ((uintptr_t)p.out % 16) == 0;
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+        const int nb = n0 + wn * WTN + f * 16 * NH + g * 4 * NH;
+        float bias[4 * NH];
+#pragma unroll
+        for (int c = 0; c < 4 * NH; ++c) bias[c] = p.bias ? load_as_f32(p.bias, nb + c, p.bias_dtype) : 0.f;
+#pragma unroll
+        for (int b = 0; b < FB; ++b) {
+            const int m = m0 + wm * WTM + b * 16 + row16;
+            if (m >= p.M) continue;
+            uint32_t pk[2 * NH];
+#pragma unroll
+            for (int c = 0; c < 4 * NH; c += 2) {
+                // channel c of the lane: int4: register c >> 1 of operand 2 f + (c & 1); int8: register c of operand f
+                const float v0 = (NH == 2 ? outv[2 * f][b][c >> 1] : outv[f][b][c]) + bias[c];
+                const float v1 = (NH == 2 ? outv[2 * f + 1][b][c >> 1] : outv[f][b][c + 1]) + bias[c + 1];
+                const uint32_t b0 = out_f16 ? f32_to_f16_bits(v0) : f32_to_bf16_bits(v0);
+                const uint32_t b1 = out_f16 ? f32_to_f16_bits(v1) : f32_to_bf16_bits(v1);
+                pk[c >> 1] = (b0 & 0xFFFFu) | (b1 << 16);
+            }
+            uint16_t* dst = (uint16_t*)p.out + (int64_t)m * p.ldc + nb;
+            if (vec_out) {
+                if constexpr (NH == 2) *(v4u*)dst = v4u{pk[0], pk[1], pk[2], pk[3]};
+                else *(v2u*)dst = v2u{pk[0], pk[1]};
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4 * NH; ++c) dst[c] = (uint16_t)(pk[c >> 1] >> (16 * (c & 1)));
+            }
+        }
+    }
+}
+
+// Launches the tiled kernel if the shape suits it; returns false otherwise.
+template <int WBITS, int ADT>
+static bool launch_tile_t(WoArgs& p, hipStream_t st) {
+    constexpr int NH = WBITS == 4 ? 2 : 1;
+    if (p.M <= 64 || p.N % 128 != 0 || p.K % 256 != 0 || p.K < 512) return false;
+    if (p.group != 0 && p.group != 128) return false;
+    if (p.lda % 8 != 0 || p.ldw % 16 != 0 || ((uintptr_t)p.qw % 16) != 0 || ((uintptr_t)p.act % 16) != 0) return false;
+    // the copies address rows with 32-bit offsets from the tile's first row
+    if ((int64_t)256 * p.lda * 2 >= (1LL << 31) || (int64_t)(128 / NH) * p.ldw >= (1LL << 31)) return false;
+    if (p.group == 128) {
+        const bool tables16 = is16(p.scale_dtype) && (!p.zp || p.zp_dtype == p.scale_dtype) &&
+                              ((uintptr_t)p.scale % 16) == 0 && (!p.zp || ((uintptr_t)p.zp % 16) == 0);
+        if (!tables16) return false;
+    }
+    const int bm = (p.M <= 128 || WBITS == 8) ? 128 : 256;
+    const int tiles_m = (p.M + bm - 1) / bm;
+    const int tiles = tiles_m * (p.N / 128);
+    const dim3 grid(((tiles + 7) / 8) * 8);   // (workgroups beyond the last tile return at once)
+#define FNN_TILE(G, SDTV)                                                                                \
+    do {                                                                                                 \
+        if constexpr (WBITS == 4) {                                                                      \
+            if (bm == 256) {                                                                             \
+                gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 256><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles); \
+                break;                                                                                   \
+            }                                                                                            \
+        }                                                                                                \
+        gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 128><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles);    \
+    } while (0)
+    if (p.group == 128) {
+        if (p.scale_dtype == FNN_F16) FNN_TILE(true, FNN_F16);
+        else FNN_TILE(true, FNN_BF16);
+    } else {
+        FNN_TILE(false, FNN_F16);
+    }
+#undef FNN_TILE
+    return true;
+}
+
+bool launch_wo_tile(WoArgs& p, int wbits, int act_dtype, hipStream_t st) {
+    if (wbits == 4) return act_dtype == FNN_F16 ? launch_tile_t<4, FNN_F16>(p, st) : launch_tile_t<4, FNN_BF16>(p, st);
+    return act_dtype == FNN_F16 ? launch_tile_t<8, FNN_F16>(p, st) : launch_tile_t<8, FNN_BF16>(p, st);
+}
+
+}  // namespace fnn

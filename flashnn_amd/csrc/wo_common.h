@@ -146,6 +146,8 @@ __device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4
 
 // gemm_wo_panel.hip: 9 .. a few hundred activation rows; false if the shape does not suit it
 bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
+// gemm_wo_tile.hip: more than 64 activation rows, tiled MFMA kernel; false if the shape does not suit it
+bool launch_wo_tile(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
 // the int4 per-channel kernel over gathered rows of a mixture of experts; false if the shape does not suit it
 bool launch_wo_panel_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t st);
 

@@ -551,6 +551,37 @@ def test_weight_only_many_rows_one_hot():
     np.testing.assert_allclose(out.float().cpu().numpy(), want.t().half().float().numpy(), rtol=2.0 ** -10, atol=1e-6)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("group", [0, 128])
+@pytest.mark.parametrize("M,N,K", [(65, 256, 512), (128, 384, 1024), (200, 128, 2560), (256, 512, 768), (300, 256, 1536),
+                                   (520, 128, 512)])
+def test_weight_only_tiled_large_m(bits, group, M, N, K):
+    """More than 64 activation rows: the tiled MFMA kernel (128- and 256-row tiles, a partial last row tile,
+    2 to 20 slabs: every position of the two- and three-stage rings), zero points, bias, fp16 and bf16
+    activations and tables."""
+    act_ty = torch.float16 if (M + N) % 256 else torch.bfloat16
+    scale_ty = torch.bfloat16 if M == 300 else torch.float16
+    case = _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp=M != 128, with_bias=M in (65, 256), seed=700 + M)
+    _wo_check(*case, group, bits, act_ty)
+
+
+def test_weight_only_tiled_one_hot():
+    """One-hot activation rows pick single weight columns exactly: the k order inside a slab, the row and
+    channel mapping of the tiled kernel (int4, group 128)."""
+    M, N, K = 160, 256, 1024
+    g = torch.Generator().manual_seed(78)
+    w = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(K // 128, N).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(-4, 4, (K // 128, N), generator=g).half()
+    ks = torch.randint(0, K, (M,), generator=g)
+    act = torch.zeros(M, K, dtype=torch.float16)
+    act[torch.arange(M), ks] = 2.0
+    qw = torch.from_numpy(O.pack_int4(w.numpy()))
+    out = flashnn_amd.GemmWeightOnly(torch.float16)(act.to(DEV), qw.to(DEV), scale.to(DEV), None, zp.to(DEV))
+    want = 2.0 * (w[:, ks].float() - zp[ks // 128].float().t()) * scale[ks // 128].float().t()   # [N, M]
+    np.testing.assert_allclose(out.float().cpu().numpy(), want.t().half().float().numpy(), rtol=2.0 ** -10, atol=1e-6)
+
+
 @pytest.mark.parametrize("M", [1, 8, 32])
 @pytest.mark.parametrize("kn", workloads.A16W8_DECODE_SHAPES)
 def test_a16w8_decode_config(M, kn):
