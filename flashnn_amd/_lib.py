@@ -17,6 +17,7 @@ _i64, _int, _ptr, _f32 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c
 _SIGNATURES = {
     "fnn_version": [],
     "fnn_last_error": [],
+    "fnn_last_kernel": [],
     "fnn_dynamic_quant": [_ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _int, _ptr],
     "fnn_rmsnorm_dquant": [_ptr, _ptr, _ptr, _ptr, _f32, _i64, _i64, _i64, _i64, _int, _int, _ptr],
     "fnn_rmsnorm": [_ptr, _ptr, _ptr, _f32, _i64, _i64, _i64, _i64, _int, _int, _ptr],
@@ -31,7 +32,7 @@ _SIGNATURES = {
     "fnn_fused_moe_a8w8": [_ptr] * 9 + [_i64] * 9 + [_int] * 7 + [_ptr],
     "fnn_fused_moe_a16w4": [_ptr] * 9 + [_i64] * 14 + [_int] * 8 + [_ptr],
 }
-_RESTYPE = {"fnn_last_error": ctypes.c_char_p}
+_RESTYPE = {"fnn_last_error": ctypes.c_char_p, "fnn_last_kernel": ctypes.c_char_p}
 
 _lib = None
 
@@ -87,6 +88,11 @@ def check(rc):
     if rc != 0:
         msg = load().fnn_last_error().decode("utf-8", "replace")
         raise FlashnnHipError(f"libflashnn_hip error {rc}: {msg}")
+
+
+def last_kernel():
+    """Name of the kernel the calling thread's last library call launched (fnn_last_kernel)."""
+    return load().fnn_last_kernel().decode("ascii", "replace")
 
 
 def require_gpu(*tensors):

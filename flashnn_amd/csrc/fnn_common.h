@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/flashnn_hip.h"
 
 namespace fnn {
@@ -85,7 +87,27 @@ __device__ __forceinline__ double wave_sum(double v) {
 
 // ---- host side ----------------------------------------------------------------------
 void set_error(const char* fmt, ...);
-int check_launch(const char* what);
+
+// Brackets the launches of one entry point: construct before the first launch, return done() after the
+// last.  done() reports an error only if the thread's last HIP error changed in between, and only then
+// takes it off the thread: an error that the caller's own HIP calls left before this call is neither
+// reported as ours nor cleared.  (A launch failing with the very code already pending goes unseen.)
+struct Call {
+    const char* fn;
+    hipError_t prior;
+    explicit Call(const char* fn);
+    int done() const;
+};
+
+// Raises a kernel's dynamic-LDS limit to the 160 KB of a gfx950 CU, once per device: `raised` is the launch
+// site's own bit mask of the devices done (function attributes are kept per device).
+void allow_large_lds(const void* kernel, std::atomic<uint64_t>& raised);
+
+// Records the kernel a launch site is about to run, with up to three numbers that tell its variants apart
+// (tile rows, tile columns, waves ...): fnn_last_kernel() returns the last one noted on the calling thread.
+// With FLASHNN_HIP_LOG=1 in the environment the first launch of every variant prints one line on stderr.
+// `name` must be a string literal (it is kept by pointer).
+void note_kernel(const char* name, int a = 0, int b = 0, int c = 0);
 
 inline bool is16(int dt) { return dt == FNN_F16 || dt == FNN_BF16; }
 inline bool isflt(int dt) { return dt == FNN_F16 || dt == FNN_BF16 || dt == FNN_F32; }

@@ -642,12 +642,32 @@ static TileChoice choose_tile(int64_t M, int64_t N) {
     return c;
 }
 
+// The same problem restricted to columns [n0, n0 + n) of the output (rows [n0, n0 + n) of B) ...
+static A8W8Args columns_from(const A8W8Args& p, int64_t n0, int n, int mode) {
+    A8W8Args q = p;
+    q.N = n;
+    q.b = p.b + n0 * p.ldb;
+    q.out = (char*)p.out + n0 * (mode == OUT_I32 ? 4 : 2);
+    if (p.acol) q.acol = (const char*)p.acol + n0 * (p.acol_dtype == FNN_F32 ? 4 : 2);
+    return q;
+}
+// ... and to rows [m0, m0 + m) of A and of the output.
+static A8W8Args rows_from(const A8W8Args& p, int64_t m0, int m, int mode) {
+    A8W8Args q = p;
+    q.M = m;
+    q.a = p.a + m0 * p.lda;
+    q.out = (char*)p.out + m0 * p.ldc * (mode == OUT_I32 ? 4 : 2);
+    if (p.arow) q.arow = (const char*)p.arow + m0 * (p.arow_dtype == FNN_F32 ? 4 : 2);
+    return q;
+}
+
 template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2>
 static void launch_mfma(A8W8Args& p, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
+    note_kernel("gemm_a8w8_ring_kernel", BM, BN, WGM * 2);
     gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, WGM><<<dim3(p.tiles_per_xcd * 8), dim3(WGM * 128), 0, st>>>(p);
 }
 
@@ -674,16 +694,15 @@ static void launch_tile(A8W8Args& p, hipStream_t st, int bm, int bn, int waves) 
     else launch_mfma<128, 128, MODE>(p, st);
 }
 
+// One launch plan for operands whose row offsets fit 32 bits (M * lda and N * ldb below 2^31 bytes).
 template <int MODE>
-static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn, int force_waves) {
-    // the MFMA kernel walks K in slabs of 128 bytes and addresses rows with 32-bit offsets
-    const bool fast = p.K % 32 == 0 && p.K >= 512 && p.lda % 16 == 0 && p.ldb % 16 == 0 &&
-                      ((uintptr_t)p.a % 16) == 0 && ((uintptr_t)p.b % 16) == 0 &&
-                      ((uintptr_t)p.out % 16) == 0 && (int64_t)p.M * p.lda < (1LL << 31) &&
-                      (int64_t)p.N * p.ldb < (1LL << 31);
+static void dispatch_band(A8W8Args& p, hipStream_t st, bool aligned, int force_bm, int force_bn, int force_waves) {
+    // the MFMA kernel walks K in slabs of 128 bytes
+    const bool fast = aligned && p.K % 32 == 0 && p.K >= 512;
     // few activation rows: stream the weights once (unless the caller names a tile of the tiled kernel)
     if (force_bm == 0 && p.M <= 64 && launch_a8w8_skinny(p, MODE, st)) return;
     if (!fast) {
+        note_kernel("gemm_a8w8_any_kernel");
         gemm_a8w8_any_kernel<MODE><<<dim3((p.N + 63) / 64, (p.M + 63) / 64), dim3(256), 0, st>>>(p);
         return;
     }
@@ -699,17 +718,35 @@ static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn, in
             A8W8Args q = p;
             q.N = 192 * c1;
             launch_tile<MODE>(q, st, 256, 192, 0);
-            const int64_t n_off = q.N;
-            q = p;
-            q.N = p.N - (int)n_off;
-            q.b = p.b + n_off * p.ldb;
-            q.out = (char*)p.out + n_off * (MODE == OUT_I32 ? 4 : 2);
-            if (p.acol) q.acol = (const char*)p.acol + n_off * (p.acol_dtype == FNN_F32 ? 4 : 2);
-            launch_tile<MODE>(q, st, 256, 128, 0);
+            launch_tile<MODE>(q = columns_from(p, q.N, p.N - q.N, MODE), st, 256, 128, 0);
             return;
         }
     }
     launch_tile<MODE>(p, st, c.bm, c.bn, 0);
+}
+
+// The kernels address a row of A or B as base + 32-bit byte offset.  Operands beyond that (M * lda or
+// N * ldb of 2^31 bytes and more: a long prefill, a very wide head) are cut on the host into bands of rows
+// and of columns that fit, each band a problem of its own on the same kernels.
+template <int MODE>
+static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn, int force_waves) {
+    const bool aligned = p.lda % 16 == 0 && p.ldb % 16 == 0 && ((uintptr_t)p.a % 16) == 0 &&
+                         ((uintptr_t)p.b % 16) == 0 && ((uintptr_t)p.out % 16) == 0;
+    constexpr int64_t kLimit = (1LL << 31) - 1;
+    const int64_t m_fit = kLimit / p.lda, n_fit = kLimit / p.ldb;
+    if (p.M <= m_fit && p.N <= n_fit) {
+        dispatch_band<MODE>(p, st, aligned, force_bm, force_bn, force_waves);
+        return;
+    }
+    // bands in whole tiles of every shape (rows: 256; columns: 768 = lcm(256, 192, 128)), so that the bands
+    // tile like the undivided problem and every band keeps the operands' alignment
+    const int64_t m_band = m_fit >= 256 ? m_fit / 256 * 256 : m_fit, n_band = n_fit >= 768 ? n_fit / 768 * 768 : n_fit;
+    for (int64_t m0 = 0; m0 < p.M; m0 += m_band)
+        for (int64_t n0 = 0; n0 < p.N; n0 += n_band) {
+            A8W8Args q = columns_from(p, n0, (int)(p.N - n0 < n_band ? p.N - n0 : n_band), MODE);
+            q = rows_from(q, m0, (int)(p.M - m0 < m_band ? p.M - m0 : m_band), MODE);
+            dispatch_band<MODE>(q, st, aligned && ((uintptr_t)q.out % 16) == 0, force_bm, force_bn, force_waves);
+        }
 }
 
 static int check_args(const char* fn, const void* out, const void* a, const void* b, int64_t M,
@@ -750,9 +787,10 @@ static int gemm_a8w8_entry(const char* fn, void* out, const void* a, const void*
     p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = out; p.arow = alpha_row; p.acol = alpha_col;
     p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
     p.out_dtype = out_dtype; p.arow_dtype = alpha_row_dtype; p.acol_dtype = alpha_col_dtype;
+    const Call call(fn);
     if (out_dtype == FNN_F16) dispatch<OUT_F16>(p, (hipStream_t)stream, tile_m, tile_n, waves);
     else dispatch<OUT_BF16>(p, (hipStream_t)stream, tile_m, tile_n, waves);
-    return check_launch(fn);
+    return call.done();
 }
 
 static int gemm_a8w8_i32_entry(const char* fn, int32_t* acc, const void* a, const void* b, int64_t M, int64_t N,
@@ -768,8 +806,9 @@ static int gemm_a8w8_i32_entry(const char* fn, int32_t* acc, const void* a, cons
     A8W8Args p{};
     p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = acc;
     p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    const Call call(fn);
     dispatch<OUT_I32>(p, (hipStream_t)stream, tile_m, tile_n, waves);
-    return check_launch(fn);
+    return call.done();
 }
 
 extern "C" int fnn_gemm_a8w8(void* out, const void* a, const void* b, const void* alpha_row,
@@ -840,6 +879,7 @@ extern "C" int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const v
     q.topk_w = topk_weights; q.topk_w_dtype = topk_weights_dtype; q.mul_w = mul_routed_weight ? 1 : 0;
     q.top_k = top_k; q.block_m = block_m; q.num_valid = (int)num_valid_tokens; q.EM = (int)EM;
     q.stride_be = stride_be; q.stride_scale_be = stride_scale_be;
+    const Call call(fn);
     launch_a8w8_moe(p, q, out_dtype == FNN_F16 ? OUT_F16 : OUT_BF16, (hipStream_t)stream);
-    return check_launch(fn);
+    return call.done();
 }

@@ -413,6 +413,7 @@ static bool launch_a8_panel_t(A8W8Args& p, hipStream_t st) {
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const int tiles = p.N / (16 * rt);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes), block(512);
+    note_kernel("gemm_a8w8_panel_kernel", mb, rt);
     if (rt == 4) {
         if (mb == 2) gemm_a8w8_panel_kernel<2, 4, MODE><<<grid, block, 0, st>>>(p, passes, MoeArgs{});
         else gemm_a8w8_panel_kernel<4, 4, MODE><<<grid, block, 0, st>>>(p, passes, MoeArgs{});
@@ -434,6 +435,7 @@ static bool launch_skinny_t(A8W8Args& p, hipStream_t st) {
         ((uintptr_t)p.a % 16) != 0 || ((uintptr_t)p.b % 16) != 0)
         return false;
     const dim3 grid((p.N + 15) / 16), block(kSkWaves * 64);
+    note_kernel("gemm_a8w8_skinny_kernel", (p.M + 15) / 16);
     if (p.M <= 16) gemm_a8w8_skinny_kernel<1, MODE><<<grid, block, 0, st>>>(p);
     else if (p.M <= 32) gemm_a8w8_skinny_kernel<2, MODE><<<grid, block, 0, st>>>(p);
     else if (p.M <= 48) gemm_a8w8_skinny_kernel<3, MODE><<<grid, block, 0, st>>>(p);
@@ -472,6 +474,7 @@ static bool launch_moe_t(A8W8Args& p, const MoeArgs& q, hipStream_t st) {
                       q.stride_be % 16 == 0 && ((uintptr_t)p.a % 16) == 0 && ((uintptr_t)p.b % 16) == 0 &&
                       q.block_m % 16 == 0 && q.EM % q.block_m == 0;
     if (!fast) {
+        note_kernel("moe_a8w8_any_kernel");
         moe_a8w8_any_kernel<MODE><<<dim3(q.EM, (p.N + 255) / 256), dim3(256), 0, st>>>(p, q);
         return true;
     }
@@ -491,6 +494,7 @@ static bool launch_moe_t(A8W8Args& p, const MoeArgs& q, hipStream_t st) {
     const int passes = q.EM / (mb * 16);
     const int tiles = p.N / (16 * rt);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes), block(512);
+    note_kernel("gemm_a8w8_panel_kernel(moe)", mb, rt);
     if (rt == 4) {
         if (mb == 2) gemm_a8w8_panel_kernel<2, 4, MODE, true><<<grid, block, 0, st>>>(p, passes, q);
         else gemm_a8w8_panel_kernel<4, 4, MODE, true><<<grid, block, 0, st>>>(p, passes, q);

@@ -1264,6 +1264,7 @@ static void launch_stream(WoArgs& p, hipStream_t st) {
     const int wrows = WBITS == 4 ? p.N / 2 : p.N;
     const int tiles = (wrows + 15) / 16;
     const dim3 grid(((tiles + 7) / 8) * 8), block(kWoWaves * 64);
+    note_kernel("gemm_wo_stream_kernel", WBITS, MB, p.group);
     if (p.group > 0) gemm_wo_stream_kernel<WBITS, ADT, MB, true><<<grid, block, 0, st>>>(p);
     else gemm_wo_stream_kernel<WBITS, ADT, MB, false><<<grid, block, 0, st>>>(p);
 }
@@ -1343,11 +1344,9 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
 #define FNN_GEMV_FLAT(MPV)                                                                                    \
     do {                                                                                                      \
         auto kfn = gemm_wo_gemv_flat_kernel<WBITS, ADT, MPV>;                                                  \
-        static bool attr_set = false;                                                                         \
-        if (!attr_set) {                                                                                      \
-            (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
-            attr_set = true;                                                                                  \
-        }                                                                                                     \
+        static std::atomic<uint64_t> raised{0};                                                               \
+        allow_large_lds((const void*)kfn, raised);                                                            \
+        note_kernel("gemm_wo_gemv_flat_kernel", WBITS, MPV, wpw);                                             \
         kfn<<<g2, dim3(512), smem_f, st>>>(p, wpw, plan);                                                     \
     } while (0)
                     if (p.M == 1) FNN_GEMV_FLAT(1);
@@ -1361,11 +1360,9 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
     do {                                                                                                  \
         auto kfn = full ? gemm_wo_gemv_kernel<WBITS, ADT, G, MPV, 8, true>                               \
                         : gemm_wo_gemv_kernel<WBITS, ADT, G, MPV, 8, false>;                             \
-        static bool attr_set[2] = {false, false};                                                         \
-        if (!attr_set[full]) {                                                                            \
-            (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
-            attr_set[full] = true;                                                                        \
-        }                                                                                                 \
+        static std::atomic<uint64_t> raised[2] = {{0}, {0}};                                              \
+        allow_large_lds((const void*)kfn, raised[full]);                                                  \
+        note_kernel("gemm_wo_gemv_kernel", WBITS, MPV, wpw);                                              \
         kfn<<<g2, b2, smem, st>>>(p, wpw);                                                                \
     } while (0)
             if (p.M == 1) FNN_GEMV(true, 1);
@@ -1383,6 +1380,7 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
         if (smem > 64 * 1024) return false;   // beyond what a launch may ask for without raising the kernel's limit
 #define FNN_DEC(G, MPV, ...)                                                                         \
     do {                                                                                             \
+        note_kernel("gemm_wo_decode_lds_kernel", WBITS, MPV, full16 ? 16 : full8 ? 8 : -16);             \
         if (full16) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, true, ##__VA_ARGS__><<<grid, block, smem, st>>>(p); \
         else if (full8) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 8, true, ##__VA_ARGS__><<<grid, block, smem, st>>>(p); \
         else gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, false, ##__VA_ARGS__><<<grid, block, smem, st>>>(p);  \
@@ -1405,6 +1403,7 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
     }
     const size_t smem = fixed + (act_lds ? act_bytes : 0);
     if (smem > 64 * 1024) return false;
+    note_kernel("gemm_wo_decode_kernel", WBITS, p.group, act_lds);
     if (p.group > 0) {
         if (act_lds) gemm_wo_decode_kernel<WBITS, ADT, true, true><<<grid, block, smem, st>>>(p);
         else gemm_wo_decode_kernel<WBITS, ADT, true, false><<<grid, block, smem, st>>>(p);
@@ -1423,6 +1422,7 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
     if (p.group == 0 && p.K % 128 != 0 && launch_wo_panel(p, WBITS, ADT, st)) return;
     if (!fast) {
         const int64_t total = (int64_t)p.M * p.N;
+        note_kernel("gemm_wo_any_kernel", WBITS);
         gemm_wo_any_kernel<WBITS, ADT><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(p);
         return;
     }
@@ -1471,9 +1471,10 @@ static int run_wo(const char* fn, void* out, const void* act, const void* qw, co
     p.act = act; p.qw = (const int8_t*)qw; p.scale = scale; p.zp = zp; p.bias = bias; p.out = out;
     p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldw = ldw; p.ldc = ldc; p.group = (int)group;
     p.out_dtype = out_dtype; p.scale_dtype = scale_dtype; p.zp_dtype = zp_dtype; p.bias_dtype = bias_dtype;
+    const Call call(fn);
     if (act_dtype == FNN_F16) dispatch_wo<WBITS, FNN_F16>(p, (hipStream_t)stream);
     else dispatch_wo<WBITS, FNN_BF16>(p, (hipStream_t)stream);
-    return check_launch(fn);
+    return call.done();
 }
 
 }  // namespace fnn
@@ -1589,10 +1590,12 @@ extern "C" int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const 
     hipStream_t st = (hipStream_t)stream;
     // the weight-streaming kernel takes per-channel scales and groups of 128 (launch_wo_panel_moe checks the layout)
     const bool fast = (group == 0 || group == 128) && (!zero_points || zp_dtype != FNN_I8);
+    const Call call(fn);
     if (!(fast && launch_wo_panel_moe(p, q, act_dtype, st))) {
         const dim3 grid((unsigned)EM, (unsigned)((2 * N + 255) / 256));
+        note_kernel("moe_a16w4_any_kernel");
         if (act_dtype == FNN_F16) moe_a16w4_any_kernel<FNN_F16><<<grid, dim3(256), 0, st>>>(p, q);
         else moe_a16w4_any_kernel<FNN_BF16><<<grid, dim3(256), 0, st>>>(p, q);
     }
-    return check_launch(fn);
+    return call.done();
 }

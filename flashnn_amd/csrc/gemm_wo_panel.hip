@@ -550,6 +550,7 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     // fp16 activations with per-channel fp16 scales (and zero points): the reference's own per-weight rounding
     constexpr bool CAN_REFQ = ADT == FNN_F16;
     const bool refq = CAN_REFQ && p.group == 0 && p.scale_dtype == FNN_F16 && (!p.zp || p.zp_dtype == FNN_F16);
+    note_kernel(refq ? "gemm_wo_panel_kernel(per-weight rounding)" : "gemm_wo_panel_kernel", WBITS, mb, rt);
 #define FNN_PANEL3(G, SDTV, MBV, RTV, NTLV)                                                              \
     do {                                                                                                 \
         if constexpr (CAN_REFQ && !G) {                                                                  \
@@ -626,6 +627,7 @@ static bool launch_panel_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
     const int passes = q.EM / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);
     p.m_base = 0;
+    note_kernel("gemm_wo_panel_kernel(moe)", 4, mb, rt);
 #define FNN_MOE2(G, SDTV, MBV, RTV) \
     gemm_wo_panel_kernel<4, ADT, G, SDTV, MBV, RTV, 4, false, true><<<grid, dim3(512), 0, st>>>(p, passes, q)
 #define FNN_MOE(G, SDTV)                                   \

@@ -352,6 +352,7 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
     const int tiles_m = (p.M + bm - 1) / bm;
     const int tiles = tiles_m * (p.N / 128);
     const dim3 grid(((tiles + 7) / 8) * 8);   // (workgroups beyond the last tile return at once)
+    note_kernel("gemm_wo_tile_kernel", WBITS, bm, 128);
 #define FNN_TILE(G, SDTV)                                                                                \
     do {                                                                                                 \
         if constexpr (WBITS == 4) {                                                                      \

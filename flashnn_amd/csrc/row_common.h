@@ -72,9 +72,9 @@ __device__ __forceinline__ float quant_rcp(float s) { return s == 0.f ? 0.f : 1.
 // Byte j of w <- the integer-valued float r as int8, saturated to [-128, 127]: r + 128 is exact, lands in
 // [0, 255] as an unsigned byte, and v_cvt_pk_u8_f32 saturates, converts and inserts it in one instruction
 // (conversion, clamp and packing took five).  The finished dword still needs its sign bits flipped:
-// w ^ 0x80808080.  Only for the operators whose reference clamps (the norm + quant layers): plain dynamic
-// quantisation casts without a clamp, and a bf16 row whose scale rounded down does reach 128 there, which
-// the cast wraps to -128.
+// w ^ 0x80808080.  Used by every quantising kernel: the norm + quant layers clamp in the reference, and plain
+// dynamic quantisation is clamped here as well (a bf16 row whose scale rounded down reaches 128, which an
+// unclamped cast wraps to -128).
 __device__ __forceinline__ uint32_t put_biased_byte(float r, int j, uint32_t w) {
     return __builtin_amdgcn_cvt_pk_u8_f32(r + 128.f, (uint32_t)j, w);
 }

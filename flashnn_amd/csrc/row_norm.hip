@@ -210,6 +210,7 @@ static void launch_norm(const NormArgs& p, int64_t M, hipStream_t st) {
                      (OP == OP_RMS || ((uintptr_t)p.beta % 16) == 0);
     if (vec) {
         const int nv = (p.K / 8 + kRowThreads - 1) / kRowThreads;
+        note_kernel("norm_vec_kernel", OP, nv, M <= 1024 && nv <= 4);
         // up to four workgroups per CU are "few rows": every row is then resident at once either way
 #define FNN_NORM(NV)                                                                   \
     do {                                                                               \
@@ -219,6 +220,7 @@ static void launch_norm(const NormArgs& p, int64_t M, hipStream_t st) {
         FNN_ROW_DISPATCH_NV(nv, FNN_NORM);
 #undef FNN_NORM
     } else {
+        note_kernel("norm_any_kernel", OP);
         norm_any_kernel<DT, OP><<<grid, block, 0, st>>>(p);
     }
 }
@@ -242,9 +244,10 @@ static int run_norm(const char* fn, void* out, void* scale, const void* x, const
     if (M > 0x7FFFFFFFLL || K > 0x7FFFFFFFLL) { set_error("%s: shape too large", fn); return FNN_ERR_UNSUPPORTED; }
     if (M == 0) return FNN_OK;
     NormArgs p{out, (uint16_t*)scale, (const uint16_t*)x, gamma, beta, gb_dtype, eps, (int)K, ldx, ldo};
+    const Call call(fn);
     if (x_dtype == FNN_F16) launch_norm<FNN_F16, OP>(p, M, (hipStream_t)stream);
     else launch_norm<FNN_BF16, OP>(p, M, (hipStream_t)stream);
-    return check_launch(fn);
+    return call.done();
 }
 
 }  // namespace fnn

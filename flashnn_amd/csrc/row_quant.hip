@@ -40,19 +40,22 @@ __global__ __launch_bounds__(kRowThreads) void dynamic_quant_vec_kernel(
     const uint32_t sbits = f32_to_bits<DT>(mx / 127.0f);
     const float s = bits_to_f32<DT>(sbits);
     if (threadIdx.x == 0) scale[row] = (uint16_t)(DT == FNN_F16 ? sbits : f32_to_f16_bits(s));
-    const float rcp = 1.0f / s;
+    // The quotient is clamped to [-128, 127] (the saturating byte conversion does it): with bf16 input the
+    // scale max/127 can round down so far that the row maximum quantises to 128, which an unclamped
+    // conversion to int8 wraps to -128 - the sign of the row's largest activation.  fp16 rows never exceed 127.
+    const float rcp = quant_rcp(s);   // 0 for an all-zero row: every quotient is then 0
     v2u* qr = (v2u*)(q + row * ldq);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int idx = threadIdx.x + i * kRowThreads;
         if (idx < nvec) {
-            int o[8];
+            uint32_t w[2] = {0, 0};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                o[2 * j] = s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(v[i][j] & 0xFFFFu), s, rcp);
-                o[2 * j + 1] = s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(v[i][j] >> 16), s, rcp);
+                w[j >> 1] = put_biased_byte(quant_in_dtype_f<DT>(bits_to_f32<DT>(v[i][j] & 0xFFFFu), s, rcp), 2 * (j & 1), w[j >> 1]);
+                w[j >> 1] = put_biased_byte(quant_in_dtype_f<DT>(bits_to_f32<DT>(v[i][j] >> 16), s, rcp), 2 * (j & 1) + 1, w[j >> 1]);
             }
-            qr[idx] = v2u{pack4(o[0], o[1], o[2], o[3]), pack4(o[4], o[5], o[6], o[7])};
+            qr[idx] = v2u{w[0] ^ 0x80808080u, w[1] ^ 0x80808080u};
         }
     }
 }
@@ -73,7 +76,7 @@ __global__ __launch_bounds__(kRowThreads) void dynamic_quant_any_kernel(
     const float rcp = 1.0f / s;
     int8_t* qr = q + row * ldq;
     for (int k = threadIdx.x; k < K; k += kRowThreads)
-        qr[k] = (int8_t)(s == 0.f ? 0 : quant_in_dtype<DT>(bits_to_f32<DT>(xr[k]), s, rcp));
+        qr[k] = (int8_t)(s == 0.f ? 0 : min(quant_in_dtype<DT>(bits_to_f32<DT>(xr[k]), s, rcp), 127));
 }
 
 // ---------------------------------------------------------------- rmsnorm + quant
@@ -261,10 +264,12 @@ static void launch_dq(int8_t* q, uint16_t* scale, const uint16_t* x, int64_t M, 
     const dim3 grid((unsigned)M), block(kRowThreads);
     if (vec_ok(x, q, K, ldx, ldq)) {
         const int nv = (K / 8 + kRowThreads - 1) / kRowThreads;
+        note_kernel("dynamic_quant_vec_kernel", nv);
 #define FNN_DQ(NV) dynamic_quant_vec_kernel<DT, NV><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq)
         FNN_ROW_DISPATCH_NV(nv, FNN_DQ);
 #undef FNN_DQ
     } else {
+        note_kernel("dynamic_quant_any_kernel");
         dynamic_quant_any_kernel<DT><<<grid, block, 0, st>>>(q, scale, x, K, ldx, ldq);
     }
 }
@@ -281,6 +286,7 @@ static void launch_rq(int8_t* q, uint16_t* scale, const uint16_t* x, const void*
         const int nvw = (K / 8 + kWave - 1) / kWave;
         if (M >= 2048 && nvw <= 4) {
             const dim3 wgrid((unsigned)((M + 3) / 4));
+            note_kernel("rmsnorm_dquant_wave_kernel", nvw <= 1 ? 1 : nvw <= 2 ? 2 : 4);
 #define FNN_RQW(NV) rmsnorm_dquant_wave_kernel<DT, NV><<<wgrid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, M, K, ldx, ldq)
             if (nvw <= 1) FNN_RQW(1);
             else if (nvw <= 2) FNN_RQW(2);
@@ -289,6 +295,7 @@ static void launch_rq(int8_t* q, uint16_t* scale, const uint16_t* x, const void*
             return;
         }
         const int nv = (K / 8 + kRowThreads - 1) / kRowThreads;
+        note_kernel("rmsnorm_dquant_vec_kernel", nv, M <= 1024 && nv <= 4);
 #define FNN_RQ(NV)                                                                                          \
     do {                                                                                                    \
         if (M <= 1024 && NV <= 4)                                                                           \
@@ -298,6 +305,7 @@ static void launch_rq(int8_t* q, uint16_t* scale, const uint16_t* x, const void*
         FNN_ROW_DISPATCH_NV(nv, FNN_RQ);
 #undef FNN_RQ
     } else {
+        note_kernel("rmsnorm_dquant_any_kernel");
         rmsnorm_dquant_any_kernel<DT><<<grid, block, 0, st>>>(q, scale, x, gamma, gdt, eps, K, ldx, ldq);
     }
 }
@@ -326,11 +334,12 @@ extern "C" int fnn_dynamic_quant(void* q, void* scale, const void* x, int64_t M,
     if (rc != FNN_OK) return rc;
     if (M == 0) return FNN_OK;
     hipStream_t st = (hipStream_t)stream;
+    const Call call("fnn_dynamic_quant");
     if (x_dtype == FNN_F16)
         launch_dq<FNN_F16>((int8_t*)q, (uint16_t*)scale, (const uint16_t*)x, M, (int)K, ldx, ldq, st);
     else
         launch_dq<FNN_BF16>((int8_t*)q, (uint16_t*)scale, (const uint16_t*)x, M, (int)K, ldx, ldq, st);
-    return check_launch("fnn_dynamic_quant");
+    return call.done();
 }
 
 extern "C" int fnn_rmsnorm_dquant(void* q, void* scale, const void* x, const void* gamma, float eps,
@@ -342,9 +351,10 @@ extern "C" int fnn_rmsnorm_dquant(void* q, void* scale, const void* x, const voi
     if (!isflt(gamma_dtype)) { set_error("fnn_rmsnorm_dquant: bad gamma type"); return FNN_ERR_UNSUPPORTED; }
     if (M == 0) return FNN_OK;
     hipStream_t st = (hipStream_t)stream;
+    const Call call("fnn_rmsnorm_dquant");
     if (x_dtype == FNN_F16)
         launch_rq<FNN_F16>((int8_t*)q, (uint16_t*)scale, (const uint16_t*)x, gamma, gamma_dtype, eps, M, (int)K, ldx, ldq, st);
     else
         launch_rq<FNN_BF16>((int8_t*)q, (uint16_t*)scale, (const uint16_t*)x, gamma, gamma_dtype, eps, M, (int)K, ldx, ldq, st);
-    return check_launch("fnn_rmsnorm_dquant");
+    return call.done();
 }

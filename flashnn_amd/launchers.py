@@ -147,11 +147,10 @@ def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col, tile=None):
             _lib.dtype_code(ar.dtype), _lib.dtype_code(ac.dtype))
     stream = _lib.current_stream(a.device)
     # shape-keyed tuned tile, named as the reference names the launch (gemm_a8w8.py:199)
-    method_name = f"gemm_a8w8_{M}_{N}_{K}"
     if tile is None:
-        tile = tuned_configs.CACHE.lookup(method_name)
+        tile = tuned_configs.CACHE.shape_tile("gemm_a8w8", M, N, K)
     if tile is None and get_autotune_triton_kernels():
-        tile = tuned_configs.tune(method_name, tuned_configs.A8W8_CANDIDATES,
+        tile = tuned_configs.tune(f"gemm_a8w8_{M}_{N}_{K}", tuned_configs.A8W8_CANDIDATES,
                                   lambda t: _lib.check(lib.fnn_gemm_a8w8_tiled(*args, *t, stream)))
     if tile is None or tile[0] == 0:
         _lib.check(lib.fnn_gemm_a8w8(*args, stream))

@@ -51,12 +51,31 @@ def deserialize_best_config(entry):
 
 
 class TunedConfigs:
-    """In-memory view of the JSON file (read once per path; written through on every new record)."""
+    """In-memory view of the JSON file (read once per path; written through on every new record).
+
+    shape_tile() is what a launcher calls on every GEMM: it answers from a dictionary keyed by the shape and
+    touches neither the environment nor the file once a shape has been resolved.  The environment (file
+    path, forced re-tune list) is therefore read when a shape is first met; after changing it inside a
+    running process call reset()."""
 
     def __init__(self):
         self._path = None
         self._data = {}
         self._tuned_now = set()      # method names tuned by this process (a forced re-tune runs once)
+        self._by_shape = {}          # (prefix, M, N, K) -> tile or None, resolved once
+
+    def reset(self):
+        """Forget everything read so far: the next lookup reads the environment and the file again."""
+        self.__init__()
+
+    def shape_tile(self, prefix, M, N, K):
+        """The recorded tile for "<prefix>_M_N_K", or None; resolved once per shape."""
+        key = (prefix, M, N, K)
+        try:
+            return self._by_shape[key]
+        except KeyError:
+            tile = self._by_shape[key] = self.lookup(f"{prefix}_{M}_{N}_{K}")
+            return tile
 
     def _load(self):
         path = json_file_path()
@@ -82,6 +101,7 @@ class TunedConfigs:
         data = self._load()
         data[method_name] = serialize_best_config(tile)
         self._tuned_now.add(method_name)
+        self._by_shape.clear()
         os.makedirs(os.path.dirname(self._path), exist_ok=True)
         tmp = self._path + ".tmp"
         with open(tmp, "w", encoding="utf-8") as f:

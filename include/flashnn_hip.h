@@ -17,8 +17,15 @@
  *   - return value: 0 ok, FNN_ERR_ARG (-1) bad argument, FNN_ERR_UNSUPPORTED (-2)
  *     shape/dtype not handled, FNN_ERR_HIP (-3) HIP runtime error.  After a non-zero
  *     return fnn_last_error() gives a thread-local, human-readable message.
- *   - the library holds no mutable global state apart from that message; calls are
- *     re-entrant and never allocate, free or synchronise.
+ *   - calls are re-entrant and never allocate, free or synchronise.  State kept between calls:
+ *     per thread the last error message and the name of the last kernel launched; per
+ *     process, set once and never changed again, which devices have had a kernel's LDS
+ *     limit raised and (only with FLASHNN_HIP_LOG=1) which kernel variants have been
+ *     logged.  No call reads a setting that another call can change.
+ *   - an error the calling thread's own HIP calls left pending before a call is neither
+ *     reported by the call nor cleared by it.
+ *   - FLASHNN_HIP_LOG=1 in the environment (read once): one line on stderr the first time
+ *     each kernel variant is launched in the process.
  */
 #ifndef FLASHNN_HIP_H_
 #define FLASHNN_HIP_H_
@@ -40,6 +47,15 @@ int fnn_version(void);
 
 /* Message describing the last failure on the calling thread ("" if none). */
 const char* fnn_last_error(void);
+
+/*
+ * Name of the kernel that the calling thread's last call launched, with the numbers that tell
+ * its variants apart, e.g. "gemm_a8w8_ring_kernel<256,192,4>" (tile rows, tile columns, waves);
+ * "" before the first launch.  A call that launches two kernels (a column split) names the
+ * last.  The pointer stays valid until the thread's next call of this function.  The reference
+ * logs the chosen configuration through loguru (flashnn/triton_kernels/triton_utils.py:112,139).
+ */
+const char* fnn_last_kernel(void);
 
 /*
  * Per-token symmetric int8 quantisation.

@@ -55,6 +55,30 @@ def test_dynamic_quant_outliers_and_zero_row():
     assert (np.delete(rows, 7) == 127).all()
 
 
+def test_dynamic_quant_bf16_row_maximum_is_clamped():
+    """bf16 rows whose maximum would quantise to 128 (see the oracle test of the same name): the kernel
+    clamps, bit-exact with the oracle, max |q| >= 127, never a sign flip of a large activation."""
+    torch.manual_seed(3)
+    x = torch.randn(4096, 1024).bfloat16()
+    for j in range(42, 63):
+        x[j, :] = 0
+        x[j, 5] = 1.0 + j / 128.0
+        x[j, 6] = -0.5
+    xn = O.to_np(x)
+    q, s = flashnn_amd.DynamicQuantize()(x.to(DEV))
+    q_o, s_o = O.dynamic_quantize(xn, O.BF16)
+    assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.cpu().numpy(), s_o)
+    qn = q.cpu().numpy()
+    big = np.abs(xn) > s_o.astype(np.float32)[:, None]
+    assert (np.sign(qn[big]) == np.sign(xn[big])).all()
+    assert (qn[42:63, 5] == 127).all()
+    # the strided (non-vector) kernel: K not a multiple of 8
+    x2 = x[:64, :1021].contiguous()
+    q2, s2 = flashnn_amd.DynamicQuantize()(x2.to(DEV))
+    q2_o, s2_o = O.dynamic_quantize(O.to_np(x2), O.BF16)
+    assert np.array_equal(q2.cpu().numpy(), q2_o) and np.array_equal(s2.cpu().numpy(), s2_o)
+
+
 # -------------------------------------------------------------------- rmsnorm + quant
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(4, 128), (3, 32, 1024), (32, 8192), (7, 1000), (2, 20480), (3, 35584),
@@ -287,6 +311,93 @@ def test_a8w8_reference_sweep_shapes(nk, M):
     assert torch.equal(acc.sum(dim=1, dtype=torch.int64), (a.to(torch.int64) * colsum).sum(dim=1))
 
 
+@pytest.mark.parametrize("side", ["activations", "weights"])
+def test_a8w8_operand_of_2_gib_and_more(side):
+    """An operand whose last rows lie 2^31 bytes and more behind its first (a long prefill; a very wide
+    head) runs on the tiled MFMA kernel in bands, not on the any-shape kernel: the rows beyond the limit
+    equal, bit for bit, a call on those rows alone, both checksum identities hold over every accumulator,
+    and the scaled output of the far rows equals the oracle's epilogue."""
+    K, small = 8192, 384
+    big = (1 << 31) // K + 300                      # rows 262144.. start beyond 2^31 bytes
+    g = torch.Generator(device=DEV).manual_seed(77)
+    far = torch.randint(-128, 128, (big, K), dtype=torch.int8, device=DEV, generator=g)
+    near = torch.randint(-128, 128, (small, K), dtype=torch.int8, device=DEV, generator=g)
+    a, b = (far, near) if side == "activations" else (near, far)
+    acc = launchers.hip_gemm_a8w8_int32(a, b)
+    assert _lib.last_kernel().startswith("gemm_a8w8_ring_kernel")
+    tail = slice(big - 812, big)
+    if side == "activations":
+        assert torch.equal(acc[tail], launchers.hip_gemm_a8w8_int32(a[tail].contiguous(), b))
+    else:
+        assert torch.equal(acc[:, tail], launchers.hip_gemm_a8w8_int32(a, b[tail].contiguous()))
+    colsum = b.sum(dim=0, dtype=torch.int64)
+    rowsum = a.sum(dim=0, dtype=torch.int64)
+    assert torch.equal(acc.sum(dim=1, dtype=torch.int64), (a.to(torch.int64) * colsum).sum(dim=1))
+    assert torch.equal(acc.sum(dim=0, dtype=torch.int64), (b.to(torch.int64) * rowsum).sum(dim=1))
+    M, N = a.shape[0], b.shape[0]
+    ar = (torch.rand(M, device=DEV, generator=g) * 1e-2 + 1e-3).half()
+    ac = (torch.rand(N, device=DEV, generator=g) * 1e-2 + 1e-3).float()
+    out = flashnn_amd.GemmA8W8(torch.bfloat16)(a, b, ar, ac)
+    ri = torch.arange(big - 5, big, device=DEV) if side == "activations" else torch.arange(0, 5, device=DEV)
+    ci = torch.arange(0, 7, device=DEV) if side == "activations" else torch.arange(big - 7, big, device=DEV)
+    want = O.gemm_a8w8_epilogue_fp32(acc[ri][:, ci].cpu().numpy(), O.to_np(ar[ri].cpu()), ac[ci].cpu().numpy(), O.BF16)
+    assert np.array_equal(out[ri][:, ci].float().cpu().numpy(), want)
+
+
+def test_foreign_hip_error_is_left_alone(hip_lib):
+    """An error the caller's own HIP calls left on the thread is neither reported by a library call as its
+    own nor cleared by it."""
+    import ctypes
+    path = next(line.split()[-1] for line in open("/proc/self/maps") if "libamdhip64" in line)
+    hip = ctypes.CDLL(path)
+    x = torch.randn(8, 256, device=DEV).half()
+    q = torch.empty(8, 256, dtype=torch.int8, device=DEV)
+    s = torch.empty(8, dtype=torch.float16, device=DEV)
+    torch.cuda.synchronize()
+    assert hip.hipGetLastError() == 0
+    bad = hip.hipSetDevice(12345)                      # fails without touching the GPU
+    assert bad != 0 and hip.hipPeekAtLastError() == bad
+    rc = hip_lib.fnn_dynamic_quant(q.data_ptr(), s.data_ptr(), x.data_ptr(), 8, 256, 256, 256, 0,
+                                   _lib.current_stream(x.device))
+    assert rc == 0
+    assert hip.hipGetLastError() == bad                 # still there; now taken off the thread
+    assert hip.hipGetLastError() == 0
+    torch.cuda.synchronize()
+    q_o, s_o = O.dynamic_quantize(O.to_np(x.cpu()), O.F16)
+    assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.cpu().numpy(), s_o)
+
+
+def test_first_use_log_and_kernel_names():
+    """FLASHNN_HIP_LOG=1: one line on stderr per kernel variant, the first time it is launched; and
+    fnn_last_kernel() names what the last call ran."""
+    import os
+    import subprocess
+    prog = (
+        "import torch, flashnn_amd\n"
+        "from flashnn_amd import _lib\n"
+        "x = torch.randn(64, 1024, device='cuda:0').half()\n"
+        "op = flashnn_amd.DynamicQuantize()\n"
+        "q, s = op(x); q, s = op(x)\n"
+        "print(_lib.last_kernel())\n"
+        "w = torch.randint(-128, 128, (256, 1024), dtype=torch.int8, device='cuda:0')\n"
+        "flashnn_amd.GemmA8W8()(q, w, s, torch.ones(256, device='cuda:0').half())\n"
+        "print(_lib.last_kernel())\n"
+        "torch.cuda.synchronize()\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, FLASHNN_HIP_LOG="1", PYTHONPATH=root)
+    r = subprocess.run([sys.executable, "-c", prog], env=env, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr
+    lines = [l for l in r.stderr.splitlines() if l.startswith("[flashnn_hip]")]
+    assert lines[0] == "[flashnn_hip] first launch of dynamic_quant_vec_kernel<1,0,0>"
+    assert len(lines) == 2 and len(set(lines)) == 2
+    names = r.stdout.split()
+    assert names[0] == "dynamic_quant_vec_kernel<1,0,0>" and names[1] in lines[1]
+    # without the variable nothing is printed
+    env.pop("FLASHNN_HIP_LOG")
+    r = subprocess.run([sys.executable, "-c", prog], env=env, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and "[flashnn_hip]" not in r.stderr
+
+
 def test_a8w8_tuned_config_cache(tmp_path, monkeypatch):
     """With tuning on, the first launch of a shape times the candidate tiles and records the best under
     the reference's method name; the next launch (and a fresh reader of the file) uses the record; the
@@ -295,6 +406,7 @@ def test_a8w8_tuned_config_cache(tmp_path, monkeypatch):
     from flashnn_amd import tuned_configs as TC
     path = tmp_path / "best.json"
     monkeypatch.setenv("FLASHNN_AMD_TUNED_CONFIGS", str(path))
+    TC.CACHE.reset()                    # the process-wide cache reads the environment once
     M, N, K = 300, 520, 1024
     a, b = _rand_i8((M, K), 31), _rand_i8((N, K), 32)
     g = torch.Generator().manual_seed(33)
@@ -314,6 +426,9 @@ def test_a8w8_tuned_config_cache(tmp_path, monkeypatch):
     again = op(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV)).cpu()     # from the record, tuning off
     assert torch.equal(plain, tuned) and torch.equal(plain, again)
     assert TC.TunedConfigs().lookup(f"gemm_a8w8_{M}_{N}_{K}") == tile
+    assert TC.CACHE.shape_tile("gemm_a8w8", M, N, K) == tile
+    monkeypatch.undo()
+    TC.CACHE.reset()
     want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.numpy(), b.numpy()), O.to_np(ar), O.to_np(ac), O.F16)
     assert np.array_equal(plain.float().numpy(), want)
 
@@ -653,6 +768,17 @@ def test_weight_only_gemv_equal_chunks(bits, M, N, K):
         assert (np.abs(got[:, band] - exact) <= np.abs(exact) * ulp + 2e-3 * spread).all()
 
 
+@pytest.mark.parametrize("bits,M,N,K,group", [(4, 1, 4096, 16384, 128), (4, 3, 2048, 16384, 128), (8, 1, 1024, 16384, 128),
+                                              (8, 2, 1024, 16384, 0), (4, 8, 2048, 14336, 128)])
+def test_weight_only_long_rows_within_the_lds_limit(bits, M, N, K, group):
+    """Decode shapes whose staged activations would push a launch past 64 KB of dynamic LDS: the call succeeds
+    (the dispatch passes such a shape to a kernel that fits or raises that kernel's limit first) and the
+    result is right."""
+    act, w, qw, scale, zp, bias = _wo_inputs(M, N, K, group, bits, torch.float16, torch.float16, True, False, 93)
+    _wo_check(act, w, qw, scale, zp, bias, group, bits, torch.float16)
+    assert _lib.last_kernel().startswith("gemm_wo_")
+
+
 # ------------------------------------------------------- rmsnorm+quant -> A8W8 chain
 @pytest.mark.parametrize("M", [1, 32, 512, 8192])
 def test_rmsnorm_quant_gemm_chain(M):
@@ -667,8 +793,15 @@ def test_rmsnorm_quant_gemm_chain(M):
     q_o, s_o = O.rmsnorm_dquant(O.to_np(h), gamma.numpy(), 1e-6, O.BF16)
     assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.float().cpu().numpy(), s_o)
     rows = np.unique(np.linspace(0, M - 1, min(M, 24)).astype(int))
-    acc = launchers.hip_gemm_a8w8_int32(q, w.to(DEV))[torch.from_numpy(rows).to(DEV)].cpu().numpy()
+    acc_all = launchers.hip_gemm_a8w8_int32(q, w.to(DEV))
+    acc = acc_all[torch.from_numpy(rows).to(DEV)].cpu().numpy()
     assert np.array_equal(acc, O.gemm_a8w8_acc(q_o[rows], w.numpy()))
+    # every accumulator, through sum_n acc[m, n] = q[m, :] . sum_n w[n, :] in exact integers
+    colsum = w.numpy().astype(np.int64).sum(axis=0)
+    assert np.array_equal(acc_all.sum(dim=1, dtype=torch.int64).cpu().numpy(), q_o.astype(np.int64) @ colsum)
+    # ... and sum_m acc[m, n] = (sum_m q[m, :]) . w[n, :]
+    rowsum = torch.from_numpy(q_o.astype(np.int64).sum(axis=0)).to(DEV)
+    assert torch.equal(acc_all.sum(dim=0, dtype=torch.int64), (w.to(DEV).to(torch.int64) * rowsum).sum(dim=1))
     want = O.gemm_a8w8(q_o[rows], w.numpy(), s_o[rows], ws.numpy(), O.BF16)
     np.testing.assert_allclose(out[torch.from_numpy(rows).to(DEV)].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
 

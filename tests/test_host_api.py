@@ -168,6 +168,14 @@ def test_tuned_config_file_format_and_lookup(tmp_path, monkeypatch):
     assert other.lookup("gemm_a8w8_2048_12288_4096") is None and other.lookup("gemm_a8w8_16_4096_4096") == (0, 0, 0)
     other.record("gemm_a8w8_2048_12288_4096", (256, 128, 0))
     assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 128, 0)
+    # the per-shape answer a launcher uses: resolved once, dropped by a new record or reset()
+    assert other.shape_tile("gemm_a8w8", 16, 4096, 4096) == (0, 0, 0) and other.shape_tile("gemm_a8w8", 1, 1, 1) is None
+    other.record("gemm_a8w8_1_1_1", (64, 128, 0))
+    assert other.shape_tile("gemm_a8w8", 1, 1, 1) == (64, 128, 0)
+    os.remove(path)
+    assert other.shape_tile("gemm_a8w8", 1, 1, 1) == (64, 128, 0)       # answered without touching the file
+    other.reset()
+    assert other.shape_tile("gemm_a8w8", 1, 1, 1) is None
     assert TC.serialize_best_config((128, 128)) == [{"BLOCK_M": 128, "BLOCK_N": 128}, {}]
     assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 192}, {}]) == (256, 192, 0)
     assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 256}, {"num_warps": 8}]) == (256, 256, 8)

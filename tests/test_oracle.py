@@ -37,9 +37,48 @@ def test_dynamic_quantize_matches_torch_ops(dtype, shape):
     for x in (torch.rand(shape) * 2 - 1, torch.randn(shape)):
         x = x.to(dtype)
         q_t, s_t = T.dynamic_quantize(x)
-        q_o, s_o = O.dynamic_quantize(O.to_np(x), O.tag_of(x))
+        q_o, s_o = O.dynamic_quantize(O.to_np(x), O.tag_of(x), clamp=False)   # the literal torch formula
         assert np.array_equal(q_o, q_t.numpy())
         assert np.array_equal(s_o, s_t.numpy())
+        # the clamped form (the default, and what the kernels compute) differs only where that formula
+        # reaches 128 and wraps
+        q_c, s_c = O.dynamic_quantize(O.to_np(x), O.tag_of(x))
+        assert np.array_equal(s_c, s_o)
+        diff = q_c != q_o
+        assert (q_o[diff] == -128).all() and (q_c[diff] == 127).all() and (O.to_np(x)[diff] > 0).all()
+        if dtype == torch.float16:
+            assert not diff.any()
+
+
+def test_dynamic_quantize_bf16_row_maximum_is_clamped():
+    """bf16 rows whose maximum has a mantissa that makes RN(max / 127) round down: max / scale rounds to
+    127.5 and on to 128, which an unclamped conversion to int8 wraps to -128 - the sign of the row's largest
+    activation.  The oracle (and the kernels) clamp: max |q| = 127 and sign(q) = sign(x) on every row."""
+    torch.manual_seed(3)
+    x = torch.randn(4096, 1024).bfloat16()
+    xn = O.to_np(x)
+    q_raw, _ = O.dynamic_quantize(xn, O.BF16, clamp=False)
+    q, s = O.dynamic_quantize(xn, O.BF16)
+    flipped = ((q_raw == -128) & (xn > 0)).any(axis=1)
+    assert 0.005 < flipped.mean() < 0.05            # a visible fraction of rows is affected without the clamp
+    # +127 is the largest value; -128 remains reachable for a negative row maximum (no wrap there); a scale
+    # that rounded up leaves the maximum at 126.5, which rounds to 126
+    assert (q.astype(np.int32).max(axis=1) <= 127).all() and (np.abs(q.astype(np.int32)).max(axis=1) >= 126).all()
+    s32 = s.astype(np.float32)[:, None]
+    big = np.abs(xn) > s32
+    assert (np.sign(q[big]) == np.sign(xn[big])).all()
+    assert not (np.sign(q_raw[big]) == np.sign(xn[big])).all()
+    # hand-made rows: maximum 1 + j/128 for j in [42, 62] (the mantissas the rounding hits)
+    hits = 0
+    for j in range(42, 63):
+        row = np.zeros((1, 64), np.float32)
+        row[0, 0] = 1.0 + j / 128.0
+        row[0, 1] = -0.5
+        qr, _ = O.dynamic_quantize(row, O.BF16, clamp=False)
+        qc, _ = O.dynamic_quantize(row, O.BF16)
+        hits += int(qr[0, 0] == -128)
+        assert qc[0, 0] == 127 and qc[0, 1] < 0
+    assert hits > 0
 
 
 def test_dynamic_quantize_bruteforce_f16():
