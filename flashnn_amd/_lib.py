@@ -11,7 +11,7 @@ FNN_F16, FNN_BF16, FNN_F32 = 0, 1, 2
 _DTYPE_CODE = {torch.float16: FNN_F16, torch.bfloat16: FNN_BF16, torch.float32: FNN_F32}
 FNN_I8 = 3   # accepted for the zero points of fnn_fused_moe_a16w4 only
 
-_i64, _int, _ptr, _f32 = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_float
+_i64, _int, _ptr, _f32, _size = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_float, ctypes.c_size_t
 
 # name -> argument types; every function returns int unless listed in _RESTYPE
 _SIGNATURES = {
@@ -25,6 +25,10 @@ _SIGNATURES = {
     "fnn_layernorm_dquant": [_ptr, _ptr, _ptr, _ptr, _ptr, _f32, _i64, _i64, _i64, _i64, _int, _int, _ptr],
     "fnn_gemm_a8w8": [_ptr] * 5 + [_i64] * 6 + [_int] * 3 + [_ptr],
     "fnn_gemm_a8w8_tiled": [_ptr] * 5 + [_i64] * 6 + [_int] * 6 + [_ptr],
+    "fnn_gemm_a8w8_workspace_bytes": [_i64] * 3,
+    "fnn_workspace_init": [_ptr, _size, _ptr],
+    "fnn_gemm_a8w8_ws": [_ptr] * 5 + [_i64] * 6 + [_int] * 3 + [_ptr, _size, _ptr],
+    "fnn_gemm_a8w8_ws_tiled": [_ptr] * 5 + [_i64] * 6 + [_int] * 6 + [_ptr, _size, _ptr],
     "fnn_gemm_a8w8_i32": [_ptr] * 3 + [_i64] * 6 + [_ptr],
     "fnn_gemm_a8w8_i32_tiled": [_ptr] * 3 + [_i64] * 6 + [_int] * 3 + [_ptr],
     "fnn_gemm_a16w8": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],
@@ -32,7 +36,8 @@ _SIGNATURES = {
     "fnn_fused_moe_a8w8": [_ptr] * 9 + [_i64] * 9 + [_int] * 7 + [_ptr],
     "fnn_fused_moe_a16w4": [_ptr] * 9 + [_i64] * 14 + [_int] * 8 + [_ptr],
 }
-_RESTYPE = {"fnn_last_error": ctypes.c_char_p, "fnn_last_kernel": ctypes.c_char_p}
+_RESTYPE = {"fnn_last_error": ctypes.c_char_p, "fnn_last_kernel": ctypes.c_char_p,
+            "fnn_gemm_a8w8_workspace_bytes": ctypes.c_size_t}
 
 _lib = None
 

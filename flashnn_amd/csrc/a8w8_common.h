@@ -18,6 +18,10 @@ struct A8W8Args {
     int64_t lda, ldb, ldc;
     int out_dtype, arow_dtype, acol_dtype;
     int tiles_m, tiles_n, tiles_per_xcd;
+    // K cut into kparts ranges of k_chunk bytes per row (the tiled kernel's split form only)
+    int kparts, k_chunk;
+    int* ws_count;          // one ticket counter per tile, zero between calls
+    int32_t* ws_part;       // kparts slots of tile-rows x tile-columns accumulators per tile
 };
 
 // gemm_a8w8_skinny.hip: up to 64 activation rows, the weights streamed once; false if the shape

@@ -67,7 +67,17 @@ struct OptionalStage<false, BYTES> {
     static __device__ __forceinline__ char* get() { return nullptr; }
 };
 
-template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2>
+// SPLIT: the workgroups of the grid are units, kparts per tile, each the tile's product over its own range
+// of K (k_chunk bytes per row, a multiple of the slab; the last part takes the rest).  A unit that is done
+// counts itself arrived at the tile's counter.  If it is the last to arrive and finds every other unit's
+// accumulators complete in the workspace, it adds them to its registers and goes on to the ordinary
+// epilogue.  Otherwise it stores its accumulators, as they lie in registers, in its slot, counts the slot
+// complete, and leaves - unless that was the last of all kparts slots: then it is the one that adds up the
+// others.  Exactly one unit per tile does, whatever the order; every slot it reads was complete before the
+// count that chose it; nobody waits for anybody.  Integer sums do not depend on the order, so the result is
+// the unsplit kernel's bit for bit.  The unit that adds up sets the counter back to zero: the counters are
+// zero whenever no call is in flight.
+template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2, bool SPLIT = false>
 __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Args p) {
     // WGM x 2 waves.  WGM = 4 puts two waves on every SIMD (at most 256 registers each): one can issue
     // MFMAs while the other waits for LDS fragments, a copy or the barrier.
@@ -106,8 +116,15 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
     float* const sc_col = sc_row + BM;
 
     const int xcd = blockIdx.x & 7;
-    const int t = xcd * p.tiles_per_xcd + (blockIdx.x >> 3);
-    if ((blockIdx.x >> 3) >= p.tiles_per_xcd || t >= p.tiles_m * p.tiles_n) return;
+    const int unit = xcd * p.tiles_per_xcd + (blockIdx.x >> 3);   // (tiles_per_xcd counts units where SPLIT)
+    if ((blockIdx.x >> 3) >= p.tiles_per_xcd || unit >= p.tiles_m * p.tiles_n * (SPLIT ? p.kparts : 1)) return;
+    // the units of a tile are neighbours in this numbering: they run on one XCD, at about the same time
+    const int t = SPLIT ? unit / p.kparts : unit;
+    const int kpart = SPLIT ? unit - t * p.kparts : 0;
+    const int8_t* const pa = SPLIT ? p.a + (int64_t)kpart * p.k_chunk : p.a;
+    const int8_t* const pb = SPLIT ? p.b + (int64_t)kpart * p.k_chunk : p.b;
+    // (the last part takes what the others leave: a few slabs more, so that it arrives last as a rule)
+    const int Kl = SPLIT ? (kpart == p.kparts - 1 ? p.K - kpart * p.k_chunk : p.k_chunk) : p.K;
     // tiles are numbered in groups of GN tile columns, the column fastest within a group: the 32 workgroups
     // an XCD runs at a time then cover 8 tile rows x 4 tile columns whatever M is, and fetch
     // 8*BM + 4*BN operand rows per slab into its L2 instead of tiles_m*BM + BN
@@ -168,7 +185,7 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
         return (const char*)(((uint64_t)hi << 32) | lo);
     };
     auto copy_a_part = [&](char* stage, int kt, int part, int fix = 0) {
-        const char* slab = slab_base(p.a, kt);
+        const char* slab = slab_base(pa, kt);
 #pragma unroll
         for (int j = 0; j < NLA; ++j)
             if (j * 3 / NLA == part)
@@ -181,14 +198,14 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
         copy_a_part(stage, kt, 2, fix);
     };
     auto copy_b = [&](char* stage, int kt) {
-        const char* slab = slab_base(p.b, kt); const int fix = 0;
+        const char* slab = slab_base(pb, kt); const int fix = 0;
 #pragma unroll
         for (int j = 0; j < NLB; ++j)
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(slab + (uint32_t)(gob[j] + fix)),
                                              (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
     auto copy_a_half = [&](char* stage, int kt, int half, int fix = 0) {
-        const char* slab = slab_base(p.a, kt);
+        const char* slab = slab_base(pa, kt);
 #pragma unroll
         for (int j = 0; j < NLA; ++j)
             if (j * 2 / NLA == half)
@@ -196,7 +213,7 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
                                                  (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
     auto copy_b_half = [&](char* stage, int kt, int half, int fix = 0) {
-        const char* slab = slab_base(p.b, kt);
+        const char* slab = slab_base(pb, kt);
 #pragma unroll
         for (int j = 0; j < NLB; ++j)
             if (j * 2 / NLB == half)
@@ -204,7 +221,7 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
                                                  (lds_ptr_t)(stage + (j * NWAVES + wave) * (8 * BK)), 16, 0, 0);
     };
     auto copy_b_part = [&](char* stage, int kt, int part, int fix = 0) {
-        const char* slab = slab_base(p.b, kt);
+        const char* slab = slab_base(pb, kt);
 #pragma unroll
         for (int j = 0; j < NLB; ++j)
             if (j * 3 / NLB == part)
@@ -298,8 +315,8 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
     };
 
     // K = 128 * (KT - 1) + 32 * last_steps: the last slab may hold fewer than 128 bytes per row
-    const int KT = (p.K + BK - 1) / BK;
-    const int last_steps = (p.K - (KT - 1) * BK) / 32;
+    const int KT = (Kl + BK - 1) / BK;
+    const int last_steps = (Kl - (KT - 1) * BK) / 32;
     const int tail_fix = lchunk * 16 >= last_steps * 32 ? -(lchunk * 16) : 0;
     // The last slab, in stages (ca, cb), after its barrier; chunk 1 of the slab before it is in registers.
     // Where K ends in the middle of a 64-byte chunk, the lanes that hold its second half feed zeros
@@ -432,6 +449,59 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
         last_iter(ls == 0 ? sa0 : ls == 1 ? sa1 : sa2, ls == 0 ? sb0 : ls == 1 ? sb1 : sb2);
     }
 #undef FNN_PHASE
+
+    if constexpr (SPLIT) {
+        // This unit's accumulators into its slot, in register order: value (i, j) of lane L at 16-byte word
+        // (i * FM + j) * NT + L of the slot.  The slots are written and read with device-scope accesses
+        // (they pass through L2 to where every XCD sees them), 8 bytes at a time.  A device-scope fence
+        // would do for plain stores, but it writes back (release) and invalidates (acquire) the XCD's whole
+        // L2, under the other workgroups' operand traffic: the split kernel then ran at half the speed of
+        // the unsplit one.
+        typedef unsigned long long u64;
+        u64* const slots = (u64*)p.ws_part + (int64_t)t * p.kparts * (BM * BN / 2);
+        // The tile's counter holds arrivals in its low half and completed slots in its high half.
+        int* const word = (int*)sb2 + BM + BN;      // behind the scales' place in the third b-stage
+        __syncthreads();                    // every wave has left the main loop: the stages are free
+        if (threadIdx.x == 0)
+            *word = __hip_atomic_fetch_add(p.ws_count + t, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        const int seen = *word;
+        // the last unit to arrive that finds every other slot complete adds them up without storing its own
+        if (!((seen & 0xffff) == p.kparts - 1 && (seen >> 16) == p.kparts - 1)) {
+            u64* const mine = slots + (int64_t)kpart * (BM * BN / 2) + 2 * threadIdx.x;
+#pragma unroll
+            for (int i = 0; i < FN; ++i)
+#pragma unroll
+                for (int j = 0; j < FM; ++j) {
+                    const v4i v = acc[i][j];
+                    u64* const w = mine + (i * FM + j) * (2 * NT);
+                    __hip_atomic_store(w, (u64)(uint32_t)v[0] | ((u64)(uint32_t)v[1] << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(w + 1, (u64)(uint32_t)v[2] | ((u64)(uint32_t)v[3] << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            // every wave waits until its stores have been acknowledged, then one lane counts the slot complete
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+            if (threadIdx.x == 0)
+                *word = __hip_atomic_fetch_add(p.ws_count + t, 0x10000, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            // whoever completes the last of all kparts slots adds up the others; otherwise this unit is done
+            if ((*word >> 16) != p.kparts - 1) return;
+        }
+        for (int q = 0; q < p.kparts; ++q) {
+            if (q == kpart) continue;
+            const u64* const theirs = slots + (int64_t)q * (BM * BN / 2) + 2 * threadIdx.x;
+#pragma unroll
+            for (int i = 0; i < FN; ++i)
+#pragma unroll
+                for (int j = 0; j < FM; ++j) {
+                    const u64* const w = theirs + (i * FM + j) * (2 * NT);
+                    const u64 lo = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const u64 hi = __hip_atomic_load(w + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    acc[i][j] += v4i{(int)(uint32_t)lo, (int)(uint32_t)(lo >> 32), (int)(uint32_t)hi, (int)(uint32_t)(hi >> 32)};
+                }
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(p.ws_count + t, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 
     // ---- epilogue ----
     // acc[i][j][r]: n = wn0 + i*16 + 4*(lane>>4) + r,  m = wm0 + j*16 + (lane&15).
@@ -671,6 +741,17 @@ static void launch_mfma(A8W8Args& p, hipStream_t st) {
     gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, WGM><<<dim3(p.tiles_per_xcd * 8), dim3(WGM * 128), 0, st>>>(p);
 }
 
+// The same tiles with K cut into p.kparts ranges (p.kparts, p.k_chunk, p.ws_count, p.ws_part set by the caller).
+template <int BM, int BN, int MODE, bool PAIR = false>
+static void launch_mfma_split(A8W8Args& p, hipStream_t st) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int units = p.tiles_m * p.tiles_n * p.kparts;
+    p.tiles_per_xcd = (units + 7) / 8;
+    note_kernel("gemm_a8w8_ring_kernel(split K)", BM, BN, p.kparts);
+    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, 2, true><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p);
+}
+
 // The tiles that exist: (rows, columns, waves per workgroup).
 static bool valid_tile(int bm, int bn, int waves) {
     if (bm == 0 && bn == 0) return waves == 0;
@@ -694,13 +775,87 @@ static void launch_tile(A8W8Args& p, hipStream_t st, int bm, int bn, int waves) 
     else launch_mfma<128, 128, MODE>(p, st);
 }
 
-// One launch plan for operands whose row offsets fit 32 bits (M * lda and N * ldb below 2^31 bytes).
+// ---- K split over several workgroups per tile (needs a workspace) ----
+// Workspace: kWsCounters ticket counters (zero between calls), then per tile kparts slots of tile-rows x
+// tile-columns accumulators.
+constexpr int kWsCounters = 1024;
+constexpr size_t kWsHeader = kWsCounters * sizeof(int);
+
+struct SplitPlan { int bm, bn, kparts, k_chunk; double us; };
+
+// Slabs per part: the last part gets kStagger slabs more than the others (and the remainder), so that the
+// others have stored their accumulators by the time it arrives and it can add them up at once.
+constexpr int kStagger = 4;
+static int split_chunk_slabs(int KT, int parts) { return (KT - kStagger) / parts; }
+
+static size_t split_ws_bytes(const SplitPlan& s, int64_t M, int64_t N) {
+    const int64_t tiles = ((M + s.bm - 1) / s.bm) * ((N + s.bn - 1) / s.bn);
+    return kWsHeader + (size_t)tiles * s.kparts * s.bm * s.bn * sizeof(int32_t);
+}
+
+// Whether to split K for this shape, and how.  Measured (bf16 out, microseconds, unsplit -> split): the split
+// pays where the unsplit kernel's tiles fill at most three quarters of the CUs and K is 8192 or more (the
+// unsplit kernel's time on such shapes follows K alone, about 0.42 us per slab whatever M and N: a
+// workgroup's chain of slabs is bound by the latency of the weights from HBM, and the split shortens it):
+//   M = 256  N = 4096 K = 8192   30.3 -> 26.2 (3 parts)     M = 128 N = 8192 K = 8192   33.3 -> 29.2 (3 parts)
+//   M = 768  N = 2048 K = 16384  53.0 -> 45.3 (2 parts)     M = 128 N = 2048 K = 16384  54.9 -> 31.2 (8 parts)
+//   M = 384  N = 1920 K = 13312  46.6 -> 31.2 (4 parts)     M = 512 N = 1024 K = 8192   28.6 -> 27.4 (7 parts)
+// and costs where they fill them anyway (M = 512 N = K = 8192: 44.5 -> 51.5; M = 2048 N = 1024 K = 8192:
+// 23.6 -> 28.7).  The tile is 128x128 in pairs of workgroups per CU: with M this small the weights stream
+// from HBM, and two workgroups per CU keep twice the bytes in flight; the 256-row tiles were slower split
+// than the small tiles unsplit.  About 224 units (seven eighths of one per CU, a pair never on one CU) was
+// the best count; a part holds at least 8 slabs.
+static SplitPlan plan_split(int64_t M, int64_t N, int64_t K, size_t ws_bytes) {
+    const int KT = (int)((K + 127) / 128);
+    const TileChoice u = choose_tile(M, N);
+    SplitPlan none{u.bm, u.bn, 1, 0, 0.0};
+    const int64_t utiles = ((M + u.bm - 1) / u.bm) * ((N + u.bn - 1) / u.bn);
+    if (KT < 64 || utiles > 192) return none;      // (K = 4096: 0.70 to 0.95 of the unsplit speed; K = 6144: 0.91 to 1.10)
+    const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
+    int parts = (int)(224 / t128);
+    if (parts > 8) parts = 8;
+    while (parts >= 2 && split_chunk_slabs(KT, parts) < 8) --parts;
+    if (parts < 2) return none;
+    const SplitPlan s{128, 128, parts, split_chunk_slabs(KT, parts) * 128, 0.0};
+    if (ws_bytes != 0 && split_ws_bytes(s, M, N) > ws_bytes) return none;
+    return s;
+}
+
 template <int MODE>
-static void dispatch_band(A8W8Args& p, hipStream_t st, bool aligned, int force_bm, int force_bn, int force_waves) {
+static void launch_split(A8W8Args& p, hipStream_t st, const SplitPlan& s, void* workspace) {
+    p.kparts = s.kparts;
+    p.k_chunk = s.k_chunk;
+    p.ws_count = (int*)workspace;
+    p.ws_part = (int32_t*)((char*)workspace + kWsHeader);
+    if (s.bm == 128) launch_mfma_split<128, 128, MODE, true>(p, st);   // two workgroups per CU
+    else if (s.bn == 192) launch_mfma_split<256, 192, MODE>(p, st);
+    else launch_mfma_split<256, 128, MODE>(p, st);
+}
+
+// One launch plan for operands whose row offsets fit 32 bits (M * lda and N * ldb below 2^31 bytes).
+struct Workspace { void* ptr; size_t bytes; int force_kparts; };
+
+template <int MODE>
+static void dispatch_band(A8W8Args& p, hipStream_t st, bool aligned, int force_bm, int force_bn, int force_waves,
+                          const Workspace& ws = Workspace{nullptr, 0, 0}) {
     // the MFMA kernel walks K in slabs of 128 bytes
     const bool fast = aligned && p.K % 32 == 0 && p.K >= 512;
     // few activation rows: stream the weights once (unless the caller names a tile of the tiled kernel)
     if (force_bm == 0 && p.M <= 64 && launch_a8w8_skinny(p, MODE, st)) return;
+    if (fast && ws.ptr) {
+        if (ws.force_kparts > 1) {          // (the entry point has checked tile, parts and workspace size)
+            const int chunk = split_chunk_slabs((p.K + 127) / 128, ws.force_kparts) * 128;
+            launch_split<MODE>(p, st, SplitPlan{force_bm, force_bn, ws.force_kparts, chunk, 0.0}, ws.ptr);
+            return;
+        }
+        if (force_bm == 0 && ws.force_kparts == 0) {
+            const SplitPlan s = plan_split(p.M, p.N, p.K, ws.bytes);
+            if (s.kparts > 1) {
+                launch_split<MODE>(p, st, s, ws.ptr);
+                return;
+            }
+        }
+    }
     if (!fast) {
         note_kernel("gemm_a8w8_any_kernel");
         gemm_a8w8_any_kernel<MODE><<<dim3((p.N + 63) / 64, (p.M + 63) / 64), dim3(256), 0, st>>>(p);
@@ -729,13 +884,14 @@ static void dispatch_band(A8W8Args& p, hipStream_t st, bool aligned, int force_b
 // N * ldb of 2^31 bytes and more: a long prefill, a very wide head) are cut on the host into bands of rows
 // and of columns that fit, each band a problem of its own on the same kernels.
 template <int MODE>
-static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn, int force_waves) {
+static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn, int force_waves,
+                     const Workspace& ws = Workspace{nullptr, 0, 0}) {
     const bool aligned = p.lda % 16 == 0 && p.ldb % 16 == 0 && ((uintptr_t)p.a % 16) == 0 &&
                          ((uintptr_t)p.b % 16) == 0 && ((uintptr_t)p.out % 16) == 0;
     constexpr int64_t kLimit = (1LL << 31) - 1;
     const int64_t m_fit = kLimit / p.lda, n_fit = kLimit / p.ldb;
     if (p.M <= m_fit && p.N <= n_fit) {
-        dispatch_band<MODE>(p, st, aligned, force_bm, force_bn, force_waves);
+        dispatch_band<MODE>(p, st, aligned, force_bm, force_bn, force_waves, ws);
         return;
     }
     // bands in whole tiles of every shape (rows: 256; columns: 768 = lcm(256, 192, 128)), so that the bands
@@ -772,7 +928,7 @@ using namespace fnn;
 static int gemm_a8w8_entry(const char* fn, void* out, const void* a, const void* b, const void* alpha_row,
                            const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                            int64_t ldc, int out_dtype, int alpha_row_dtype, int alpha_col_dtype, int tile_m,
-                           int tile_n, int waves, void* stream) {
+                           int tile_n, int waves, void* stream, const Workspace& ws = Workspace{nullptr, 0, 0}) {
     int rc = check_args(fn, out, a, b, M, N, K, lda, ldb, ldc);
     if (rc != FNN_OK) return rc;
     if (M != 0 && N != 0 && (!alpha_row || !alpha_col)) { set_error("%s: null scale pointer", fn); return FNN_ERR_ARG; }
@@ -782,14 +938,42 @@ static int gemm_a8w8_entry(const char* fn, void* out, const void* a, const void*
         set_error("%s: no such tile %dx%d with %d waves", fn, tile_m, tile_n, waves);
         return FNN_ERR_ARG;
     }
+    if (ws.force_kparts < 0 || (ws.bytes > 0 && !ws.ptr)) {
+        set_error("%s: bad workspace or number of parts (%d)", fn, ws.force_kparts);
+        return FNN_ERR_ARG;
+    }
+    if (ws.ptr && (((uintptr_t)ws.ptr % 16) != 0 || ws.bytes < kWsHeader)) {
+        set_error("%s: the workspace must be 16-byte aligned and hold at least %zu bytes", fn, kWsHeader);
+        return FNN_ERR_ARG;
+    }
+    if (ws.force_kparts > 1) {
+        // a named split: one of the two large tiles, parts of at least 4 slabs, a workspace that holds it
+        const int KT = (int)((K + 127) / 128), chunk = split_chunk_slabs(KT, ws.force_kparts);
+        const SplitPlan s{tile_m, tile_n, ws.force_kparts, chunk * 128, 0.0};
+        const bool tile_ok = ((tile_m == 256 && (tile_n == 128 || tile_n == 192)) || (tile_m == 128 && tile_n == 128)) &&
+                             (waves == 0 || waves == 4);
+        const bool shape_ok = K % 32 == 0 && lda % 16 == 0 && ldb % 16 == 0 && ((uintptr_t)a % 16) == 0 &&
+                              ((uintptr_t)b % 16) == 0 && ((uintptr_t)out % 16) == 0 && M * lda < (1LL << 31) &&
+                              N * ldb < (1LL << 31);
+        if (!tile_ok || !shape_ok || chunk < 4 ||
+            ((M + tile_m - 1) / (tile_m ? tile_m : 1)) * ((N + tile_n - 1) / (tile_n ? tile_n : 1)) > kWsCounters) {
+            set_error("%s: K = %lld cannot be split %d ways on a %dx%d tile for these operands", fn, (long long)K,
+                      ws.force_kparts, tile_m, tile_n);
+            return FNN_ERR_ARG;
+        }
+        if (!ws.ptr || split_ws_bytes(s, M, N) > ws.bytes) {
+            set_error("%s: workspace of %zu bytes, the split needs %zu", fn, ws.bytes, split_ws_bytes(s, M, N));
+            return FNN_ERR_ARG;
+        }
+    }
     if (M == 0 || N == 0) return FNN_OK;
     A8W8Args p{};
     p.a = (const int8_t*)a; p.b = (const int8_t*)b; p.out = out; p.arow = alpha_row; p.acol = alpha_col;
     p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
     p.out_dtype = out_dtype; p.arow_dtype = alpha_row_dtype; p.acol_dtype = alpha_col_dtype;
     const Call call(fn);
-    if (out_dtype == FNN_F16) dispatch<OUT_F16>(p, (hipStream_t)stream, tile_m, tile_n, waves);
-    else dispatch<OUT_BF16>(p, (hipStream_t)stream, tile_m, tile_n, waves);
+    if (out_dtype == FNN_F16) dispatch<OUT_F16>(p, (hipStream_t)stream, tile_m, tile_n, waves, ws);
+    else dispatch<OUT_BF16>(p, (hipStream_t)stream, tile_m, tile_n, waves, ws);
     return call.done();
 }
 
@@ -825,6 +1009,49 @@ extern "C" int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, cons
                                    int alpha_col_dtype, int tile_m, int tile_n, int waves, void* stream) {
     return gemm_a8w8_entry("fnn_gemm_a8w8_tiled", out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc, out_dtype,
                            alpha_row_dtype, alpha_col_dtype, tile_m, tile_n, waves, stream);
+}
+
+extern "C" size_t fnn_gemm_a8w8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 64 || N <= 0 || K < 512 || K % 32 != 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return 0;
+    const SplitPlan s = plan_split(M, N, K, 0);
+    return s.kparts > 1 ? split_ws_bytes(s, M, N) : 0;
+}
+
+namespace fnn {
+__global__ __launch_bounds__(256) void clear_words_kernel(int* w, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) w[i] = 0;
+}
+}  // namespace fnn
+
+extern "C" int fnn_workspace_init(void* workspace, size_t ws_bytes, void* stream) {
+    const char* fn = "fnn_workspace_init";
+    if (!workspace || ((uintptr_t)workspace % 16) != 0 || ws_bytes < kWsHeader) {
+        set_error("%s: the workspace must be 16-byte aligned and hold at least %zu bytes", fn, kWsHeader);
+        return FNN_ERR_ARG;
+    }
+    const Call call(fn);
+    note_kernel("clear_words_kernel");
+    clear_words_kernel<<<dim3(kWsCounters / 256), dim3(256), 0, (hipStream_t)stream>>>((int*)workspace, kWsCounters);
+    return call.done();
+}
+
+extern "C" int fnn_gemm_a8w8_ws(void* out, const void* a, const void* b, const void* alpha_row,
+                                const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
+                                int alpha_col_dtype, void* workspace, size_t ws_bytes, void* stream) {
+    return gemm_a8w8_entry("fnn_gemm_a8w8_ws", out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc, out_dtype,
+                           alpha_row_dtype, alpha_col_dtype, 0, 0, 0, stream, Workspace{workspace, ws_bytes, 0});
+}
+
+extern "C" int fnn_gemm_a8w8_ws_tiled(void* out, const void* a, const void* b, const void* alpha_row,
+                                      const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                      int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
+                                      int alpha_col_dtype, int tile_m, int tile_n, int kparts, void* workspace,
+                                      size_t ws_bytes, void* stream) {
+    return gemm_a8w8_entry("fnn_gemm_a8w8_ws_tiled", out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc,
+                           out_dtype, alpha_row_dtype, alpha_col_dtype, tile_m, tile_n, 0, stream,
+                           Workspace{workspace, ws_bytes, kparts == 1 ? 0 : kparts});
 }
 
 extern "C" int fnn_gemm_a8w8_i32(int32_t* acc, const void* a, const void* b, int64_t M, int64_t N,

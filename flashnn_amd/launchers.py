@@ -120,6 +120,27 @@ def _flat_scale(t, n, what):
     return t if t.is_contiguous() else t.contiguous()
 
 
+_A8W8_WS_BYTES = {}      # (M, N, K) -> bytes of workspace the library would use for the shape (0: none)
+_A8W8_WORKSPACES = {}    # (device index, stream handle) -> zero-initialised workspace tensor
+
+
+def _a8w8_workspace(lib, device, stream, M, N, K):
+    """The workspace for a shape whose K the library would split over several workgroups per tile, or
+    None.  One buffer per device and stream (calls on one stream run in order; calls that overlap must not
+    share it), allocated at the first shape that needs one and sized for every shape (no plan takes more
+    than 224 slots of 64 KB).  It starts zeroed and every call leaves its counters zeroed."""
+    need = _A8W8_WS_BYTES.get((M, N, K))
+    if need is None:
+        need = _A8W8_WS_BYTES[(M, N, K)] = int(lib.fnn_gemm_a8w8_workspace_bytes(M, N, K))
+    if need == 0:
+        return None
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws = _A8W8_WORKSPACES.get(key)
+    if ws is None or ws.numel() < need:
+        ws = _A8W8_WORKSPACES[key] = torch.zeros(max(need, 16 << 20), dtype=torch.uint8, device=device)
+    return ws
+
+
 def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col, tile=None):
     """Replaces triton_gemm_a8w8_forward (flashnn/triton_kernels/gemm_a8w8.py:182-221).
 
@@ -153,7 +174,11 @@ def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col, tile=None):
         tile = tuned_configs.tune(f"gemm_a8w8_{M}_{N}_{K}", tuned_configs.A8W8_CANDIDATES,
                                   lambda t: _lib.check(lib.fnn_gemm_a8w8_tiled(*args, *t, stream)))
     if tile is None or tile[0] == 0:
-        _lib.check(lib.fnn_gemm_a8w8(*args, stream))
+        ws = _a8w8_workspace(lib, a.device, stream, M, N, K) if M > 64 else None
+        if ws is None:
+            _lib.check(lib.fnn_gemm_a8w8(*args, stream))
+        else:
+            _lib.check(lib.fnn_gemm_a8w8_ws(*args, ws.data_ptr(), ws.numel(), stream))
     else:
         _lib.check(lib.fnn_gemm_a8w8_tiled(*args, *tile, stream))
     return out

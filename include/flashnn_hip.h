@@ -179,6 +179,43 @@ int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, const void* alp
                         int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
                         int alpha_col_dtype, int tile_m, int tile_n, int waves, void* stream);
 
+/*
+ * fnn_gemm_a8w8 with a workspace: where few tiles would leave most CUs idle over a long K (M and N small,
+ * K of 8192 and more), K is cut into parts that run as separate workgroups; the parts' int32 accumulators
+ * meet in the workspace and the last part to finish a tile adds them up and writes the scaled output.
+ * Integer addition does not depend on the order, so the result equals fnn_gemm_a8w8's bit for bit.  Shapes
+ * that do not gain run exactly as in fnn_gemm_a8w8.  The role of the SPLIT_K meta-parameter of the
+ * reference's kernel (flashnn/triton_kernels/gemm_a8w8.py:17-50, 74-179), whose parts meet through
+ * tl.atomic_add on an output the caller has zeroed.
+ *
+ * workspace  device memory, 16-byte aligned; its first 4096 bytes are counters that must be zero when a
+ *            call starts and are zero again when it ends: zero them once after allocation
+ *            (fnn_workspace_init, or hipMemset / a zero-filled tensor) and never again.  The rest needs no
+ *            initialisation.  Calls that overlap in time (other streams, other threads) need a workspace
+ *            each.
+ * ws_bytes   its size.  fnn_gemm_a8w8_workspace_bytes(M, N, K) is what the call would use for a shape (0:
+ *            the shape is not split); 16 MiB hold every shape.  With less than a shape needs the call
+ *            runs unsplit.
+ */
+size_t fnn_gemm_a8w8_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int fnn_workspace_init(void* workspace, size_t ws_bytes, void* stream);
+int fnn_gemm_a8w8_ws(void* out, const void* a, const void* b, const void* alpha_row,
+                     const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                     int64_t ldc, int out_dtype, int alpha_row_dtype, int alpha_col_dtype,
+                     void* workspace, size_t ws_bytes, void* stream);
+
+/*
+ * fnn_gemm_a8w8_ws with the tile and the number of parts named: tiles 256x128, 256x192 and 128x128, kparts
+ * from 2 up as long as a part holds four slabs of 128 bytes of K; kparts 0 or 1 is fnn_gemm_a8w8_tiled.
+ * FNN_ERR_ARG if the shape cannot be split so or the workspace is too small (the message says what is
+ * needed).  For tests and tuning; results are bit-identical for every choice.
+ */
+int fnn_gemm_a8w8_ws_tiled(void* out, const void* a, const void* b, const void* alpha_row,
+                           const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
+                           int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
+                           int alpha_col_dtype, int tile_m, int tile_n, int kparts, void* workspace,
+                           size_t ws_bytes, void* stream);
+
 /* fnn_gemm_a8w8_i32 through a named tile (same tiles as fnn_gemm_a8w8_tiled): lets a test check the integer
  * result of every tile bit for bit.  No counterpart in the reference API. */
 int fnn_gemm_a8w8_i32_tiled(int32_t* acc, const void* a, const void* b, int64_t M, int64_t N, int64_t K,

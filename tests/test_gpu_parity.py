@@ -311,6 +311,80 @@ def test_a8w8_reference_sweep_shapes(nk, M):
     assert torch.equal(acc.sum(dim=1, dtype=torch.int64), (a.to(torch.int64) * colsum).sum(dim=1))
 
 
+def _a8w8_ws_call(hip_lib, out, a, b, ar, ac, ws, plan=None):
+    M, K = a.shape
+    N = b.shape[0]
+    args = (out.data_ptr(), a.data_ptr(), b.data_ptr(), ar.data_ptr(), ac.data_ptr(), M, N, K, K, K, N,
+            _lib.dtype_code(out.dtype), _lib.dtype_code(ar.dtype), _lib.dtype_code(ac.dtype))
+    st = _lib.current_stream(a.device)
+    if plan is None:
+        return hip_lib.fnn_gemm_a8w8_ws(*args, ws.data_ptr(), ws.numel(), st)
+    return hip_lib.fnn_gemm_a8w8_ws_tiled(*args, *plan, ws.data_ptr(), ws.numel(), st)
+
+
+@pytest.mark.parametrize("plan", [(256, 128, 2), (256, 128, 3), (256, 192, 2), (256, 192, 5), (128, 128, 2), (128, 128, 4),
+                                  (128, 128, 7)])
+@pytest.mark.parametrize("mnk", [(300, 520, 4096), (128, 1024, 8192), (257, 385, 5152), (96, 200, 4128), (640, 256, 6240)])
+def test_a8w8_split_k_bit_exact(hip_lib, plan, mnk):
+    """K cut into parts that meet in a workspace: the int32 sums do not depend on the order of arrival, so
+    the scaled output equals the unsplit kernel's and the oracle's bit for bit - for every tile, number of
+    parts, ragged edges and a partial last slab; the counters are zero again afterwards; a second call on
+    the same workspace (holding the first call's slots) gives the same bits."""
+    M, N, K = mnk
+    a, b = _rand_i8((M, K), 61).to(DEV), _rand_i8((N, K), 62).to(DEV)
+    g = torch.Generator().manual_seed(63)
+    ar = (torch.rand(M, generator=g) * 1e-2 + 1e-3).half().to(DEV)
+    ac = (torch.rand(N, generator=g) * 1e-2 + 1e-3).float().to(DEV)
+    ws = torch.zeros(24 << 20, dtype=torch.uint8, device=DEV)
+    ws[4096:] = 0x5a                                   # only the counters need to start at zero
+    want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.cpu().numpy(), b.cpu().numpy()), O.to_np(ar.cpu()),
+                                     ac.cpu().numpy(), O.BF16)
+    for rep in range(2):
+        out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        rc = _a8w8_ws_call(hip_lib, out, a, b, ar, ac, ws, plan)
+        assert rc == 0, hip_lib.fnn_last_error()
+        assert _lib.last_kernel() == f"gemm_a8w8_ring_kernel(split K)<{plan[0]},{plan[1]},{plan[2]}>"
+        assert np.array_equal(out.float().cpu().numpy(), want)
+        assert int(ws[:4096].view(torch.int32).abs().sum()) == 0
+    plain = torch.empty_like(out)
+    launchers.hip_gemm_a8w8_forward(plain, a, b, ar, ac, tile=(plan[0], plan[1], 0))
+    assert torch.equal(plain, out)
+
+
+@pytest.mark.parametrize("mnk", [(256, 4096, 8192), (128, 2048, 16384), (384, 1920, 13312), (100, 1000, 9248), (2048, 4096, 4096)])
+def test_a8w8_workspace_entry_matches_plain(hip_lib, mnk):
+    """fnn_gemm_a8w8_ws: shapes the library splits (and one it does not) against fnn_gemm_a8w8, bit for bit,
+    through the operator too (its launcher keeps a workspace per stream); a workspace smaller than the
+    shape needs runs unsplit."""
+    M, N, K = mnk
+    g = torch.Generator(device=DEV).manual_seed(K + M)
+    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+    b = torch.randint(-128, 128, (N, K), dtype=torch.int8, device=DEV, generator=g)
+    ar = (torch.rand(M, device=DEV, generator=g) * 1e-2 + 1e-3).half()
+    ac = (torch.rand(N, device=DEV, generator=g) * 1e-2 + 1e-3).half()
+    need = hip_lib.fnn_gemm_a8w8_workspace_bytes(M, N, K)
+    assert (need > 0) == (M < 2048) and need <= 16 << 20
+    plain = torch.empty(M, N, dtype=torch.float16, device=DEV)
+    assert hip_lib.fnn_gemm_a8w8(plain.data_ptr(), a.data_ptr(), b.data_ptr(), ar.data_ptr(), ac.data_ptr(), M, N, K, K, K, N,
+                                 0, 0, 0, _lib.current_stream(a.device)) == 0
+    unsplit_kernel = _lib.last_kernel()
+    ws = torch.empty(16 << 20, dtype=torch.uint8, device=DEV)
+    assert hip_lib.fnn_workspace_init(ws.data_ptr(), ws.numel(), _lib.current_stream(a.device)) == 0
+    out = torch.empty_like(plain)
+    assert _a8w8_ws_call(hip_lib, out, a, b, ar, ac, ws) == 0
+    assert ("split K" in _lib.last_kernel()) == (need > 0)
+    assert torch.equal(out, plain)
+    via_op = flashnn_amd.GemmA8W8(torch.float16)(a, b, ar, ac)
+    assert ("split K" in _lib.last_kernel()) == (need > 0) and torch.equal(via_op, plain)
+    if need:
+        out.zero_()
+        assert _a8w8_ws_call(hip_lib, out, a, b, ar, ac, ws[:need - 16]) == 0
+        assert _lib.last_kernel() == unsplit_kernel and torch.equal(out, plain)
+    want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a[:3].cpu().numpy(), b.cpu().numpy()), O.to_np(ar[:3].cpu()),
+                                     O.to_np(ac.cpu()), O.F16)
+    assert np.array_equal(out[:3].float().cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("side", ["activations", "weights"])
 def test_a8w8_operand_of_2_gib_and_more(side):
     """An operand whose last rows lie 2^31 bytes and more behind its first (a long prefill; a very wide

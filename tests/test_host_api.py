@@ -192,6 +192,30 @@ def test_tiled_entry_rejects_unknown_tiles(hip_lib):
     assert rc == -1 and b"no such tile 256x256 with 4 waves" in hip_lib.fnn_last_error()
 
 
+def test_workspace_entries_reject_bad_arguments(hip_lib):
+    one = ctypes.c_void_p(4096)
+    odd = ctypes.c_void_p(4100)
+    null = ctypes.c_void_p(0)
+    base = (one, one, one, one, one, 256, 256, 8192, 8192, 8192, 256, 0, 0, 0)
+    assert hip_lib.fnn_workspace_init(null, 1 << 20, null) == -1
+    assert hip_lib.fnn_workspace_init(one, 100, null) == -1 and b"at least 4096 bytes" in hip_lib.fnn_last_error()
+    assert hip_lib.fnn_gemm_a8w8_ws(*base, odd, 1 << 20, null) == -1 and b"16-byte aligned" in hip_lib.fnn_last_error()
+    assert hip_lib.fnn_gemm_a8w8_ws(*base, null, 1 << 20, null) == -1
+    # a named split the shape cannot take, an unknown tile for a split, a workspace that is too small
+    assert hip_lib.fnn_gemm_a8w8_ws_tiled(*base, 256, 128, 40, one, 1 << 30, null) == -1
+    assert b"cannot be split 40 ways" in hip_lib.fnn_last_error()
+    assert hip_lib.fnn_gemm_a8w8_ws_tiled(*base, 64, 128, 2, one, 1 << 30, null) == -1
+    assert hip_lib.fnn_gemm_a8w8_ws_tiled(*base, 256, 128, 2, one, 8192, null) == -1
+    assert b"the split needs 528384" in hip_lib.fnn_last_error()
+    assert hip_lib.fnn_gemm_a8w8_ws_tiled(*base, 256, 128, -1, one, 1 << 30, null) == -1
+    # which shapes the library would split, and that nothing needs more than 16 MiB
+    f = hip_lib.fnn_gemm_a8w8_workspace_bytes
+    assert f(2048, 12288, 4096) == 0 and f(16, 4096, 8192) == 0 and f(512, 8192, 8192) == 0
+    assert f(256, 4096, 8192) == 4096 + 64 * 3 * 65536
+    assert all(f(M, N, K) <= 16 << 20 for M in (65, 100, 128, 500, 1000, 3000) for N in (128, 1000, 4096, 20000)
+               for K in (8192, 16384, 32768))
+
+
 def test_empty_calls_need_no_addresses(hip_lib):
     """M = 0 / N = 0 returns before anything is launched and accepts NULL tensors (an empty torch tensor
     has data_ptr() == 0); with rows present the same NULLs are rejected."""
