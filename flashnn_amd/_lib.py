@@ -29,6 +29,7 @@ _SIGNATURES = {
     "fnn_workspace_init": [_ptr, _size, _ptr],
     "fnn_gemm_a8w8_ws": [_ptr] * 5 + [_i64] * 6 + [_int] * 3 + [_ptr, _size, _ptr],
     "fnn_gemm_a8w8_ws_tiled": [_ptr] * 5 + [_i64] * 6 + [_int] * 6 + [_ptr, _size, _ptr],
+    "fnn_gemm_a8w8_static": [_ptr] * 5 + [_i64] * 6 + [_int] * 6 + [_ptr],
     "fnn_gemm_a8w8_i32": [_ptr] * 3 + [_i64] * 6 + [_ptr],
     "fnn_gemm_a8w8_i32_tiled": [_ptr] * 3 + [_i64] * 6 + [_int] * 3 + [_ptr],
     "fnn_gemm_a16w8": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],

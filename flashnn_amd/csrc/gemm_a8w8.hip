@@ -27,6 +27,8 @@
 
 #include "a8w8_common.h"
 
+#include <atomic>
+
 // The scaled output is two fp32 multiplications and one rounding to 16 bits, each rounded on its
 // own as in the reference's torch path.
 #pragma clang fp contract(off)
@@ -1052,6 +1054,62 @@ extern "C" int fnn_gemm_a8w8_ws_tiled(void* out, const void* a, const void* b, c
     return gemm_a8w8_entry("fnn_gemm_a8w8_ws_tiled", out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc,
                            out_dtype, alpha_row_dtype, alpha_col_dtype, tile_m, tile_n, 0, stream,
                            Workspace{workspace, ws_bytes, kparts == 1 ? 0 : kparts});
+}
+
+// ---- the workspace held by the library itself, for callers that cannot allocate ----
+// One array per GPU, part of the code object: every GPU the library runs on holds it from the moment the
+// library's code is loaded there until the process ends.  In host code the array's name is only a handle
+// for hipGetSymbolAddress - the device address differs per GPU and is looked up once per device.
+constexpr size_t kStaticScratchBytes = 16u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static std::atomic<void*> g_scratch_of[64];     // device address of `scratch` on each device, once known
+
+static int static_scratch(const char* fn, void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) {
+        set_error("%s: no current device (%s)", fn, hipGetErrorString(e));
+        return FNN_ERR_HIP;
+    }
+    void* ptr = g_scratch_of[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));     // the current device's copy of the array
+        if (e != hipSuccess || !ptr) {
+            set_error("%s: hipGetSymbolAddress failed on device %d: %s", fn, dev, hipGetErrorString(e));
+            return FNN_ERR_HIP;
+        }
+        g_scratch_of[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return FNN_OK;
+}
+
+extern "C" int fnn_gemm_a8w8_static(void* out, const void* a, const void* b, const void* alpha_row,
+                                    const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                    int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
+                                    int alpha_col_dtype, int tile_m, int tile_n, int kparts, void* stream) {
+    const char* fn = "fnn_gemm_a8w8_static";
+    if (kparts > 1 && M > 0 && N > 0 && K > 0 && tile_m > 0 && tile_n > 0) {
+        // a named split is the only way to ask for more than the array holds (the library's own plans fit)
+        const SplitPlan s{tile_m, tile_n, kparts, 0, 0.0};
+        const size_t need = split_ws_bytes(s, M, N);
+        if (need > kStaticScratchBytes) {
+            set_error("%s: this split needs %zu bytes of workspace, the library's own holds %zu; use "
+                      "fnn_gemm_a8w8_ws_tiled with a workspace of that size, or fewer parts", fn, need,
+                      kStaticScratchBytes);
+            return FNN_ERR_UNSUPPORTED;
+        }
+    }
+    void* ws = nullptr;
+    const int rc = static_scratch(fn, &ws);
+    if (rc != FNN_OK) return rc;
+    // The counters at the start of the array are zero when the code is loaded and every call's kernel
+    // returns the counters it used to zero before it ends (the unit that adds up a tile clears the tile's
+    // counter), so this call finds them zero; the slots behind them need no clearing.
+    return gemm_a8w8_entry(fn, out, a, b, alpha_row, alpha_col, M, N, K, lda, ldb, ldc, out_dtype, alpha_row_dtype,
+                           alpha_col_dtype, tile_m, tile_n, 0, stream,
+                           Workspace{ws, kStaticScratchBytes, kparts == 1 ? 0 : kparts});
 }
 
 extern "C" int fnn_gemm_a8w8_i32(int32_t* acc, const void* a, const void* b, int64_t M, int64_t N,

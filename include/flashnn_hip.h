@@ -17,7 +17,8 @@
  *   - return value: 0 ok, FNN_ERR_ARG (-1) bad argument, FNN_ERR_UNSUPPORTED (-2)
  *     shape/dtype not handled, FNN_ERR_HIP (-3) HIP runtime error.  After a non-zero
  *     return fnn_last_error() gives a thread-local, human-readable message.
- *   - calls are re-entrant and never allocate, free or synchronise.  State kept between calls:
+ *   - calls are re-entrant (fnn_gemm_a8w8_static excepted: see there) and never allocate, free or
+ *     synchronise.  State kept between calls:
  *     per thread the last error message and the name of the last kernel launched; per
  *     process, set once and never changed again, which devices have had a kernel's LDS
  *     limit raised and (only with FLASHNN_HIP_LOG=1) which kernel variants have been
@@ -215,6 +216,25 @@ int fnn_gemm_a8w8_ws_tiled(void* out, const void* a, const void* b, const void* 
                            int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
                            int alpha_col_dtype, int tile_m, int tile_n, int kparts, void* workspace,
                            size_t ws_bytes, void* stream);
+
+/*
+ * fnn_gemm_a8w8_ws_tiled without the workspace argument: the workspace is an array of 16 MiB that the
+ * library holds on every GPU it runs on (part of its code object, from load to the end of the process).
+ * No counterpart in the reference.  It is for callers that cannot allocate: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc - the call allocates and frees nothing (the device
+ * address of the array is looked up once per device, on the first call there).
+ *   tile_m = tile_n = kparts = 0: the library's choice, as fnn_gemm_a8w8_ws; its plans always fit.
+ *   a named split that needs more than the array holds: FNN_ERR_UNSUPPORTED, and the message says how
+ *   much; use fnn_gemm_a8w8_ws_tiled with a workspace of that size.
+ * All calls on a GPU share that GPU's array: calls that overlap in time (other streams, other threads)
+ * race on it and must use fnn_gemm_a8w8_ws with workspaces of their own.  The counters in the array are
+ * zero at load and every call's kernel sets the ones it used back to zero before it ends; the rest keeps
+ * the last call's contents and needs no clearing.  Results equal fnn_gemm_a8w8's bit for bit.
+ */
+int fnn_gemm_a8w8_static(void* out, const void* a, const void* b, const void* alpha_row,
+                         const void* alpha_col, int64_t M, int64_t N, int64_t K, int64_t lda,
+                         int64_t ldb, int64_t ldc, int out_dtype, int alpha_row_dtype,
+                         int alpha_col_dtype, int tile_m, int tile_n, int kparts, void* stream);
 
 /* fnn_gemm_a8w8_i32 through a named tile (same tiles as fnn_gemm_a8w8_tiled): lets a test check the integer
  * result of every tile bit for bit.  No counterpart in the reference API. */
