@@ -7,16 +7,25 @@ per-token x per-channel scale epilogue writing bf16 (the Llama-7B QKV prefill sh
 `value` is 2*M*N*K / step time in TOPS with all inputs resident in HBM.
 
 Also measured in the same run and reported in the same JSON line:
-  roofline          the A8W8 GEMM kernel alone against the dense int8 MFMA peak
-  secondary         the other configurations: the remaining prefill shapes, A16W4 group-128 at
-                    M = 1 .. 256 (M=1 is the decode GEMV of the second headline metric), A8W8 with
-                    few activation rows, A16W8 decode and the row kernels, each against its bound
-  cpu_baseline      the reference's torch CPU path (oracle/torch_path.py) on the host cores
+  roofline      the A8W8 GEMM kernel alone against the dense int8 MFMA peak
+  secondary     one entry per point of every configuration the path is quoted on, each against its bound:
+                  c1     DynamicQuant + A8W8 at M=16 K=N=4096, fp16 out
+                  c2     the four M=2048 prefill shapes (quant + GEMM, and the GEMM alone)
+                  c3     A16W8 decode, M in {1, 8, 32} x three (K, N)
+                  c4     A16W4 group-128 at K=8192 N=28672, M in {1, 4, 16, 64, 256}
+                  c5     RMSNormDquant -> A8W8 at K=N=8192, M in {1, 32, 512, 8192}
+                  g64    A16W4 group-64 at the reference test's shape M=3 N=1024 K=4096
+                  splitk A8W8 shapes whose K the library splits, against the unsplit kernel
+                  rows   the row kernels on their own;  moe  the fused mixture-of-experts GEMMs
+  cpu_baseline  the reference's torch CPU path (oracle/torch_path.py) on the host cores
 
-Operand sets are rotated so that the working set exceeds the 256 MB Infinity Cache; kernel
-durations come from HIP events recorded on the stream the kernels run on.
+Inputs come from flashnn_amd/workloads.py (the configured distributions); int8 activations are produced by
+the library's own quantisation of them.  Operand sets are rotated so that the working set exceeds the
+256 MB Infinity Cache.  Kernel durations are HIP events recorded on the stream the kernels run on; the
+kernel named in an entry is the one the library reports having launched (fnn_last_kernel).
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -27,14 +36,16 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA, published (5.0 POP/s)
+PEAK_F16_TFLOPS = 2500.0    # dense bf16 / fp16 MFMA, published (2.5 PFLOP/s)
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published (8 TB/s)
+ALL_LEGS = ("c1", "c2", "c3", "c4", "c5", "g64", "splitk", "rows", "moe")
 
 
-def _events_ms(fn, iters, torch, preroll_s=0.04):
-    """Average duration of fn() over `iters` back-to-back calls, HIP events on the current stream.
-    The calls are preceded by an untimed pre-roll of the same call: host-side input generation between the
-    measurements leaves the device idle long enough for its clocks to drop, and a hundred launches of a
-    20 us kernel would otherwise be over before they have come back."""
+def _timed(fn, iters, torch, preroll_s=0.04):
+    """(average milliseconds by HIP events on the current stream, average host wall milliseconds) of
+    fn(i) over `iters` back-to-back calls.  An untimed pre-roll of the same call comes first and is in
+    neither figure: host-side input generation between the measurements leaves the device idle long enough
+    for its clocks to drop, and a hundred launches of a 20 us kernel would be over before they are back."""
     t0 = time.perf_counter()
     k = 0
     while time.perf_counter() - t0 < preroll_s:
@@ -45,21 +56,41 @@ def _events_ms(fn, iters, torch, preroll_s=0.04):
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
+    w0 = time.perf_counter()
     start.record()
     for i in range(iters):
         fn(i)
     end.record()
     torch.cuda.synchronize()
-    return start.elapsed_time(end) / iters
+    wall = (time.perf_counter() - w0) * 1e3 / iters
+    return start.elapsed_time(end) / iters, wall
 
 
-def _traffic(kernel):
-    """HBM bytes per launch measured with rocprofv3 --pmc (profiles/traffic.json), or None."""
+def _traffic(key):
+    """HBM bytes per launch measured with rocprofv3 --pmc for the workload `key` (profiles/traffic.json:
+    FETCH_SIZE and WRITE_SIZE readings scaled by what a plain copy of known size reads), or None."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     if not os.path.exists(path):
         return None
     with open(path) as f:
-        return json.load(f).get(kernel)
+        rec = json.load(f).get(key)
+    return rec["bytes"] if rec else None
+
+
+def _entry(workload, ms, bound, amount, kernels, traffic_key=None, **extra):
+    """One secondary entry.  amount: algorithmic operations (bound 'mfma' / 'mfma16') or bytes ('hbm') per
+    call of the timed function."""
+    if bound == "hbm":
+        achieved, peak, unit = amount / (ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+    else:
+        achieved, unit = amount / (ms * 1e-3) / 1e12, "TOP/s" if bound == "mfma" else "TFLOP/s"
+        peak = PEAK_INT8_TOPS if bound == "mfma" else PEAK_F16_TFLOPS
+    e = {"workload": workload, "kernel": kernels, "us_per_launch": round(ms * 1e3, 2),
+         "roofline": {"bound": "hbm" if bound == "hbm" else "mfma", "achieved": round(achieved, 1), "peak": peak,
+                      "unit": unit, "frac": round(achieved / peak, 4),
+                      "traffic": _traffic(traffic_key) if traffic_key else None}}
+    e.update(extra)
+    return e
 
 
 def main():
@@ -68,7 +99,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="comma list of legs: a8w8,a16w4,rows,moe,calib (default: all but calib)")
+    ap.add_argument("--only", default="", help="comma list of secondary legs (%s, calib, none); default: all but calib"
+                    % ", ".join(ALL_LEGS))
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (one MI355X per box); run with --gpus 1. "
@@ -80,13 +112,24 @@ def main():
     import flashnn_amd
     from flashnn_amd import _lib, launchers, workloads
 
-    _lib.load()
+    lib = _lib.load()
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = "cuda:0"
-    legs = set(args.only.split(",")) if args.only else {"a8w8", "a16w4", "rows", "moe"}
+    legs = set(args.only.split(",")) if args.only else set(ALL_LEGS)
     props = torch.cuda.get_device_properties(0)
-    result = {}
+    secondary = []
+    iters = max(20, min(args.steps, 100))
+
+    def kernel_of(fn):
+        fn(0)
+        return _lib.last_kernel()
+
+    def rotating(t, total_bytes=300e6, at_least=2, at_most=64):
+        """Copies of a device tensor, enough that one pass over them exceeds the Infinity Cache."""
+        n = int(total_bytes // max(1, t.numel() * t.element_size())) + 1
+        n = max(at_least, min(at_most, n))
+        return [t] + [t.clone() for _ in range(n - 1)]
 
     if "calib" in legs:
         # a plain copy of known size: the counter readings of FETCH_SIZE / WRITE_SIZE for this
@@ -99,58 +142,66 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
-    # ------------------------------------------------------------------ primary: A8W8
-    M, K, N = 2048, 4096, 12288
-    x_cpu = workloads.activations(M, K, torch.float16, seed=0, outlier_frac=0.01)
-    w_cpu, ws_cpu = workloads.int8_weights(N, K, seed=1)
-    nset = 4   # 4 x (8 + 50 + 50 + 17) MB > 256 MB
-    xs = [x_cpu.to(dev).clone() for _ in range(nset)]
-    ws = [w_cpu.to(dev).clone() for _ in range(nset)]
-    wscale = ws_cpu.to(dev)
-    qs = [torch.empty(M, K, dtype=torch.int8, device=dev) for _ in range(nset)]
-    ss = [torch.empty(M, dtype=torch.float16, device=dev) for _ in range(nset)]
-    outs = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nset)]
+    # --------------------------------------------- c2: A8W8 prefill, M = 2048 (qkv is the primary workload)
+    M = 2048
+    x_cpu = workloads.activations(M, 4096, torch.float16, seed=0, outlier_frac=0.01)
+    primary = None
+    w_qkv = ws_qkv = None
+    for name, (K, N) in workloads.A8W8_PREFILL_SHAPES.items():
+        if name != "qkv" and "c2" not in legs:
+            continue
+        x = x_cpu if K == 4096 else workloads.activations(M, K, torch.float16, seed=0, outlier_frac=0.01)
+        w_cpu, wsc_cpu = workloads.int8_weights(N, K, seed=1)
+        if name == "qkv":
+            w_qkv, ws_qkv = w_cpu, wsc_cpu
+        ws = rotating(w_cpu.to(dev), at_least=3)
+        n = len(ws)
+        xs = [x.to(dev).clone() for _ in range(n)]
+        wscale = wsc_cpu.to(dev)
+        qs = [torch.empty(M, K, dtype=torch.int8, device=dev) for _ in range(n)]
+        ss = [torch.empty(M, dtype=torch.float16, device=dev) for _ in range(n)]
+        outs = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(n)]
 
-    def step(i):
-        j = i % nset
-        launchers.hip_dynamic_quantize(qs[j], xs[j], ss[j])
-        launchers.hip_gemm_a8w8_forward(outs[j], qs[j], ws[j], ss[j], wscale)
+        def quant_only(i):
+            launchers.hip_dynamic_quantize(qs[i % n], xs[i % n], ss[i % n])
 
-    def gemm_only(i):
-        j = i % nset
-        launchers.hip_gemm_a8w8_forward(outs[j], qs[j], ws[j], ss[j], wscale)
+        def gemm_only(i):
+            launchers.hip_gemm_a8w8_forward(outs[i % n], qs[i % n], ws[i % n], ss[i % n], wscale)
 
-    def quant_only(i):
-        j = i % nset
-        launchers.hip_dynamic_quantize(qs[j], xs[j], ss[j])
+        def step(i):
+            quant_only(i)
+            gemm_only(i)
 
-    # The device leaves its idle clocks only after some tens of milliseconds of work (measured: 113 us per
-    # step right after 20 warm-up steps, 102 us from 200 warm-up steps on), so whatever --warmup says the
-    # steps are preceded by an untimed pre-roll of about 60 ms of the same step.
-    preroll_steps = 0
-    t_pre = time.perf_counter()
-    while time.perf_counter() - t_pre < 0.06:
-        for i in range(50):
-            step(i)
-        torch.cuda.synchronize()
-        preroll_steps += 50
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ms_step = _events_ms(step, args.steps, torch)
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ops = 2.0 * M * N * K
-    value = ops / (ms_step * 1e-3) / 1e12
-    ms_gemm = _events_ms(gemm_only, args.steps, torch)
-    ms_quant = _events_ms(quant_only, args.steps, torch)
-    gemm_tops = ops / (ms_gemm * 1e-3) / 1e12
-    roofline = {"kernel": "gemm_a8w8_ring_kernel", "bound": "mfma", "achieved": round(gemm_tops, 2),
+        ops = 2.0 * M * N * K
+        k_quant, k_gemm = kernel_of(quant_only), kernel_of(gemm_only)
+        if name == "qkv":
+            # The device leaves its idle clocks only after some tens of milliseconds of work (measured:
+            # 113 us per step right after 20 warm-up steps, 102 us from 200 warm-up steps on): whatever
+            # --warmup says, the steps are preceded by an untimed pre-roll of the same step.
+            for i in range(args.warmup):
+                step(i)
+            torch.cuda.synchronize()
+            ms_step, wall_ms = _timed(step, args.steps, torch, preroll_s=0.06)
+            ms_gemm, _ = _timed(gemm_only, args.steps, torch)
+            ms_quant, _ = _timed(quant_only, args.steps, torch)
+            primary = dict(M=M, K=K, N=N, ops=ops, ms_step=ms_step, wall_ms=wall_ms, ms_gemm=ms_gemm, nset=n,
+                           k_gemm=k_gemm, k_quant=k_quant)
+            if "rows" in legs:
+                secondary.append(_entry(f"dynamic_quant fp16 M={M} K={K}", ms_quant, "hbm", 3.0 * M * K + 2.0 * M,
+                                        k_quant, "dynamic_quant M=2048 K=4096"))
+        else:
+            ms_step, _ = _timed(step, iters, torch)
+            ms_gemm, _ = _timed(gemm_only, iters, torch)
+            secondary.append(_entry(f"c2 a8w8 {name} M={M} K={K} N={N} bf16: GEMM", ms_gemm, "mfma", ops, k_gemm,
+                                    f"a8w8 {name}", us_quant_plus_gemm=round(ms_step * 1e3, 2)))
+        del ws, xs, qs, ss, outs
+        torch.cuda.empty_cache()
+    gemm_tops = primary["ops"] / (primary["ms_gemm"] * 1e-3) / 1e12
+    roofline = {"kernel": primary["k_gemm"], "bound": "mfma", "achieved": round(gemm_tops, 2),
                 "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
-                "us_per_launch": round(ms_gemm * 1e3, 2), "traffic": _traffic("gemm_a8w8_ring_kernel")}
+                "us_per_launch": round(primary["ms_gemm"] * 1e3, 2), "traffic": _traffic("a8w8 qkv")}
     # what this device sustains on int8 MFMAs alone (operands in registers, about 0.1 s each): the
     # clock follows the power drawn, so random operand bytes run well below the datasheet rate
-    import ctypes
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     sustained = {}
     probe = ctypes.CDLL(os.path.join(ROOT, "flashnn_amd", "benchmarks", "libfnn_probe.so"))
@@ -165,212 +216,225 @@ def main():
         sustained[label] = round(rate.value, 1)
     roofline["mfma_only_sustained"] = dict(sustained, unit="TOP/s")
     roofline["frac_of_sustained_random"] = round(gemm_tops / sustained["random_operand_bytes"], 4)
-    secondary = []
-    qbytes = 3.0 * M * K + 2.0 * M
-    secondary.append({"workload": f"dynamic_quant fp16 M={M} K={K}", "kernel": "dynamic_quant_vec_kernel",
-                      "us_per_launch": round(ms_quant * 1e3, 2),
-                      "roofline": {"bound": "hbm", "achieved": round(qbytes / (ms_quant * 1e-3) / 1e9, 1),
-                                   "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                   "frac": round(qbytes / (ms_quant * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                                   "traffic": _traffic("dynamic_quant_vec_kernel")}})
-    del xs, ws, outs
-    torch.cuda.empty_cache()
 
-    # other prefill shapes (reported)
-    if "a8w8" in legs:
-        for name, (k2, n2) in workloads.A8W8_PREFILL_SHAPES.items():
-            if name == "qkv":
-                continue
-            a2 = [torch.randint(-127, 128, (M, k2), dtype=torch.int8, device=dev) for _ in range(3)]
-            b2 = [torch.randint(-127, 128, (n2, k2), dtype=torch.int8, device=dev) for _ in range(3)]
-            o2 = [torch.empty(M, n2, dtype=torch.bfloat16, device=dev) for _ in range(3)]
-            s2 = torch.rand(M, device=dev).half()
-            c2 = torch.rand(n2, device=dev)
-            f = lambda i: launchers.hip_gemm_a8w8_forward(o2[i % 3], a2[i % 3], b2[i % 3], s2, c2)
-            for i in range(5):
-                f(i)
-            ms = _events_ms(f, 50, torch)
-            t = 2.0 * M * n2 * k2 / (ms * 1e-3) / 1e12
-            secondary.append({"workload": f"a8w8 {name} M={M} K={k2} N={n2} bf16", "kernel": "gemm_a8w8_ring_kernel",
-                              "us_per_launch": round(ms * 1e3, 2),
-                              "roofline": {"bound": "mfma", "achieved": round(t, 2), "peak": PEAK_INT8_TOPS,
-                                           "unit": "TOP/s", "frac": round(t / PEAK_INT8_TOPS, 4), "traffic": None}})
-            del a2, b2, o2
+    # ------------------------------------------------------- c1: DynamicQuant + A8W8, M = 16, fp16 out
+    x1_cpu = workloads.activations(16, 4096, torch.float16, seed=10)
+    w1_cpu, ws1_cpu = workloads.int8_weights(4096, 4096, seed=11)
+    if "c1" in legs:
+        M1, K1, N1 = 16, 4096, 4096
+        ws = rotating(w1_cpu.to(dev))
+        n = len(ws)
+        x1, wsc = x1_cpu.to(dev), ws1_cpu.to(dev)
+        q1 = torch.empty(M1, K1, dtype=torch.int8, device=dev)
+        s1 = torch.empty(M1, dtype=torch.float16, device=dev)
+        o1 = torch.empty(M1, N1, dtype=torch.float16, device=dev)
+
+        def gemm1(i):
+            launchers.hip_gemm_a8w8_forward(o1, q1, ws[i % n], s1, wsc)
+
+        def step1(i):
+            launchers.hip_dynamic_quantize(q1, x1, s1)
+            gemm1(i)
+
+        kq = kernel_of(lambda i: launchers.hip_dynamic_quantize(q1, x1, s1))
+        kg = kernel_of(gemm1)
+        ms_s, _ = _timed(step1, iters, torch)
+        ms_g, _ = _timed(gemm1, iters, torch)
+        b1 = float(N1) * K1 + M1 * K1 + 2.0 * M1 * N1 + 2.0 * M1 + 4.0 * N1
+        secondary.append(_entry(f"c1 a8w8 M={M1} K={K1} N={N1} fp16: GEMM", ms_g, "hbm", b1, kg,
+                                us_quant_plus_gemm=round(ms_s * 1e3, 2), quant_kernel=kq))
+        del ws
         torch.cuda.empty_cache()
 
-    # -------------------------------------------------------------- A16W4 decode GEMV
+    # ----------------------------------------------- c5: RMSNormDquant -> A8W8, K = N = 8192, bf16
+    if "c5" in legs:
+        K5 = N5 = 8192
+        w5_cpu, ws5_cpu = workloads.int8_weights(N5, K5, seed=52)
+        ws = rotating(w5_cpu.to(dev), at_least=4)
+        n = len(ws)
+        wsc = ws5_cpu.to(dev)
+        norm = flashnn_amd.RMSNormDquant(K5, eps=1e-6).to(dev)
+        norm.weight.data = workloads.rmsnorm_gamma(K5).to(dev)
+        gemm5 = flashnn_amd.GemmA8W8(torch.bfloat16)
+        for M5 in (1, 32, 512, 8192):
+            h = workloads.activations(M5, K5, torch.bfloat16, seed=51, outlier_frac=0.01).to(dev)
+            hs = rotating(h, total_bytes=300e6 if M5 >= 512 else 0, at_least=1, at_most=3)
+            nh = len(hs)
+            q5, s5 = norm(h)
+
+            def chain(i):
+                q, s = norm(hs[i % nh])
+                gemm5(q, ws[i % n], s, wsc)
+
+            def gemm_alone(i):
+                gemm5(q5, ws[i % n], s5, wsc)
+
+            kn = kernel_of(lambda i: norm(h))
+            kg = kernel_of(gemm_alone)
+            ms_c, _ = _timed(chain, iters if M5 < 8192 else 20, torch)
+            ms_g, _ = _timed(gemm_alone, iters if M5 < 8192 else 20, torch)
+            if M5 <= 32:
+                amount, bound = float(N5) * K5 + M5 * K5 + 2.0 * M5 * N5 + 2.0 * M5 + 4.0 * N5, "hbm"
+            else:
+                amount, bound = 2.0 * M5 * N5 * K5, "mfma"
+            secondary.append(_entry(f"c5 rmsnorm_dquant -> a8w8 M={M5} K={K5} N={N5} bf16: GEMM", ms_g, bound, amount,
+                                    kg, f"a8w8 c5 M={M5}", us_norm_plus_gemm=round(ms_c * 1e3, 2), norm_kernel=kn))
+            del hs
+        del ws
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------- c4: A16W4 group 128, K = 8192, N = 28672, bf16
     K4, N4 = workloads.A16W4_SHAPE
     packed, scale4, zp4, _, _ = workloads.int4_group_weights(N4, K4, 128)
-    if "a16w4" in legs:
-        nset4 = 5   # 5 x 125 MB
-        pk = [packed.to(dev).clone() for _ in range(nset4)]
-        sc = [scale4.to(dev).clone() for _ in range(nset4)]
-        zp = [zp4.to(dev).clone() for _ in range(nset4)]
+    if "c4" in legs:
+        pk = rotating(packed.to(dev), total_bytes=500e6)
+        n = len(pk)
+        sc = [scale4.to(dev).clone() for _ in range(n)]
+        zp = [zp4.to(dev).clone() for _ in range(n)]
+        wbytes = N4 * K4 / 2 + 2 * (K4 // 128) * N4 * 2
         for m4 in (1, 4, 16, 64, 256):
             act = workloads.activations(m4, K4, torch.bfloat16, seed=3).to(dev)
             o4 = torch.empty(m4, N4, dtype=torch.bfloat16, device=dev)
-            f = lambda i: launchers.hip_gemm_a16w4_forward(o4, act, pk[i % nset4], sc[i % nset4], None, zp[i % nset4])
-            for i in range(10):
-                f(i)
-            ms = _events_ms(f, 100, torch)
-            wbytes = N4 * K4 / 2 + 2 * (K4 // 128) * N4 * 2
-            allbytes = wbytes + 2.0 * m4 * K4 + 2.0 * m4 * N4
-            gbs = allbytes / (ms * 1e-3) / 1e9
-            secondary.append({"workload": f"a16w4 g128 decode M={m4} K={K4} N={N4} bf16",
-                              "kernel": "gemm_wo_gemv_kernel" if m4 <= 4 else "gemm_wo_panel_kernel", "us_per_launch": round(ms * 1e3, 2),
-                              "weight_GBps": round(wbytes / (ms * 1e-3) / 1e9, 1),
-                              "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-                                           "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
-                                           "traffic": _traffic("gemm_wo_gemv_kernel") if m4 == 1 else None}})
+            f = lambda i: launchers.hip_gemm_a16w4_forward(o4, act, pk[i % n], sc[i % n], None, zp[i % n])
+            kern = kernel_of(f)
+            ms, _ = _timed(f, iters, torch)
+            extra = {"weight_GBps": round(wbytes / (ms * 1e-3) / 1e9, 1)}
+            if m4 >= 64:      # also as a matrix-core workload
+                extra["bf16_TFLOPs"] = round(2.0 * m4 * N4 * K4 / (ms * 1e-3) / 1e12, 1)
+                extra["frac_of_bf16_peak"] = round(2.0 * m4 * N4 * K4 / (ms * 1e-3) / 1e12 / PEAK_F16_TFLOPS, 4)
+            secondary.append(_entry(f"c4 a16w4 g128 M={m4} K={K4} N={N4} bf16", ms, "hbm",
+                                    wbytes + 2.0 * m4 * K4 + 2.0 * m4 * N4, kern, f"a16w4 g128 M={m4}", **extra))
         del pk, sc, zp
         torch.cuda.empty_cache()
 
-    # ------------------------------------- few activation rows: RMSNorm+quant -> A8W8, K = N = 8192
-    if "a8w8" in legs:
-        k5 = n5 = 8192
-        w5 = [torch.randint(-127, 128, (n5, k5), dtype=torch.int8, device=dev) for _ in range(5)]
-        c5 = torch.rand(n5, device=dev) * 0.01
-        for m5 in (1, 32):
-            a5 = torch.randint(-127, 128, (m5, k5), dtype=torch.int8, device=dev)
-            s5 = torch.rand(m5, device=dev).bfloat16()
-            o5 = torch.empty(m5, n5, dtype=torch.bfloat16, device=dev)
-            f = lambda i: launchers.hip_gemm_a8w8_forward(o5, a5, w5[i % 5], s5, c5)
-            for i in range(10):
-                f(i)
-            ms = _events_ms(f, 100, torch)
-            b5 = float(n5) * k5 + m5 * k5 + 2.0 * m5 * n5 + 2.0 * m5 + 4.0 * n5
-            secondary.append({"workload": f"a8w8 few rows M={m5} K={k5} N={n5} bf16",
-                              "kernel": "gemm_a8w8_skinny_kernel" if m5 == 1 else "gemm_a8w8_panel_kernel",
-                              "us_per_launch": round(ms * 1e3, 2),
-                              "roofline": {"bound": "hbm", "achieved": round(b5 / (ms * 1e-3) / 1e9, 1),
-                                           "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                           "frac": round(b5 / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
-        del w5
+    # ------------------------------------------------------------ c3: A16W8 decode, fp16, per-channel
+    if "c3" in legs:
+        for (K8, N8) in workloads.A16W8_DECODE_SHAPES:
+            w8_cpu, s8_cpu = workloads.int8_weights(N8, K8, seed=40)
+            w8 = rotating(w8_cpu.to(dev), total_bytes=600e6, at_least=3)
+            n = len(w8)
+            s8 = s8_cpu.half().to(dev)
+            for m8 in (1, 8, 32):
+                act = workloads.activations(m8, K8, torch.float16, seed=4).to(dev)
+                o8 = torch.empty(m8, N8, dtype=torch.float16, device=dev)
+                f = lambda i: launchers.hip_gemm_a16w8_forward(o8, act, w8[i % n], s8)
+                kern = kernel_of(f)
+                ms, _ = _timed(f, iters, torch)
+                secondary.append(_entry(f"c3 a16w8 decode M={m8} K={K8} N={N8} fp16", ms, "hbm",
+                                        N8 * K8 + 2.0 * N8 + 2.0 * m8 * K8 + 2.0 * m8 * N8, kern))
+            del w8
         torch.cuda.empty_cache()
 
-    # ------------------------------------------------------- A16W8 decode + row kernels
+    # ----------------------------- g64: the reference test's A16W4 shape, M = 3, N = 1024, K = 4096, group 64
+    if "g64" in legs:
+        Mg, Ng, Kg = 3, 1024, 4096
+        pg, sg, zg, _, _ = workloads.int4_group_weights(Ng, Kg, 64, seed=64)
+        pgs = rotating(pg.to(dev), at_most=160)
+        n = len(pgs)
+        sgs = [sg.to(dev).clone() for _ in range(n)]
+        zgs = [zg.to(dev).clone() for _ in range(n)]
+        act = workloads.activations(Mg, Kg, torch.float16, seed=65).to(dev)
+        og = torch.empty(Mg, Ng, dtype=torch.float16, device=dev)
+        f = lambda i: launchers.hip_gemm_a16w4_forward(og, act, pgs[i % n], sgs[i % n], None, zgs[i % n])
+        kern = kernel_of(f)
+        ms, _ = _timed(f, iters, torch)
+        secondary.append(_entry(f"g64 a16w4 group 64 M={Mg} K={Kg} N={Ng} fp16 (the reference test's shape)", ms, "hbm",
+                                Ng * Kg / 2 + 4.0 * (Kg // 64) * Ng + 2.0 * Mg * Kg + 2.0 * Mg * Ng, kern))
+        del pgs, sgs, zgs
+        torch.cuda.empty_cache()
+
+    # --------------------- splitk: A8W8 shapes whose K the library splits over workgroups, and the unsplit kernel
+    if "splitk" in legs:
+        for (Ms, Ns, Ks) in ((256, 4096, 8192), (128, 2048, 16384), (384, 1920, 13312)):
+            xq = workloads.activations(Ms, Ks, torch.float16, seed=70, outlier_frac=0.01).to(dev)
+            qs_ = torch.empty(Ms, Ks, dtype=torch.int8, device=dev)
+            ss_ = torch.empty(Ms, dtype=torch.float16, device=dev)
+            launchers.hip_dynamic_quantize(qs_, xq, ss_)
+            wk_cpu, wks_cpu = workloads.int8_weights(Ns, Ks, seed=71)
+            wk = rotating(wk_cpu.to(dev))
+            n = len(wk)
+            wks = wks_cpu.to(dev)
+            ok = torch.empty(Ms, Ns, dtype=torch.bfloat16, device=dev)
+            split = lambda i: launchers.hip_gemm_a8w8_forward(ok, qs_, wk[i % n], ss_, wks)
+            st = _lib.current_stream(torch.device(dev))
+            plain = lambda i: _lib.check(lib.fnn_gemm_a8w8(
+                ok.data_ptr(), qs_.data_ptr(), wk[i % n].data_ptr(), ss_.data_ptr(), wks.data_ptr(), Ms, Ns, Ks, Ks, Ks, Ns,
+                _lib.dtype_code(ok.dtype), _lib.dtype_code(ss_.dtype), _lib.dtype_code(wks.dtype), st))
+            k_split, k_plain = kernel_of(split), kernel_of(plain)
+            ms_split, _ = _timed(split, iters, torch)
+            ms_plain, _ = _timed(plain, iters, torch)
+            secondary.append(_entry(f"splitk a8w8 M={Ms} K={Ks} N={Ns} bf16", ms_split, "mfma", 2.0 * Ms * Ns * Ks, k_split,
+                                    unsplit_us=round(ms_plain * 1e3, 2), unsplit_kernel=k_plain))
+            del wk
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------- rows: the row kernels on an 8192 x 8192 matrix
     if "rows" in legs:
-        for (k8, n8) in workloads.A16W8_DECODE_SHAPES:
-            nset8 = max(3, int(600e6 // (k8 * n8)) + 1)
-            w8 = [torch.randint(-127, 128, (n8, k8), dtype=torch.int8, device=dev) for _ in range(nset8)]
-            s8 = torch.rand(n8, device=dev).half() * 0.01
-            for m8 in (1, 8, 32):
-                act = workloads.activations(m8, k8, torch.float16, seed=4).to(dev)
-                o8 = torch.empty(m8, n8, dtype=torch.float16, device=dev)
-                f = lambda i: launchers.hip_gemm_a16w8_forward(o8, act, w8[i % nset8], s8)
-                for i in range(10):
-                    f(i)
-                ms = _events_ms(f, 100, torch)
-                b8 = n8 * k8 + 2.0 * n8 + 2.0 * m8 * k8 + 2.0 * m8 * n8
-                secondary.append({"workload": f"a16w8 decode M={m8} K={k8} N={n8} fp16",
-                                  "kernel": "gemm_wo_decode_lds_kernel" if m8 == 1 else "gemm_wo_panel_kernel",
-                                  "us_per_launch": round(ms * 1e3, 2),
-                                  "roofline": {"bound": "hbm", "achieved": round(b8 / (ms * 1e-3) / 1e9, 1),
-                                               "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                               "frac": round(b8 / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
-            del w8
         Mr, Kr = 8192, 8192
         hs = [workloads.activations(Mr, Kr, torch.bfloat16, seed=5, outlier_frac=0.01).to(dev) for _ in range(3)]
         norm = flashnn_amd.RMSNormDquant(Kr).to(dev)
         norm.weight.data = workloads.rmsnorm_gamma(Kr).to(dev)
         f = lambda i: norm(hs[i % 3])
-        for i in range(5):
-            f(i)
-        ms = _events_ms(f, 50, torch)
-        rb = 3.0 * Mr * Kr + 4.0 * Kr + 2.0 * Mr
-        secondary.append({"workload": f"rmsnorm_dquant bf16 M={Mr} K={Kr}", "kernel": "rmsnorm_dquant_vec_kernel",
-                          "us_per_launch": round(ms * 1e3, 2),
-                          "roofline": {"bound": "hbm", "achieved": round(rb / (ms * 1e-3) / 1e9, 1),
-                                       "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                       "frac": round(rb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+        kern = kernel_of(f)
+        ms, _ = _timed(f, 50, torch)
+        secondary.append(_entry(f"rmsnorm_dquant bf16 M={Mr} K={Kr}", ms, "hbm", 3.0 * Mr * Kr + 4.0 * Kr + 2.0 * Mr, kern))
         # the layers one step before the path, same matrix
-        for name, mod, kern, wr in (("rmsnorm", flashnn_amd.RMSNorm(Kr), "norm_vec_kernel", 2.0),
-                                    ("layernorm", flashnn_amd.LayerNorm(Kr), "norm_vec_kernel", 2.0),
-                                    ("layernorm_dquant", flashnn_amd.LayernormDquant(Kr), "norm_vec_kernel", 1.0)):
+        for name, mod, wr in (("rmsnorm", flashnn_amd.RMSNorm(Kr), 2.0), ("layernorm", flashnn_amd.LayerNorm(Kr), 2.0),
+                              ("layernorm_dquant", flashnn_amd.LayernormDquant(Kr), 1.0)):
             mod = mod.to(torch.bfloat16).to(dev)
             f = lambda i: mod(hs[i % 3])
-            for i in range(5):
-                f(i)
-            ms = _events_ms(f, 50, torch)
-            nb = (2.0 + wr) * Mr * Kr
-            secondary.append({"workload": f"{name} bf16 M={Mr} K={Kr}", "kernel": kern,
-                              "us_per_launch": round(ms * 1e3, 2),
-                              "roofline": {"bound": "hbm", "achieved": round(nb / (ms * 1e-3) / 1e9, 1),
-                                           "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                           "frac": round(nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+            kern = kernel_of(f)
+            ms, _ = _timed(f, 50, torch)
+            secondary.append(_entry(f"{name} bf16 M={Mr} K={Kr}", ms, "hbm", (2.0 + wr) * Mr * Kr, kern))
         del hs
         torch.cuda.empty_cache()
 
-    # ------------------------------------------------ mixture of experts, int8 (decode-sized batches)
+    # ------------------------------------------------ moe: mixture of experts (decode-sized batches)
     if "moe" in legs:
         E, Nm, Km, top_k, BMm = 8, 28672, 4096, 2, 16     # Mixtral-8x7B-like gate+up projection
         g = torch.Generator(device=dev).manual_seed(7)
-        bm = torch.randint(-127, 128, (E, Nm, Km), dtype=torch.int8, device=dev, generator=g)
-        acm = torch.rand(E, Nm, device=dev, generator=g) * 0.01
-        for Mt in (16, 64):
-            am = torch.randint(-127, 128, (Mt, Km), dtype=torch.int8, device=dev, generator=g)
-            arm = torch.rand(Mt, device=dev, generator=g).half()
+
+        def routing(Mt):
             tw, tid = torch.topk(torch.softmax(torch.randn(Mt, E, generator=torch.Generator().manual_seed(8)), -1), top_k)
             sid, eid, used = workloads.moe_align_block_size(tid, BMm, E)
             active = len(set(tid.flatten().tolist()))
-            tw, tid, sid, eid, used = (t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used))
+            return [t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used)] + [active]
+
+        bm = torch.randint(-127, 128, (E, Nm, Km), dtype=torch.int8, device=dev, generator=g)
+        acm = torch.rand(E, Nm, device=dev, generator=g) * 9e-3 + 1e-3
+        for Mt in (16, 64):
+            xm = workloads.activations(Mt, Km, torch.float16, seed=72, outlier_frac=0.01).to(dev)
+            am = torch.empty(Mt, Km, dtype=torch.int8, device=dev)
+            arm = torch.empty(Mt, dtype=torch.float16, device=dev)
+            launchers.hip_dynamic_quantize(am, xm, arm)
+            tw, tid, sid, eid, used, active = routing(Mt)
             cm = torch.empty(Mt, top_k, Nm, dtype=torch.bfloat16, device=dev)
             f = lambda i: flashnn_amd.fused_moe_a8w8_forward(am, bm, cm, arm, acm, tw, tid, sid, eid, used, True, top_k, BMm)
-            for i in range(3):
-                f(i)
-            ms = _events_ms(f, 20, torch)
-            mb_ = float(active) * Nm * Km + 2.0 * Mt * top_k * Nm      # weights of the experts in use + output
-            secondary.append({"workload": f"fused_moe_a8w8 tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={BMm} "
-                                          f"({active} experts in use)", "kernel": "gemm_a8w8_panel_kernel",
-                              "us_per_launch": round(ms * 1e3, 2),
-                              "roofline": {"bound": "hbm", "achieved": round(mb_ / (ms * 1e-3) / 1e9, 1),
-                                           "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                           "frac": round(mb_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+            kern = kernel_of(f)
+            ms, _ = _timed(f, 20, torch)
+            secondary.append(_entry(f"fused_moe_a8w8 tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={BMm} "
+                                    f"({active} experts in use)", ms, "hbm",
+                                    float(active) * Nm * Km + 2.0 * Mt * top_k * Nm, kern))
         del bm
         torch.cuda.empty_cache()
-        # int4 expert weights, per-channel scales, same layer
+        # int4 expert weights of the same layer: per-channel tables, then tables per group of 128 ([E, N, K/128])
         N2 = Nm // 2
         b4 = torch.randint(-128, 128, (E, N2, Km), dtype=torch.int8, device=dev, generator=g)
-        sc4 = (torch.rand(E, Nm, device=dev, generator=g) * 0.01).to(torch.bfloat16)
-        zp4m = torch.randint(-3, 4, (E, Nm), device=dev, generator=g).to(torch.bfloat16)
-        for Mt in (16, 64):
-            a4 = torch.randn(Mt, Km, device=dev, generator=g).to(torch.bfloat16)
-            tw, tid = torch.topk(torch.softmax(torch.randn(Mt, E, generator=torch.Generator().manual_seed(8)), -1), top_k)
-            sid, eid, used = workloads.moe_align_block_size(tid, BMm, E)
-            active = len(set(tid.flatten().tolist()))
-            tw, tid, sid, eid, used = (t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used))
-            cm = torch.empty(Mt, top_k, Nm, dtype=torch.bfloat16, device=dev)
-            f = lambda i: flashnn_amd.fused_moe_a16w4_forward(a4, b4, cm, sc4, zp4m, tw, tid, sid, eid, used, True, top_k, BMm)
-            for i in range(3):
-                f(i)
-            ms = _events_ms(f, 20, torch)
-            mb_ = float(active) * N2 * Km + 2.0 * Mt * top_k * Nm
-            secondary.append({"workload": f"fused_moe_a16w4 per-channel tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} "
-                                          f"block={BMm} ({active} experts in use)", "kernel": "gemm_wo_panel_kernel",
-                              "us_per_launch": round(ms * 1e3, 2),
-                              "roofline": {"bound": "hbm", "achieved": round(mb_ / (ms * 1e-3) / 1e9, 1),
-                                           "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                           "frac": round(mb_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
-        # ... and with scales and zero points per group of 128, [E, N, K/128] as the reference lays them out
-        sc4g = (torch.rand(E, Nm, Km // 128, device=dev, generator=g) * 0.01).to(torch.bfloat16)
-        zp4g = torch.randint(-3, 4, (E, Nm, Km // 128), device=dev, generator=g).to(torch.bfloat16)
-        a4 = torch.randn(16, Km, device=dev, generator=g).to(torch.bfloat16)
-        tw, tid = torch.topk(torch.softmax(torch.randn(16, E, generator=torch.Generator().manual_seed(8)), -1), top_k)
-        sid, eid, used = workloads.moe_align_block_size(tid, BMm, E)
-        active = len(set(tid.flatten().tolist()))
-        tw, tid, sid, eid, used = (t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used))
-        cm = torch.empty(16, top_k, Nm, dtype=torch.bfloat16, device=dev)
-        f = lambda i: flashnn_amd.fused_moe_a16w4_forward(a4, b4, cm, sc4g, zp4g, tw, tid, sid, eid, used, True, top_k, BMm)
-        for i in range(3):
-            f(i)
-        ms = _events_ms(f, 20, torch)
-        mb_ = float(active) * (N2 * Km + 4.0 * Nm * (Km // 128)) + 2.0 * 16 * top_k * Nm
-        secondary.append({"workload": f"fused_moe_a16w4 group 128 tokens=16 E={E} top_k={top_k} K={Km} N={Nm} "
-                                      f"block={BMm} ({active} experts in use)", "kernel": "gemm_wo_panel_kernel",
-                          "us_per_launch": round(ms * 1e3, 2),
-                          "roofline": {"bound": "hbm", "achieved": round(mb_ / (ms * 1e-3) / 1e9, 1),
-                                       "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                       "frac": round(mb_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None}})
+        for label, tshape, Mts in (("per-channel", (E, Nm), (16, 64)), ("group 128", (E, Nm, Km // 128), (16,))):
+            sc4 = (torch.rand(*tshape, device=dev, generator=g) * 9e-3 + 1e-3).to(torch.bfloat16)
+            zp4m = torch.randint(-3, 4, tshape, device=dev, generator=g).to(torch.bfloat16)
+            for Mt in Mts:
+                a4 = workloads.activations(Mt, Km, torch.bfloat16, seed=73).to(dev)
+                tw, tid, sid, eid, used, active = routing(Mt)
+                cm = torch.empty(Mt, top_k, Nm, dtype=torch.bfloat16, device=dev)
+                f = lambda i: flashnn_amd.fused_moe_a16w4_forward(a4, b4, cm, sc4, zp4m, tw, tid, sid, eid, used, True,
+                                                                  top_k, BMm)
+                kern = kernel_of(f)
+                ms, _ = _timed(f, 20, torch)
+                tables = 4.0 * Nm * (Km // 128) if len(tshape) == 3 else 4.0 * Nm
+                secondary.append(_entry(f"fused_moe_a16w4 {label} tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} "
+                                        f"block={BMm} ({active} experts in use)", ms, "hbm",
+                                        float(active) * (N2 * Km + tables) + 2.0 * Mt * top_k * Nm, kern))
         del b4
         torch.cuda.empty_cache()
 
@@ -379,10 +443,11 @@ def main():
     if not args.no_cpu:
         from oracle import torch_path as T
         cores = torch.get_num_threads()
+        Mq, Kq, Nq = primary["M"], primary["K"], primary["N"]
 
         def cpu_step():
             q, s = T.dynamic_quantize(x_cpu)
-            return T.gemm_a8w8(q, w_cpu, s.float(), ws_cpu, torch.bfloat16)
+            return T.gemm_a8w8(q, w_qkv, s.float(), ws_qkv, torch.bfloat16)
 
         cpu_step()
         ts = []
@@ -395,22 +460,31 @@ def main():
         t0 = time.perf_counter()
         T.gemm_weight_only(act1, packed, scale4, None, zp4, torch.bfloat16)
         t_cpu4 = time.perf_counter() - t0
-        cpu_baseline = {"value": round(ops / t_cpu / 1e12, 4), "unit": "TOPS", "cores": cores, "kind": "port",
-                        "sample": f"the whole step (dynamic quant + fp32-matmul A8W8, M={M} K={K} N={N}) through "
+        # the reference's own CPU-runnable case (c1)
+        t0 = time.perf_counter()
+        for _ in range(5):
+            q, s = T.dynamic_quantize(x1_cpu)
+            T.gemm_a8w8(q, w1_cpu, s.float(), ws1_cpu, torch.float16)
+        t_cpu1 = (time.perf_counter() - t0) / 5
+        cpu_baseline = {"value": round(primary["ops"] / t_cpu / 1e12, 4), "unit": "TOPS", "cores": cores, "kind": "port",
+                        "sample": f"the whole step (dynamic quant + fp32-matmul A8W8, M={Mq} K={Kq} N={Nq}) through "
                                   f"the torch-op restatement of the reference's CPU path, median of 3 runs "
                                   f"({t_cpu * 1e3:.0f} ms each)",
+                        "c1_m16_ms": round(t_cpu1 * 1e3, 2),
                         "a16w4_decode_m1_ms": round(t_cpu4 * 1e3, 1),
                         "a16w4_decode_m1_weight_GBps": round((N4 * K4 / 2 + 4 * (K4 // 128) * N4) / t_cpu4 / 1e9, 3)}
 
+    value = primary["ops"] / (primary["ms_step"] * 1e-3) / 1e12
     result = {
         "metric": "a8w8_int8_tops_m2048", "value": round(value, 2), "unit": "TOPS", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "preroll_steps": preroll_steps, "ms_per_step": round(ms_step, 5),
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(primary["ms_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": "DynamicQuant(fp16 [2048,4096], 1% outlier channels x20) + A8W8 GEMM "
                                "M=2048 K=4096 N=12288, int8 per-channel weights, bf16 out (Llama-7B QKV prefill)",
-                   "rotating_operand_sets": nset, "device": props.name, "cus": props.multi_processor_count,
-                   "host_wall_ms_per_step": round(wall_ms, 5)},
+                   "kernels": [primary["k_quant"], primary["k_gemm"]],
+                   "rotating_operand_sets": primary["nset"], "device": props.name, "cus": props.multi_processor_count,
+                   "host_wall_ms_per_step": round(primary["wall_ms"], 5)},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "secondary": secondary,
     }
     print(json.dumps(result))
