@@ -325,22 +325,31 @@ def main():
             del w8
         torch.cuda.empty_cache()
 
-    # ----------------------------- g64: the reference test's A16W4 shape, M = 3, N = 1024, K = 4096, group 64
+    # ----------- g64: the reference test's weight-only shape, M = 3, N = 1024, K = 4096, group 64, fp16, int8 and int4
     if "g64" in legs:
         Mg, Ng, Kg = 3, 1024, 4096
-        pg, sg, zg, _, _ = workloads.int4_group_weights(Ng, Kg, 64, seed=64)
-        pgs = rotating(pg.to(dev), at_most=160)
-        n = len(pgs)
-        sgs = [sg.to(dev).clone() for _ in range(n)]
-        zgs = [zg.to(dev).clone() for _ in range(n)]
+        gg = torch.Generator().manual_seed(64)
         act = workloads.activations(Mg, Kg, torch.float16, seed=65).to(dev)
         og = torch.empty(Mg, Ng, dtype=torch.float16, device=dev)
-        f = lambda i: launchers.hip_gemm_a16w4_forward(og, act, pgs[i % n], sgs[i % n], None, zgs[i % n])
-        kern = kernel_of(f)
-        ms, _ = _timed(f, iters, torch)
-        secondary.append(_entry(f"g64 a16w4 group 64 M={Mg} K={Kg} N={Ng} fp16 (the reference test's shape)", ms, "hbm",
-                                Ng * Kg / 2 + 4.0 * (Kg // 64) * Ng + 2.0 * Mg * Kg + 2.0 * Mg * Ng, kern))
-        del pgs, sgs, zgs
+        for bits in (8, 4):
+            if bits == 8:
+                qg = torch.randint(-127, 128, (Ng, Kg), generator=gg, dtype=torch.int8)
+                sg = torch.empty(Kg // 64, Ng).uniform_(1e-3, 1e-2, generator=gg).half()
+                zg = torch.randint(-8, 9, (Kg // 64, Ng), generator=gg).half()
+                fwd = launchers.hip_gemm_a16w8_forward
+            else:
+                qg, sg, zg, _, _ = workloads.int4_group_weights(Ng, Kg, 64, seed=64)
+                fwd = launchers.hip_gemm_a16w4_forward
+            qgs = rotating(qg.to(dev), at_most=160)
+            n = len(qgs)
+            sgs = [sg.to(dev).clone() for _ in range(n)]
+            zgs = [zg.to(dev).clone() for _ in range(n)]
+            f = lambda i: fwd(og, act, qgs[i % n], sgs[i % n], None, zgs[i % n])
+            kern = kernel_of(f)
+            ms, _ = _timed(f, iters, torch)
+            secondary.append(_entry(f"g64 a16w{bits} group 64 M={Mg} K={Kg} N={Ng} fp16 (the reference test's shape)", ms,
+                                    "hbm", Ng * Kg * bits / 8 + 4.0 * (Kg // 64) * Ng + 2.0 * Mg * Kg + 2.0 * Mg * Ng, kern))
+            del qgs, sgs, zgs
         torch.cuda.empty_cache()
 
     # --------------------- splitk: A8W8 shapes whose K the library splits over workgroups, and the unsplit kernel

@@ -450,9 +450,14 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_kernel(const Wo
 // REFQ (1, or 2 with zero points; fp16 activations, per-channel fp16 scales and zero points): every weight is dequantised and rounded
 // to fp16 as the reference's torch path does before the dot product (ref_dq_f16), and the scale tables, the
 // MFMAs against ones and the fold are not needed.
+// REFQ 3 (4 with zero points): the same with fp16 tables per group of 32 or 64 values of K.  A lane's 16
+// weights of a step lie in one group; its scale and zero point come from an LDS table of (scale, zero point)
+// pairs, [K / group][channels of the tile], one 4-byte read per channel and step.
 template <int WBITS, int ADT, bool G128, int MP, int CH, bool FULL, int REFQ = 0>
 __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(const WoArgs p) {
-    static_assert(!REFQ || (ADT == FNN_F16 && !G128), "reference rounding: fp16, per-channel");
+    static_assert(!REFQ || (ADT == FNN_F16 && !G128), "reference rounding: fp16, tables per channel or per small group");
+    constexpr bool RQG = REFQ >= 3;              // tables per group of 32 or 64
+    constexpr bool RQZ = REFQ == 2 || REFQ == 4;
     typedef MfmaT<ADT> MT;
     constexpr int NH = WBITS == 4 ? 2 : 1;
     constexpr int NC = 8 * NH;
@@ -484,9 +489,10 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     const int nblk = (steps + 7) / 8;
     const int s_begin = (nblk * wave / kDecWaves) * 8;
     const int s_end = min((nblk * (wave + 1) / kDecWaves) * 8, steps);
-    const int ngroups = G128 ? steps : 1;
+    const int ngroups = G128 ? steps : RQG ? p.K / p.group : 1;
 
     // LDS: [zeros][scale ngroups*NC f32][zoff ngroups*NC f32][red 4*NH*4*64 f32][acts]
+    // (RQG: the first table holds the (scale, zero point) pairs of fp16 instead, the second is unused)
     float* s_lds = (float*)(smem + ZERO_BYTES);
     float* z_lds = s_lds + ngroups * NC;
     float* red = z_lds + ngroups * NC;
@@ -503,7 +509,7 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     // REFQ: the scale and zero point of this lane's weight row (two channels per row with int4 weights),
     // requested ahead of the weights: loads return in order, and the first conversion needs them
     uint32_t rq_sb[NH], rq_zb[NH];
-    if constexpr (REFQ) {
+    if constexpr (REFQ == 1 || REFQ == 2) {
 #pragma unroll
         for (int h = 0; h < NH; ++h) {
             const int n = min(n0 + j7 * NH + h, p.N - 1);
@@ -519,7 +525,7 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     }
     v2h rq_s[NH], rq_z[NH];
     const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
-    if constexpr (REFQ) {
+    if constexpr (REFQ == 1 || REFQ == 2) {
 #pragma unroll
         for (int h = 0; h < NH; ++h) { rq_s[h] = pair_of_f16_bits(rq_sb[h]); rq_z[h] = pair_of_f16_bits(rq_zb[h]); }
     }
@@ -541,6 +547,26 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     if constexpr (!REFQ) {
         if (p.scale_dtype == FNN_F16) fill_scales_lds<FNN_F16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
         else fill_scales_lds<FNN_BF16, NC>(s_lds, z_lds, p, n0, ngroups, c_off, threadIdx.x, NT);
+    }
+    if constexpr (RQG) {
+        // (scale | zero point << 16) of group g, channel c at word g * NC + c; loads in batches of four
+        uint32_t* const tab = (uint32_t*)s_lds;
+        const int total = ngroups * NC;
+        for (int e0 = 0; e0 < total; e0 += 4 * NT) {
+            uint32_t sv[4], zv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int e = min(e0 + u * NT + (int)threadIdx.x, total - 1);
+                const int64_t idx = (int64_t)(e / NC) * p.N + min(n0 + e % NC, p.N - 1);
+                sv[u] = ((const uint16_t*)p.scale)[idx];
+                zv[u] = RQZ ? (uint32_t)((const uint16_t*)p.zp)[idx] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int e = e0 + u * NT + threadIdx.x;
+                if (e < total) tab[e] = sv[u] | (zv[u] << 16);
+            }
+        }
     }
     {
         for (int m = 0; m < p.M; ++m) {
@@ -575,6 +601,13 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     const uint32_t a_zero = 0;
     uint32_t sz_addr = (uint32_t)((const char*)(s_lds + (s_begin + gslot) * (G128 ? NC : 0) + NH * 4 * (lg & 1)) - smem);
     const uint32_t z_delta = (uint32_t)(ngroups * NC * 4);
+
+    // RQG: word address of this lane's table entries at step 0 (group of its K segment, its weight row's
+    // channels); a step adds 128 / group groups
+    const int rqg_gps = RQG ? 128 / p.group : 0;
+    const uint32_t rqg_base = RQG ? (uint32_t)((const char*)s_lds - smem) +
+                                        (uint32_t)(((lg * 32 + half * 16) / (RQG ? p.group : 1)) * NC + j7 * NH) * 4u : 0u;
+    const uint32_t rqg_step = (uint32_t)(rqg_gps * NC * 4);
 
     v4f outv[NH], accg[NH], asum;
 #pragma unroll
@@ -621,6 +654,14 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
                 const v4u a0 = *(const v4u*)(smem + aa);
                 const v4u a1 = *(const v4u*)(smem + aa + 16);
                 const bool first = G128 ? (i % GS == 0) : (step == s_begin);
+                if constexpr (RQG) {
+#pragma unroll
+                    for (int h = 0; h < NH; ++h) {
+                        const uint32_t t = *(const uint32_t*)(smem + rqg_base + (uint32_t)step * rqg_step + h * 4);
+                        rq_s[h] = pair_of_f16_bits(t);
+                        rq_z[h] = pair_of_f16_bits(t >> 16);
+                    }
+                }
                 if constexpr (WBITS == 4) {
                     v4u e0, e1, o0, o1;
                     convert_w4<ADT>(w, e0, e1, o0, o1);
@@ -628,10 +669,10 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
                     // in the same registers
                     if (i + UN < CH) wq[i % UN] = load_w(step + UN);
                     if constexpr (REFQ) {
-                        e0 = ref_dq_f16<REFQ == 2>(e0, rq_c, rq_z[0], rq_s[0]);
-                        e1 = ref_dq_f16<REFQ == 2>(e1, rq_c, rq_z[0], rq_s[0]);
-                        o0 = ref_dq_f16<REFQ == 2>(o0, rq_c, rq_z[NH - 1], rq_s[NH - 1]);
-                        o1 = ref_dq_f16<REFQ == 2>(o1, rq_c, rq_z[NH - 1], rq_s[NH - 1]);
+                        e0 = ref_dq_f16<RQZ>(e0, rq_c, rq_z[0], rq_s[0]);
+                        e1 = ref_dq_f16<RQZ>(e1, rq_c, rq_z[0], rq_s[0]);
+                        o0 = ref_dq_f16<RQZ>(o0, rq_c, rq_z[NH - 1], rq_s[NH - 1]);
+                        o1 = ref_dq_f16<RQZ>(o1, rq_c, rq_z[NH - 1], rq_s[NH - 1]);
                     }
                     accg[0] = MT::mma(e0, a0, first ? zero4 : accg[0]);
                     accg[1] = MT::mma(o0, a0, first ? zero4 : accg[1]);
@@ -644,8 +685,8 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
                     convert_w8<ADT>(w, s0, s1);
                     if (i + UN < CH) wq[i % UN] = load_w(step + UN);
                     if constexpr (REFQ) {
-                        s0 = ref_dq_f16<REFQ == 2>(s0, rq_c, rq_z[0], rq_s[0]);
-                        s1 = ref_dq_f16<REFQ == 2>(s1, rq_c, rq_z[0], rq_s[0]);
+                        s0 = ref_dq_f16<RQZ>(s0, rq_c, rq_z[0], rq_s[0]);
+                        s1 = ref_dq_f16<RQZ>(s1, rq_c, rq_z[0], rq_s[0]);
                     }
                     accg[0] = MT::mma(s0, a0, first ? zero4 : accg[0]);
                     if constexpr (!REFQ) asum = MT::mma(ones, a0, first ? zero4 : asum);
@@ -1274,7 +1315,10 @@ template <int WBITS, int ADT>
 static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
     constexpr int NH = WBITS == 4 ? 2 : 1;
     if (p.M > 8 || p.K % 128 != 0) return false;
-    if (p.group > 0 && (p.group % 128 != 0)) return false;
+    // groups of 32 or 64: only with fp16 activations and fp16 tables (every weight dequantised to fp16 first)
+    const bool small_groups = (p.group == 32 || p.group == 64) && ADT == FNN_F16 && p.scale_dtype == FNN_F16 &&
+                              (!p.zp || p.zp_dtype == FNN_F16);
+    if (p.group > 0 && p.group % 128 != 0 && !small_groups) return false;
     const int ngroups = p.group > 0 ? p.K / p.group : 1;
     const size_t fixed = (size_t)ngroups * 8 * NH * 8 + (size_t)kDecWaves * NH * 4 * 64 * 4;
     if (fixed > 40 * 1024) return false;
@@ -1373,7 +1417,8 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
         }
     }
     if (gemv_only) return false;
-    if (tables16 && act_lds && (p.group == 0 || p.group == 128)) {
+    // (the small-group tables are read element by element: any N, any alignment)
+    if (act_lds && (small_groups || (tables16 && (p.group == 0 || p.group == 128)))) {
         const int steps = p.K / 128;
         const bool full16 = steps % (kDecWaves * 16) == 0, full8 = steps % (kDecWaves * 8) == 0;
         const size_t smem = fixed + act_bytes + 16 * 256 + 32;
@@ -1388,8 +1433,10 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
         // fp16 activations with per-channel fp16 scales: the reference's own per-weight rounding
         bool refq = false;
         if constexpr (ADT == FNN_F16) {
-            refq = p.group == 0 && p.scale_dtype == FNN_F16;
-            if (refq && p.zp) FNN_DEC(false, 8, 2);
+            refq = (p.group == 0 && p.scale_dtype == FNN_F16) || small_groups;
+            if (small_groups && p.zp) FNN_DEC(false, 8, 4);
+            else if (small_groups) FNN_DEC(false, 8, 3);
+            else if (refq && p.zp) FNN_DEC(false, 8, 2);
             else if (refq) FNN_DEC(false, 8, 1);
         }
         if (refq) {}
@@ -1401,6 +1448,7 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
 #undef FNN_DEC
         return true;
     }
+    if (small_groups) return false;      // the kernel below walks groups of whole 128-value steps
     const size_t smem = fixed + (act_lds ? act_bytes : 0);
     if (smem > 64 * 1024) return false;
     note_kernel("gemm_wo_decode_kernel", WBITS, p.group, act_lds);
@@ -1416,10 +1464,14 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
 
 template <int WBITS, int ADT>
 static void dispatch_wo(WoArgs& p, hipStream_t st) {
-    const bool fast = p.K % 64 == 0 && (p.group == 0 || p.group % 64 == 0) && p.ldw % 16 == 0 &&
-                      p.lda % 8 == 0 && ((uintptr_t)p.qw % 16) == 0 && ((uintptr_t)p.act % 16) == 0;
+    const bool aligned = p.K % 64 == 0 && p.ldw % 16 == 0 && p.lda % 8 == 0 && ((uintptr_t)p.qw % 16) == 0 &&
+                         ((uintptr_t)p.act % 16) == 0;
+    const bool fast = aligned && (p.group == 0 || p.group % 64 == 0);
     // per-channel scales with K a multiple of 32 only: the panel kernel handles the partial last slab
     if (p.group == 0 && p.K % 128 != 0 && launch_wo_panel(p, WBITS, ADT, st)) return;
+    // groups of 32: only the decode kernel that dequantises every weight takes them (the kernels below walk
+    // groups of 64 and more)
+    if (aligned && p.group == 32 && launch_decode<WBITS, ADT>(p, st, false)) return;
     if (!fast) {
         const int64_t total = (int64_t)p.M * p.N;
         note_kernel("gemm_wo_any_kernel", WBITS);

@@ -665,7 +665,20 @@ def test_weight_only_reference_test_shape():
         for with_zp in (False, True):
             for with_bias in (False, True):
                 case = _wo_inputs(3, 1024, 4096, group, 8, torch.float16, torch.float16, with_zp, with_bias, seed=9)
-                _wo_check(*case, group, 8, torch.float16)
+                _wo_check(*case, group, 8, torch.float16, strict=True)
+                assert _lib.last_kernel().startswith("gemm_wo_decode_lds_kernel" if group else "gemm_wo_panel_kernel(per-weight")
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("group", [32, 64])
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 4096), (3, 1024, 4096), (8, 520, 1152), (5, 4096, 2944), (2, 96, 128)])
+def test_weight_only_small_groups_decode(bits, group, M, N, K):
+    """Tables per group of 32 or 64 with fp16 activations and tables: every weight is dequantised and rounded to
+    fp16 as the reference's block dequantisation does, so the stated tolerance holds without exception."""
+    for with_zp in (False, True):
+        case = _wo_inputs(M, N, K, group, bits, torch.float16, torch.float16, with_zp, M == 3, seed=M + K)
+        _wo_check(*case, group, bits, torch.float16, strict=True)
+        assert _lib.last_kernel().startswith("gemm_wo_decode_lds_kernel")
 
 
 @pytest.mark.parametrize("bits", [8, 4])
