@@ -1554,12 +1554,6 @@ extern "C" int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const 
 // ------------------------------------------------------------------ mixture of experts, int4 weights
 namespace fnn {
 
-constexpr int FNN_I8 = 3;   // zero points may be integers
-
-__device__ __forceinline__ float load_zp_f32(const void* p, int64_t i, int dtype) {
-    return dtype == FNN_I8 ? (float)((const int8_t*)p)[i] : load_as_f32(p, i, dtype);
-}
-
 // Any shape, per-channel or grouped scales with any strides: one thread per output value.
 // out[t, n] = sum over K blocks g of scale[e, n, g] * sum_{k in g} act[t / top_k, k] * (nibble(e, n, k) - zp[e, n, g])
 template <int ADT>
@@ -1640,8 +1634,9 @@ extern "C" int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const 
     q.stride_scale_n = stride_scale_n; q.stride_scale_k = stride_scale_k;
     q.stride_zp_n = stride_zp_n; q.stride_zp_k = stride_zp_k;
     hipStream_t st = (hipStream_t)stream;
-    // the weight-streaming kernel takes per-channel scales and groups of 128 (launch_wo_panel_moe checks the layout)
-    const bool fast = (group == 0 || group == 128) && (!zero_points || zp_dtype != FNN_I8);
+    // the weight-streaming kernel takes per-channel scales (zero points of any type) and groups of 128 (zero points
+    // of the scales' type; launch_wo_panel_moe checks the layout)
+    const bool fast = group == 0 || (group == 128 && (!zero_points || zp_dtype != FNN_I8));
     const Call call(fn);
     if (!(fast && launch_wo_panel_moe(p, q, act_dtype, st))) {
         const dim3 grid((unsigned)EM, (unsigned)((2 * N + 255) / 256));

@@ -419,7 +419,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
 #pragma unroll
         for (int c = 0; c < NCL; ++c) {
             sc[c] = load_as_f32(p.scale, (MOE ? (int64_t)expert * q.stride_scale_be : 0) + n0 + c, p.scale_dtype);
-            zc[c] = c_off + (has_zp ? load_as_f32(p.zp, (MOE ? (int64_t)expert * q.stride_zp_be : 0) + n0 + c, p.zp_dtype)
+            zc[c] = c_off + (has_zp ? load_zp_f32(p.zp, (MOE ? (int64_t)expert * q.stride_zp_be : 0) + n0 + c, p.zp_dtype)
                                     : 0.f);
         }
 #pragma unroll

@@ -111,6 +111,12 @@ __device__ __forceinline__ v4u ref_dq_f16(v4u x, const v2h coff, const v2h zp, c
     return v4u{ref_dq_f16<ZP>(x[0], coff, zp, s), ref_dq_f16<ZP>(x[1], coff, zp, s), ref_dq_f16<ZP>(x[2], coff, zp, s),
                ref_dq_f16<ZP>(x[3], coff, zp, s)};
 }
+constexpr int FNN_I8 = 3;   // type code of int8 zero points (mixture-of-experts entry point only)
+
+__device__ __forceinline__ float load_zp_f32(const void* p, int64_t i, int dtype) {
+    return dtype == FNN_I8 ? (float)((const int8_t*)p)[i] : load_as_f32(p, i, dtype);
+}
+
 // an fp16 bit pattern in both halves of a packed pair
 __device__ __forceinline__ v2h pair_of_f16_bits(uint32_t h) {
     return __builtin_bit_cast(v2h, (h & 0xFFFFu) * 0x10001u);

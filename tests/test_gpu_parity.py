@@ -577,6 +577,8 @@ def test_fused_moe_a16w4_close(shape, group, zp_kind, act_ty):
     flashnn_amd.fused_moe_a16w4_forward(a.to(DEV), packed.to(DEV), cd, scale.to(DEV), None if zp is None else zp.to(DEV),
                                         tw.to(DEV), ids.to(DEV), s.to(DEV), e.to(DEV), used.to(DEV), True, top_k, BM)
     np.testing.assert_allclose(cd.float().cpu().reshape(M * top_k, 2 * N2).numpy(), want, rtol=RTOL, atol=ATOL)
+    if group == 0 and K >= 1024 and K % 32 == 0 and (2 * N2) % 32 == 0 and BM % 16 == 0:
+        assert _lib.last_kernel().startswith("gemm_wo_panel_kernel(moe)")      # int8 zero points included
     # the same list cut after its first block: every other routed row keeps the fill value
     cd2 = c.to(DEV)
     flashnn_amd.fused_moe_a16w4_forward(a.to(DEV), packed.to(DEV), cd2, scale.to(DEV), None if zp is None else zp.to(DEV),
