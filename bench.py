@@ -386,7 +386,8 @@ def main():
         f = lambda i: norm(hs[i % 3])
         kern = kernel_of(f)
         ms, _ = _timed(f, 50, torch)
-        secondary.append(_entry(f"rmsnorm_dquant bf16 M={Mr} K={Kr}", ms, "hbm", 3.0 * Mr * Kr + 4.0 * Kr + 2.0 * Mr, kern))
+        secondary.append(_entry(f"rmsnorm_dquant bf16 M={Mr} K={Kr}", ms, "hbm", 3.0 * Mr * Kr + 4.0 * Kr + 2.0 * Mr, kern,
+                                "rmsnorm_dquant M=8192 K=8192"))
         # the layers one step before the path, same matrix
         for name, mod, wr in (("rmsnorm", flashnn_amd.RMSNorm(Kr), 2.0), ("layernorm", flashnn_amd.LayerNorm(Kr), 2.0),
                               ("layernorm_dquant", flashnn_amd.LayernormDquant(Kr), 1.0)):
