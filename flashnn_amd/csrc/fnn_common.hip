@@ -74,7 +74,7 @@ void note_kernel(const char* name, int a, int b, int c) {
 
 }  // namespace fnn
 
-extern "C" int fnn_version(void) { return 1; }
+extern "C" int fnn_version(void) { return 2; }
 extern "C" const char* fnn_last_error(void) { return fnn::g_err; }
 extern "C" const char* fnn_last_kernel(void) {
     fnn::format_note(fnn::g_note, fnn::g_note_text, sizeof(fnn::g_note_text));

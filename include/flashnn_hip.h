@@ -43,7 +43,7 @@ enum fnn_dtype { FNN_F16 = 0, FNN_BF16 = 1, FNN_F32 = 2 };
 
 enum fnn_status { FNN_OK = 0, FNN_ERR_ARG = -1, FNN_ERR_UNSUPPORTED = -2, FNN_ERR_HIP = -3 };
 
-/* ABI version of this header (bumped on any signature change). */
+/* ABI version of this header (bumped on any signature change): 2 since fnn_gemm_a8w8_tiled names the waves and the workspace entry points exist. */
 int fnn_version(void);
 
 /* Message describing the last failure on the calling thread ("" if none). */

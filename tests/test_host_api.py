@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol(hip_lib):
     for name in declared:
         assert hasattr(hip_lib, name), f"{name} is declared in include/flashnn_hip.h but not exported"
     assert set(_lib.exported_symbols()) == set(declared)
-    assert hip_lib.fnn_version() == 1
+    assert hip_lib.fnn_version() == 2
 
 
 def test_argument_errors_are_reported_without_a_gpu(hip_lib):
