@@ -44,7 +44,8 @@ ALL_LEGS = ("c1", "c2", "c3", "c4", "c5", "g64", "splitk", "rows", "moe")
 def _timed(fn, iters, torch, preroll_s=0.04):
     """(average milliseconds by HIP events on the current stream, average host wall milliseconds) of
     fn(i) over `iters` back-to-back calls.  An untimed pre-roll of the same call comes first and is in
-    neither figure: host-side input generation between the measurements leaves the device idle long enough
+    neither figure (its length in calls is kept in _timed.preroll_calls): host-side input generation between
+    the measurements leaves the device idle long enough
     for its clocks to drop, and a hundred launches of a 20 us kernel would be over before they are back."""
     t0 = time.perf_counter()
     k = 0
@@ -63,6 +64,7 @@ def _timed(fn, iters, torch, preroll_s=0.04):
     end.record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - w0) * 1e3 / iters
+    _timed.preroll_calls = k
     return start.elapsed_time(end) / iters, wall
 
 
@@ -182,9 +184,11 @@ def main():
                 step(i)
             torch.cuda.synchronize()
             ms_step, wall_ms = _timed(step, args.steps, torch, preroll_s=0.06)
+            preroll_steps = _timed.preroll_calls
             ms_gemm, _ = _timed(gemm_only, args.steps, torch)
             ms_quant, _ = _timed(quant_only, args.steps, torch)
             primary = dict(M=M, K=K, N=N, ops=ops, ms_step=ms_step, wall_ms=wall_ms, ms_gemm=ms_gemm, nset=n,
+                           preroll_steps=preroll_steps,
                            k_gemm=k_gemm, k_quant=k_quant)
             if "rows" in legs:
                 secondary.append(_entry(f"dynamic_quant fp16 M={M} K={K}", ms_quant, "hbm", 3.0 * M * K + 2.0 * M,
@@ -487,7 +491,7 @@ def main():
     value = primary["ops"] / (primary["ms_step"] * 1e-3) / 1e12
     result = {
         "metric": "a8w8_int8_tops_m2048", "value": round(value, 2), "unit": "TOPS", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(primary["ms_step"], 5),
+        "steps": args.steps, "warmup": args.warmup, "preroll_steps": primary["preroll_steps"], "ms_per_step": round(primary["ms_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": "DynamicQuant(fp16 [2048,4096], 1% outlier channels x20) + A8W8 GEMM "

@@ -1634,9 +1634,9 @@ extern "C" int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const 
     q.stride_scale_n = stride_scale_n; q.stride_scale_k = stride_scale_k;
     q.stride_zp_n = stride_zp_n; q.stride_zp_k = stride_zp_k;
     hipStream_t st = (hipStream_t)stream;
-    // the weight-streaming kernel takes per-channel scales (zero points of any type) and groups of 128 (zero points
-    // of the scales' type; launch_wo_panel_moe checks the layout)
-    const bool fast = group == 0 || (group == 128 && (!zero_points || zp_dtype != FNN_I8));
+    // the weight-streaming kernel takes per-channel tables and groups of 128 (launch_wo_panel_moe checks the layout
+    // and the types)
+    const bool fast = group == 0 || group == 128;
     const Call call(fn);
     if (!(fast && launch_wo_panel_moe(p, q, act_dtype, st))) {
         const dim3 grid((unsigned)EM, (unsigned)((2 * N + 255) / 256));

@@ -387,10 +387,25 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         const uint16_t* sg = (const uint16_t*)p.scale + (int64_t)expert * q.stride_scale_be + (int64_t)ch0 * G;
         const uint16_t* zg = p.zp ? (const uint16_t*)p.zp + (int64_t)expert * q.stride_zp_be + (int64_t)ch0 * G : sg;
         const int per_ch = G / 8;
+        // int8 zero points (one byte per group) are widened to the scales' type on their way into the table
+        const bool zp_i8 = p.zp && p.zp_dtype == FNN_I8;
+        const int8_t* zg8 = zp_i8 ? (const int8_t*)p.zp + (int64_t)expert * q.stride_zp_be + (int64_t)ch0 * G : nullptr;
         for (int v = threadIdx.x; v < CHW * per_ch; v += 512) {
             const int ch = v / per_ch, g8 = v % per_ch;
             const v4u a = *(const v4u*)(sg + (int64_t)ch * G + g8 * 8);
-            const v4u b = *(const v4u*)(zg + (int64_t)ch * G + g8 * 8);
+            v4u b;
+            if (zp_i8) {
+                const v2u raw = *(const v2u*)(zg8 + (int64_t)ch * G + g8 * 8);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float lo = (float)(int8_t)(raw[i >> 1] >> (16 * (i & 1)));
+                    const float hi = (float)(int8_t)(raw[i >> 1] >> (16 * (i & 1) + 8));
+                    b[i] = SDT == FNN_F16 ? (f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16))
+                                          : (f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16));
+                }
+            } else {
+                b = *(const v4u*)(zg + (int64_t)ch * G + g8 * 8);
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 tabs[(g8 * 8 + i) * CHW + ch] = (uint16_t)(a[i >> 1] >> (16 * (i & 1)));
@@ -604,8 +619,8 @@ static bool launch_panel_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
         // tables [expert][channel][group] of one 16-bit type, every channel's groups contiguous and 16-byte aligned
         const bool ok = p.K % 128 == 0 && G % 8 == 0 && G <= 64 && is16(p.scale_dtype) && q.stride_scale_k == 1 &&
                         q.stride_scale_n == G && q.stride_scale_be % 8 == 0 && ((uintptr_t)p.scale % 16) == 0 &&
-                        (!p.zp || (p.zp_dtype == p.scale_dtype && q.stride_zp_k == 1 && q.stride_zp_n == G &&
-                                   q.stride_zp_be % 8 == 0 && ((uintptr_t)p.zp % 16) == 0));
+                        (!p.zp || ((p.zp_dtype == p.scale_dtype || p.zp_dtype == FNN_I8) && q.stride_zp_k == 1 &&
+                                   q.stride_zp_n == G && q.stride_zp_be % 8 == 0 && ((uintptr_t)p.zp % 16) == 0));
         if (!ok) return false;
     } else if (q.stride_scale_n != 1 || (p.zp && q.stride_zp_n != 1)) {
         return false;

@@ -279,7 +279,7 @@ def test_a8w8_prefill_full_size(name):
 _SWEEP_B = {}
 
 
-@pytest.mark.parametrize("M", [1, 10, 40, 764, 2048])
+@pytest.mark.parametrize("M", [1, 10, 40, 764, 2048, 4096, 8192])
 @pytest.mark.parametrize("nk", workloads.sharded_model_gemm_shapes())
 def test_a8w8_reference_sweep_shapes(nk, M):
     """The (N, K) pairs and row counts of the reference's A8W8 sweep, inputs drawn as its own test
@@ -544,7 +544,8 @@ def test_fused_moe_a8w8_bit_exact(shape, mul_w, out_ty):
 
 
 @pytest.mark.parametrize("act_ty", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("group,zp_kind", [(0, "float"), (0, None), (0, "int8"), (128, "float"), (128, None), (64, "int8")])
+@pytest.mark.parametrize("group,zp_kind", [(0, "float"), (0, None), (0, "int8"), (128, "float"), (128, None), (128, "int8"),
+                                           (64, "int8")])
 @pytest.mark.parametrize("shape", [
     # M, E, packed rows (half the output channels), K, top_k, BM
     (16, 8, 512, 1024, 2, 16), (33, 4, 1024, 2048, 2, 32), (70, 4, 528, 1152, 1, 64), (5, 16, 128, 4096, 4, 16),
@@ -577,7 +578,7 @@ def test_fused_moe_a16w4_close(shape, group, zp_kind, act_ty):
     flashnn_amd.fused_moe_a16w4_forward(a.to(DEV), packed.to(DEV), cd, scale.to(DEV), None if zp is None else zp.to(DEV),
                                         tw.to(DEV), ids.to(DEV), s.to(DEV), e.to(DEV), used.to(DEV), True, top_k, BM)
     np.testing.assert_allclose(cd.float().cpu().reshape(M * top_k, 2 * N2).numpy(), want, rtol=RTOL, atol=ATOL)
-    if group == 0 and K >= 1024 and K % 32 == 0 and (2 * N2) % 32 == 0 and BM % 16 == 0:
+    if (group == 0 and K >= 1024 and K % 32 == 0 or group == 128 and K % 1024 == 0) and (2 * N2) % 32 == 0 and BM % 16 == 0:
         assert _lib.last_kernel().startswith("gemm_wo_panel_kernel(moe)")      # int8 zero points included
     # the same list cut after its first block: every other routed row keeps the fill value
     cd2 = c.to(DEV)
