@@ -195,8 +195,8 @@ int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, const void* alp
  *            initialisation.  Calls that overlap in time (other streams, other threads) need a workspace
  *            each.
  * ws_bytes   its size.  fnn_gemm_a8w8_workspace_bytes(M, N, K) is what the call would use for a shape (0:
- *            the shape is not split); 16 MiB hold every shape.  With less than a shape needs the call
- *            runs unsplit.
+ *            the shape is not split); 16 MiB hold every shape.  With less than a shape needs (at least
+ *            the 4096 bytes of counters; or workspace = NULL with ws_bytes = 0) the call runs unsplit.
  */
 size_t fnn_gemm_a8w8_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int fnn_workspace_init(void* workspace, size_t ws_bytes, void* stream);
