@@ -916,8 +916,8 @@ static int check_args(const char* fn, const void* out, const void* a, const void
                   (long long)N, (long long)K, (long long)lda, (long long)ldb, (long long)ldc);
         return FNN_ERR_ARG;
     }
-    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) {
-        set_error("%s: shape too large", fn);
+    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30) || lda > (1LL << 30) || ldb > (1LL << 30)) {
+        set_error("%s: shape or row stride too large", fn);
         return FNN_ERR_UNSUPPORTED;
     }
     return FNN_OK;

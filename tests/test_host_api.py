@@ -192,6 +192,13 @@ def test_tiled_entry_rejects_unknown_tiles(hip_lib):
     assert rc == -1 and b"no such tile 256x256 with 4 waves" in hip_lib.fnn_last_error()
 
 
+def test_a8w8_rejects_row_strides_beyond_the_band_logic(hip_lib):
+    one = ctypes.c_void_p(4096)
+    null = ctypes.c_void_p(0)
+    rc = hip_lib.fnn_gemm_a8w8(one, one, one, one, one, 128, 128, 1024, 1 << 31, 1024, 128, 0, 0, 0, null)
+    assert rc == -2 and b"row stride too large" in hip_lib.fnn_last_error()
+
+
 def test_workspace_entries_reject_bad_arguments(hip_lib):
     one = ctypes.c_void_p(4096)
     odd = ctypes.c_void_p(4100)
