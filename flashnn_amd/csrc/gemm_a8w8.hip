@@ -670,25 +670,32 @@ struct TileChoice { int bm, bn; };
 // them exist, so a last round that is mostly empty is expensive; the columns are then cut where the first
 // launch ends on a full round.  Costs in 256x192 tile times: a 256x128 tile takes 128/192/0.85 of one, the
 // second launch about 0.08 (its launch gap and start-up).
-static int split_columns_192(int64_t M, int64_t N) {
+static int split_columns_192(int64_t M, int64_t N, double* cost_out = nullptr) {
     const int64_t tm = (M + 255) / 256, c = (N + 191) / 192;
     const double single = (double)((tm * c + 255) / 256);
     double best = single - 0.1;      // worth a second launch only from a tenth of a round
     int best_c1 = 0;
+    if (cost_out) *cost_out = single;
     for (int64_t c1 = c - 1; c1 >= 1 && c1 >= c - 64; --c1) {
         const int64_t rem = N - 192 * c1;
         const int64_t r1 = (tm * c1 + 255) / 256, r2 = (tm * ((rem + 127) / 128) + 255) / 256;
         const double cost = (double)r1 + (double)r2 * (128.0 / 192.0 / 0.85) + 0.08;
         if (cost < best) { best = cost; best_c1 = (int)c1; }
     }
+    if (cost_out && best_c1 > 0) *cost_out = best;
     return best_c1;
 }
 
 // Pick the tile whose last, partly filled round of workgroups costs least on 256 CUs.
 static TileChoice choose_tile(int64_t M, int64_t N) {
     static const struct { int bm, bn; double eff; } cand[] = {
-        {256, 192, 1.00}, {256, 128, 0.85}, {128, 128, 0.72}, {64, 128, 0.62}};
-    // eff = throughput per tile area relative to the 256x192 tile, measured with every round full.  It
+        {256, 192, 1.00}, {256, 256, 1.17}, {256, 128, 0.85}, {128, 128, 0.72}, {64, 128, 0.62}};
+    // eff = throughput per tile area relative to the 256x192 tile, measured with every round full.  The
+    // 256x256 tile (all 256 accumulator registers of a lane beside 256 others, all 160 KB of LDS: two a-stages,
+    // three b-stages) takes 1.13 of a 256x192 tile's time for 1.33 of its outputs - the kernel is bound by the
+    // operand bytes a CU takes in per slab, (rows + columns) * 128, and the square tile needs fewest per
+    // output - so it wins where its rounds are full (M = K = N = 8192: 390 -> 366 us, gate_up 154 -> 149 us)
+    // and loses where they are not (QKV: 384 tiles, 82 -> 94 us).  It
     // depends on the shape: the 256x128 tile reaches 1.0 at M=2048, K=4096, N=12288, 0.93 at N=22016 and
     // 0.74 at M=K=N=8192; 128x128 0.71 to 0.76; 64x128 0.64 to 0.67 (a 64x128 tile takes 0.55 to 0.6 of
     // the time of a 128x128 one, so it pays where it doubles the workgroups without adding a round).
@@ -706,7 +713,7 @@ static TileChoice choose_tile(int64_t M, int64_t N) {
     // replaces a smaller or narrower tile where it is cheaper.  It never replaces the 256x192 tile: the two
     // shapes where this pricing did so were slower on the box (116 -> 122 us, 118 -> 121 us).
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
-    if (t128 > 256 && !(c.bm == 256 && c.bn == 192)) {
+    if (t128 > 256 && !(c.bm == 256 && c.bn >= 192)) {
         const int64_t rem = t128 % 512;
         const double pair = ((double)(t128 / 512) + (rem == 0 ? 0.0 : rem <= 256 ? 0.64 : 1.0)) * 2.0 * 128 * 128 / 0.85;
         if (pair < best) c = {128, 128};
@@ -758,7 +765,7 @@ static void launch_mfma_split(A8W8Args& p, hipStream_t st) {
 static bool valid_tile(int bm, int bn, int waves) {
     if (bm == 0 && bn == 0) return waves == 0;
     if (waves == 0 || waves == 4)
-        return (bm == 256 && (bn == 192 || bn == 128)) || (bm == 128 && bn == 128) || (bm == 64 && bn == 128);
+        return (bm == 256 && (bn == 256 || bn == 192 || bn == 128)) || (bm == 128 && bn == 128) || (bm == 64 && bn == 128);
     if (waves == 8) return bm == 256 && (bn == 256 || bn == 192 || bn == 128);
     return false;
 }
@@ -771,6 +778,7 @@ static void launch_tile(A8W8Args& p, hipStream_t st, int bm, int bn, int waves) 
         else launch_mfma<256, 128, MODE, false, 4>(p, st);
     }
     else if (bm == 256 && bn == 192) launch_mfma<256, 192, MODE>(p, st);
+    else if (bm == 256 && bn == 256) launch_mfma<256, 256, MODE>(p, st);
     else if (bm == 256 && bn == 128) launch_mfma<256, 128, MODE>(p, st);
     else if (bm == 64 && bn == 128) launch_mfma<64, 128, MODE>(p, st);
     else if ((int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128) > 256) launch_mfma<128, 128, MODE, true>(p, st);
@@ -867,7 +875,17 @@ static void dispatch_band(A8W8Args& p, hipStream_t st, bool aligned, int force_b
         launch_tile<MODE>(p, st, force_bm, force_bn, force_waves);
         return;
     }
-    const TileChoice c = choose_tile(p.M, p.N);
+    TileChoice c = choose_tile(p.M, p.N);
+    if (c.bm == 256 && c.bn >= 192) {
+        // the 256x256 tile in full rounds against 256x192 tiles with their column split, in 256x192 tile times
+        double cost192 = 0.0;
+        const int c1 = split_columns_192(p.M, p.N, &cost192);
+        const int64_t t256 = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+        const double cost256 = (double)((t256 + 255) / 256) * (256.0 / 192.0 / 1.17);
+        // (by a margin: a partly filled last round is cheaper than the model's whole tile time, for either tile;
+        // the cases within 7 % measured between 0.955 and 1.04)
+        c.bn = cost256 < 0.93 * cost192 ? 256 : 192;
+    }
     if (c.bm == 256 && c.bn == 192) {
         const int c1 = split_columns_192(p.M, p.N);
         if (c1 > 0) {

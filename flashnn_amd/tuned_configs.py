@@ -24,7 +24,7 @@ JSON_FILENAME = "hip_autotune_best_configs.json"
 
 # candidate (rows, columns, waves) of the A8W8 MFMA kernel; (0, 0, 0) = static choice (which may be a
 # few-row kernel); waves = 0 is the tile's default (four)
-A8W8_CANDIDATES = [(0, 0, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0),
+A8W8_CANDIDATES = [(0, 0, 0), (256, 256, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0),
                    (256, 256, 8), (256, 192, 8), (256, 128, 8)]
 
 

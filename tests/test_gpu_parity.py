@@ -107,8 +107,8 @@ def _rand_i8(shape, seed, lo=-128, hi=128):
 
 
 # every tile of the MFMA kernel: (rows, columns, waves); (0, 0, 0) = the library's own choice
-TILES = [(0, 0, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0), (256, 256, 8), (256, 192, 8),
-         (256, 128, 8)]
+TILES = [(0, 0, 0), (256, 256, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0), (256, 256, 8),
+         (256, 192, 8), (256, 128, 8)]
 
 
 def _scaled(out_ty, a, b, ar, ac, tile):

@@ -188,8 +188,8 @@ def test_tiled_entry_rejects_unknown_tiles(hip_lib):
     assert rc == -1 and b"no such tile 64x64" in hip_lib.fnn_last_error()
     rc = hip_lib.fnn_gemm_a8w8_tiled(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 0, 0, 0, 128, 128, 8, null)
     assert rc == -1 and b"no such tile 128x128 with 8 waves" in hip_lib.fnn_last_error()
-    rc = hip_lib.fnn_gemm_a8w8_i32_tiled(one, one, one, 4, 4, 128, 128, 128, 4, 256, 256, 4, null)
-    assert rc == -1 and b"no such tile 256x256 with 4 waves" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a8w8_i32_tiled(one, one, one, 4, 4, 128, 128, 128, 4, 64, 128, 8, null)
+    assert rc == -1 and b"no such tile 64x128 with 8 waves" in hip_lib.fnn_last_error()
 
 
 def test_a8w8_rejects_row_strides_beyond_the_band_logic(hip_lib):
