@@ -470,18 +470,25 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
         const int seen = *word;
         // the last unit to arrive that finds every other slot complete adds them up without storing its own
         if (!((seen & 0xffff) == p.kparts - 1 && (seen >> 16) == p.kparts - 1)) {
-            u64* const mine = slots + (int64_t)kpart * (BM * BN / 2) + 2 * threadIdx.x;
+            // 16 bytes per lane, so that a wave's store covers whole 128-byte lines: written as two 8-byte
+            // halves every line went to memory twice, half filled each time (M=256 N=4096 K=8192 in three
+            // parts: 27.1 us, with whole lines 24.2 us).  Device scope (sc1) through the buffer form of
+            // the store, which takes the cache policy as an argument.
+            const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
+                (char*)slots + (int64_t)kpart * (BM * BN * 4), 0, BM * BN * 4, 0x00027000);
 #pragma unroll
             for (int i = 0; i < FN; ++i)
 #pragma unroll
-                for (int j = 0; j < FM; ++j) {
-                    const v4i v = acc[i][j];
-                    u64* const w = mine + (i * FM + j) * (2 * NT);
-                    __hip_atomic_store(w, (u64)(uint32_t)v[0] | ((u64)(uint32_t)v[1] << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(w + 1, (u64)(uint32_t)v[2] | ((u64)(uint32_t)v[3] << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-            // every wave waits until its stores have been acknowledged, then one lane counts the slot complete
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                for (int j = 0; j < FM; ++j)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, acc[i][j]), mine, threadIdx.x * 16,
+                                                           (i * FM + j) * (NT * 16), 16 /* sc1 */);
+            // Every wave waits here until all of its slot stores have been acknowledged (vmcnt counts a
+            // store until the memory side has taken it); only behind the barrier that follows does one
+            // lane count the slot complete.  The order "slot written, then counted" rests on this wait: a
+            // workgroup-scope fence promises nothing about when stores reach device scope.
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0x0070);
+            asm volatile("" ::: "memory");
             __syncthreads();
             if (threadIdx.x == 0)
                 *word = __hip_atomic_fetch_add(p.ws_count + t, 0x10000, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -489,6 +496,10 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
             // whoever completes the last of all kparts slots adds up the others; otherwise this unit is done
             if ((*word >> 16) != p.kparts - 1) return;
         }
+        // The count that chose this unit was returned to lane 0 before the barrier above, and the loads
+        // below are issued behind that barrier: they reach memory after every slot they read was counted
+        // complete.  They are device-scope loads, served where the stores went.
+        asm volatile("" ::: "memory");
         for (int q = 0; q < p.kparts; ++q) {
             if (q == kpart) continue;
             const u64* const theirs = slots + (int64_t)q * (BM * BN / 2) + 2 * threadIdx.x;
@@ -803,32 +814,38 @@ static size_t split_ws_bytes(const SplitPlan& s, int64_t M, int64_t N) {
     return kWsHeader + (size_t)tiles * s.kparts * s.bm * s.bn * sizeof(int32_t);
 }
 
-// Whether to split K for this shape, and how.  Measured (bf16 out, microseconds, unsplit -> split): the split
-// pays where the unsplit kernel's tiles fill at most three quarters of the CUs and K is 8192 or more (the
-// unsplit kernel's time on such shapes follows K alone, about 0.42 us per slab whatever M and N: a
-// workgroup's chain of slabs is bound by the latency of the weights from HBM, and the split shortens it):
-//   M = 256  N = 4096 K = 8192   30.3 -> 26.2 (3 parts)     M = 128 N = 8192 K = 8192   33.3 -> 29.2 (3 parts)
-//   M = 768  N = 2048 K = 16384  53.0 -> 45.3 (2 parts)     M = 128 N = 2048 K = 16384  54.9 -> 31.2 (8 parts)
-//   M = 384  N = 1920 K = 13312  46.6 -> 31.2 (4 parts)     M = 512 N = 1024 K = 8192   28.6 -> 27.4 (7 parts)
-// and costs where they fill them anyway (M = 512 N = K = 8192: 44.5 -> 51.5; M = 2048 N = 1024 K = 8192:
-// 23.6 -> 28.7).  The tile is 128x128 in pairs of workgroups per CU: with M this small the weights stream
-// from HBM, and two workgroups per CU keep twice the bytes in flight; the 256-row tiles were slower split
-// than the small tiles unsplit.  About 224 units (seven eighths of one per CU, a pair never on one CU) was
-// the best count; a part holds at least 8 slabs.
+// Whether to split K for this shape, and how.  The tile is 128x128 in pairs of workgroups per CU: with few
+// activation rows the weights stream from HBM, and two workgroups per CU keep twice the bytes in flight; a
+// workgroup's chain of slabs is bound by the latency of the weights, and the split shortens it (the 256-row
+// tiles were slower split than the small tiles unsplit).  Measured, bf16 out, microseconds, unsplit -> split
+// (parts; units = 128x128 tiles x parts):
+//   M = 256  N = 4096 K = 8192   27.1 -> 24.2 (3; 192)      M = 128  N = 2048 K = 16384  54.9 -> 30.2 (8; 128)
+//   M = 512  N = 2048 K = 8192   29.3 -> 22.9 (4; 256)      M = 256  N = 4096 K = 6144   24.6 -> 20.9 (4; 256)
+//   M = 1024 N = 1920 K = 13312  48.3 -> 39.5 (2; 240)      M = 512  N = 4096 K = 11008  41.4 -> 35.5 (2; 256)
+//   M = 384  N = 3584 K = 18944  68.6 -> 44.1 (3; 252)      M = 1024 N = 2048 K = 8192   29.7 -> 27.2 (2; 256)
+// About one unit per CU is the best count (84 tiles: 3 parts 44.1, 2 parts 52.8, 4 parts 49.0), a part
+// needs 8 slabs and K at least 6144 (K = 4096: 17.0 -> 17.8 and worse).  Up to two units per CU - every CU
+// holding a pair - pay only over a long K, from about 40 slabs per part:
+//   M = 764  N = 3584 K = 18944  85.8 -> 63.0 (3; 504)      M = 1024 N = 3584 K = 18944  86.3 -> 71.1 (2; 448)
+//   M = 1024 N = 4096 K = 11008  53.3 -> 51.7 (2; 512)      M = 512  N = 8192 K = 8192   40.7 -> 45.1 (2; 512: not taken)
 static SplitPlan plan_split(int64_t M, int64_t N, int64_t K, size_t ws_bytes) {
     const int KT = (int)((K + 127) / 128);
     const TileChoice u = choose_tile(M, N);
-    SplitPlan none{u.bm, u.bn, 1, 0, 0.0};
-    const int64_t utiles = ((M + u.bm - 1) / u.bm) * ((N + u.bn - 1) / u.bn);
-    if (KT < 64 || utiles > 192) return none;      // (K = 4096: 0.70 to 0.95 of the unsplit speed; K = 6144: 0.91 to 1.10)
+    const SplitPlan none{u.bm, u.bn, 1, 0, 0.0};
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
-    int parts = (int)(224 / t128);
-    if (parts > 8) parts = 8;
-    while (parts >= 2 && split_chunk_slabs(KT, parts) < 8) --parts;
-    if (parts < 2) return none;
-    const SplitPlan s{128, 128, parts, split_chunk_slabs(KT, parts) * 128, 0.0};
-    if (ws_bytes != 0 && split_ws_bytes(s, M, N) > ws_bytes) return none;
-    return s;
+    if (KT < 48 || t128 > 256) return none;
+    int parts = 1;
+    for (int q = 2; q <= 8; ++q) {
+        const int64_t units = t128 * q;
+        const int slabs = split_chunk_slabs(KT, q);
+        if ((units <= 288 && slabs >= 8) || (units <= 512 && slabs >= 40)) parts = q;
+    }
+    // (a workspace too small for the best count takes the largest one it holds)
+    for (; parts >= 2; --parts) {
+        const SplitPlan s{128, 128, parts, split_chunk_slabs(KT, parts) * 128, 0.0};
+        if (ws_bytes == 0 || split_ws_bytes(s, M, N) <= ws_bytes) return s;
+    }
+    return none;
 }
 
 template <int MODE>
@@ -1044,9 +1061,15 @@ __global__ __launch_bounds__(256) void clear_words_kernel(int* w, int n) {
 }
 }  // namespace fnn
 
+static int static_scratch(const char* fn, void** out);
+
 extern "C" int fnn_workspace_init(void* workspace, size_t ws_bytes, void* stream) {
     const char* fn = "fnn_workspace_init";
-    if (!workspace || ((uintptr_t)workspace % 16) != 0 || ws_bytes < kWsHeader) {
+    if (!workspace && ws_bytes == 0) {
+        // the library's own workspace on the current device (fnn_gemm_a8w8_static)
+        const int rc = static_scratch(fn, &workspace);
+        if (rc != FNN_OK) return rc;
+    } else if (!workspace || ((uintptr_t)workspace % 16) != 0 || ws_bytes < kWsHeader) {
         set_error("%s: the workspace must be 16-byte aligned and hold at least %zu bytes", fn, kWsHeader);
         return FNN_ERR_ARG;
     }

@@ -124,11 +124,15 @@ _A8W8_WS_BYTES = {}      # (M, N, K) -> bytes of workspace the library would use
 _A8W8_WORKSPACES = {}    # (device index, stream handle) -> zero-initialised workspace tensor
 
 
+_A8W8_WS_ALLOC = (32 << 20) + 4096      # holds every plan of the library
+
+
 def _a8w8_workspace(lib, device, stream, M, N, K):
     """The workspace for a shape whose K the library would split over several workgroups per tile, or
-    None.  One buffer per device and stream (calls on one stream run in order; calls that overlap must not
-    share it), allocated at the first shape that needs one and sized for every shape (no plan takes more
-    than 224 slots of 64 KB).  It starts zeroed and every call leaves its counters zeroed."""
+    None.  One buffer per device and stream (calls on one stream run in order; calls that overlap in time
+    must not share a workspace: a graph captured here and replayed on several streams at once needs the
+    C entry point with a workspace per replay), allocated at the first shape that needs one and sized
+    for every shape.  It starts zeroed and every call leaves its counters zeroed."""
     need = _A8W8_WS_BYTES.get((M, N, K))
     if need is None:
         need = _A8W8_WS_BYTES[(M, N, K)] = int(lib.fnn_gemm_a8w8_workspace_bytes(M, N, K))
@@ -137,7 +141,9 @@ def _a8w8_workspace(lib, device, stream, M, N, K):
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     ws = _A8W8_WORKSPACES.get(key)
     if ws is None or ws.numel() < need:
-        ws = _A8W8_WORKSPACES[key] = torch.zeros(max(need, 16 << 20), dtype=torch.uint8, device=device)
+        if len(_A8W8_WORKSPACES) >= 16:         # streams come and go: keep the table small
+            _A8W8_WORKSPACES.clear()
+        ws = _A8W8_WORKSPACES[key] = torch.zeros(max(need, _A8W8_WS_ALLOC), dtype=torch.uint8, device=device)
     return ws
 
 
@@ -178,7 +184,11 @@ def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col, tile=None):
         if ws is None:
             _lib.check(lib.fnn_gemm_a8w8(*args, stream))
         else:
-            _lib.check(lib.fnn_gemm_a8w8_ws(*args, ws.data_ptr(), ws.numel(), stream))
+            rc = lib.fnn_gemm_a8w8_ws(*args, ws.data_ptr(), ws.numel(), stream)
+            if rc != 0:
+                # a split call that failed half way may have left counters behind: never reuse the buffer
+                _A8W8_WORKSPACES.clear()
+            _lib.check(rc)
     else:
         _lib.check(lib.fnn_gemm_a8w8_tiled(*args, *tile, stream))
     return out

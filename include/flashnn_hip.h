@@ -181,8 +181,8 @@ int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, const void* alp
                         int alpha_col_dtype, int tile_m, int tile_n, int waves, void* stream);
 
 /*
- * fnn_gemm_a8w8 with a workspace: where few tiles would leave most CUs idle over a long K (M and N small,
- * K of 8192 and more), K is cut into parts that run as separate workgroups; the parts' int32 accumulators
+ * fnn_gemm_a8w8 with a workspace: where few tiles would leave most CUs idle over a long K (at most 256
+ * tiles of 128x128, K of 6144 and more), K is cut into parts that run as separate workgroups; the parts' int32 accumulators
  * meet in the workspace and the last part to finish a tile adds them up and writes the scaled output.
  * Integer addition does not depend on the order, so the result equals fnn_gemm_a8w8's bit for bit.  Shapes
  * that do not gain run exactly as in fnn_gemm_a8w8.  The role of the SPLIT_K meta-parameter of the
@@ -191,12 +191,18 @@ int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, const void* alp
  *
  * workspace  device memory, 16-byte aligned; its first 4096 bytes are counters that must be zero when a
  *            call starts and are zero again when it ends: zero them once after allocation
- *            (fnn_workspace_init, or hipMemset / a zero-filled tensor) and never again.  The rest needs no
- *            initialisation.  Calls that overlap in time (other streams, other threads) need a workspace
- *            each.
+ *            (fnn_workspace_init, or hipMemset / a zero-filled tensor) and never again - except after a
+ *            call on it failed with FNN_ERR_HIP or its kernel was aborted: counters may then be left
+ *            behind, and every later split on that workspace would be wrong until it is initialised
+ *            again.  The rest needs no initialisation.  Calls that overlap in time (other streams, other
+ *            threads, a captured graph replayed on several streams at once) need a workspace each.
+ *            fnn_workspace_init(NULL, 0, stream) clears the counters of the library's own workspace
+ *            on the current device (the one fnn_gemm_a8w8_static uses).
  * ws_bytes   its size.  fnn_gemm_a8w8_workspace_bytes(M, N, K) is what the call would use for a shape (0:
- *            the shape is not split); 16 MiB hold every shape.  With less than a shape needs (at least
- *            the 4096 bytes of counters; or workspace = NULL with ws_bytes = 0) the call runs unsplit.
+ *            the shape is not split); 32 MiB + 4096 bytes hold every shape.  With less than a shape needs
+ *            the call takes the largest split that fits (16 MiB hold all but the splits into more units
+ *            than there are CUs), and with none that fits (at least the 4096 bytes of counters; or
+ *            workspace = NULL with ws_bytes = 0) it runs unsplit.
  */
 size_t fnn_gemm_a8w8_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int fnn_workspace_init(void* workspace, size_t ws_bytes, void* stream);
@@ -223,7 +229,7 @@ int fnn_gemm_a8w8_ws_tiled(void* out, const void* a, const void* b, const void* 
  * No counterpart in the reference.  It is for callers that cannot allocate: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc - the call allocates and frees nothing (the device
  * address of the array is looked up once per device, on the first call there).
- *   tile_m = tile_n = kparts = 0: the library's choice, as fnn_gemm_a8w8_ws; its plans always fit.
+ *   tile_m = tile_n = kparts = 0: the library's choice, as fnn_gemm_a8w8_ws with a workspace of 16 MiB.
  *   a named split that needs more than the array holds: FNN_ERR_UNSUPPORTED, and the message says how
  *   much; use fnn_gemm_a8w8_ws_tiled with a workspace of that size.
  * All calls on a GPU share that GPU's array: calls that overlap in time (other streams, other threads)

@@ -351,7 +351,8 @@ def test_a8w8_split_k_bit_exact(hip_lib, plan, mnk):
     assert torch.equal(plain, out)
 
 
-@pytest.mark.parametrize("mnk", [(256, 4096, 8192), (128, 2048, 16384), (384, 1920, 13312), (100, 1000, 9248), (2048, 4096, 4096)])
+@pytest.mark.parametrize("mnk", [(256, 4096, 8192), (128, 2048, 16384), (384, 1920, 13312), (100, 1000, 9248), (2048, 4096, 4096),
+                                 (1024, 1920, 13312), (640, 3584, 18944), (256, 4096, 6144)])
 def test_a8w8_workspace_entry_matches_plain(hip_lib, mnk):
     """fnn_gemm_a8w8_ws: shapes the library splits (and one it does not) against fnn_gemm_a8w8, bit for bit,
     through the operator too (its launcher keeps a workspace per stream); a workspace smaller than the
@@ -363,12 +364,12 @@ def test_a8w8_workspace_entry_matches_plain(hip_lib, mnk):
     ar = (torch.rand(M, device=DEV, generator=g) * 1e-2 + 1e-3).half()
     ac = (torch.rand(N, device=DEV, generator=g) * 1e-2 + 1e-3).half()
     need = hip_lib.fnn_gemm_a8w8_workspace_bytes(M, N, K)
-    assert (need > 0) == (M < 2048) and need <= 16 << 20
+    assert (need > 0) == (M < 2048) and need <= (32 << 20) + 4096
     plain = torch.empty(M, N, dtype=torch.float16, device=DEV)
     assert hip_lib.fnn_gemm_a8w8(plain.data_ptr(), a.data_ptr(), b.data_ptr(), ar.data_ptr(), ac.data_ptr(), M, N, K, K, K, N,
                                  0, 0, 0, _lib.current_stream(a.device)) == 0
     unsplit_kernel = _lib.last_kernel()
-    ws = torch.empty(16 << 20, dtype=torch.uint8, device=DEV)
+    ws = torch.empty((32 << 20) + 4096, dtype=torch.uint8, device=DEV)
     assert hip_lib.fnn_workspace_init(ws.data_ptr(), ws.numel(), _lib.current_stream(a.device)) == 0
     out = torch.empty_like(plain)
     assert _a8w8_ws_call(hip_lib, out, a, b, ar, ac, ws) == 0
@@ -378,7 +379,10 @@ def test_a8w8_workspace_entry_matches_plain(hip_lib, mnk):
     assert ("split K" in _lib.last_kernel()) == (need > 0) and torch.equal(via_op, plain)
     if need:
         out.zero_()
-        assert _a8w8_ws_call(hip_lib, out, a, b, ar, ac, ws[:need - 16]) == 0
+        assert _a8w8_ws_call(hip_lib, out, a, b, ar, ac, ws[:need - 16]) == 0      # a split into fewer parts, or none
+        assert torch.equal(out, plain)
+        out.zero_()
+        assert _a8w8_ws_call(hip_lib, out, a, b, ar, ac, ws[:4096]) == 0           # room for the counters only
         assert _lib.last_kernel() == unsplit_kernel and torch.equal(out, plain)
     want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a[:3].cpu().numpy(), b.cpu().numpy()), O.to_np(ar[:3].cpu()),
                                      O.to_np(ac.cpu()), O.F16)

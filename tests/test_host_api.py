@@ -215,12 +215,15 @@ def test_workspace_entries_reject_bad_arguments(hip_lib):
     assert hip_lib.fnn_gemm_a8w8_ws_tiled(*base, 256, 128, 2, one, 8192, null) == -1
     assert b"the split needs 528384" in hip_lib.fnn_last_error()
     assert hip_lib.fnn_gemm_a8w8_ws_tiled(*base, 256, 128, -1, one, 1 << 30, null) == -1
-    # which shapes the library would split, and that nothing needs more than 16 MiB
+    # which shapes the library would split, and that nothing needs more than 32 MiB + 4 KiB
     f = hip_lib.fnn_gemm_a8w8_workspace_bytes
     assert f(2048, 12288, 4096) == 0 and f(16, 4096, 8192) == 0 and f(512, 8192, 8192) == 0
-    assert f(256, 4096, 8192) == 4096 + 64 * 3 * 65536
-    assert all(f(M, N, K) <= 16 << 20 for M in (65, 100, 128, 500, 1000, 3000) for N in (128, 1000, 4096, 20000)
-               for K in (8192, 16384, 32768))
+    assert f(256, 4096, 4096) == 0 and f(1024, 4096, 4096) == 0
+    assert f(256, 4096, 8192) == 4096 + 64 * 4 * 65536
+    assert f(1024, 1920, 13312) == 4096 + 120 * 2 * 65536        # one unit per CU
+    assert f(764, 3584, 18944) == 4096 + 168 * 3 * 65536         # a long K: two per CU
+    assert all(f(M, N, K) <= (32 << 20) + 4096 for M in (65, 100, 128, 500, 1000, 3000) for N in (128, 1000, 4096, 20000)
+               for K in (6144, 8192, 16384, 32768))
 
 
 def test_empty_calls_need_no_addresses(hip_lib):

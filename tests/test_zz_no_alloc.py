@@ -71,3 +71,8 @@ def test_static_workspace_entry_rejects_what_does_not_fit(hip_lib):
     assert torch.equal(out, want)
     assert hip_lib.fnn_gemm_a8w8_static(*_args(out, a, b, ar, ac), 0, 0, 0, st) == 0
     assert torch.equal(out, want)
+    # the counters of the library's own workspace can be cleared from outside (after a failed call)
+    assert hip_lib.fnn_workspace_init(None, 0, st) == 0, hip_lib.fnn_last_error()
+    out.zero_()
+    assert hip_lib.fnn_gemm_a8w8_static(*_args(out, a, b, ar, ac), 0, 0, 0, st) == 0
+    assert torch.equal(out, want)
