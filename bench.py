@@ -7,12 +7,14 @@ per-token x per-channel scale epilogue writing bf16 (the Llama-7B QKV prefill sh
 `value` is 2*M*N*K / step time in TOPS with all inputs resident in HBM.
 
 Also measured in the same run and reported in the same JSON line:
-  roofline      the A8W8 GEMM kernel alone against the dense int8 MFMA peak
+  roofline      the A8W8 GEMM kernel alone against the dense int8 MFMA peak, and under "a16w4_decode_m1" the
+                second half of the metric: the A16W4 decode at M=1 against the 8 TB/s of HBM, on the
+                reference's weight layout and on the packed form of GemmWeightOnly.prepack
   secondary     one entry per point of every configuration the path is quoted on, each against its bound:
                   c1     DynamicQuant + A8W8 at M=16 K=N=4096, fp16 out
                   c2     the four M=2048 prefill shapes (quant + GEMM, and the GEMM alone)
                   c3     A16W8 decode, M in {1, 8, 32} x three (K, N)
-                  c4     A16W4 group-128 at K=8192 N=28672, M in {1, 4, 16, 64, 256}
+                  c4     A16W4 group-128 at K=8192 N=28672, M in {1, 4, 16, 64, 256} (M=1 always runs)
                   c5     RMSNormDquant -> A8W8 at K=N=8192, M in {1, 32, 512, 8192}
                   g64    A16W4 group-64 at the reference test's shape M=3 N=1024 K=4096
                   splitk A8W8 shapes whose K the library splits, against the unsplit kernel
@@ -80,17 +82,21 @@ def _traffic(key):
 
 
 def _entry(workload, ms, bound, amount, kernels, traffic_key=None, **extra):
-    """One secondary entry.  amount: algorithmic operations (bound 'mfma' / 'mfma16') or bytes ('hbm') per
-    call of the timed function."""
+    """One secondary entry, kept short (the whole line has to fit the tail a harness keeps): w = workload,
+    k = kernel as the library names it, us = microseconds per launch, bound = the roofline that applies
+    ('hbm': 8000 GB/s; 'mfma': 5000 TOP/s int8; 'mfma16': 2500 TFLOP/s bf16/fp16), ach = achieved GB/s, TOP/s
+    or TFLOP/s on the algorithmic bytes or operations of the call, frac = ach / peak, traffic = measured HBM
+    bytes per launch where counted."""
     if bound == "hbm":
-        achieved, peak, unit = amount / (ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+        achieved, peak = amount / (ms * 1e-3) / 1e9, PEAK_HBM_GBS
     else:
-        achieved, unit = amount / (ms * 1e-3) / 1e12, "TOP/s" if bound == "mfma" else "TFLOP/s"
+        achieved = amount / (ms * 1e-3) / 1e12
         peak = PEAK_INT8_TOPS if bound == "mfma" else PEAK_F16_TFLOPS
-    e = {"workload": workload, "kernel": kernels, "us_per_launch": round(ms * 1e3, 2),
-         "roofline": {"bound": "hbm" if bound == "hbm" else "mfma", "achieved": round(achieved, 1), "peak": peak,
-                      "unit": unit, "frac": round(achieved / peak, 4),
-                      "traffic": _traffic(traffic_key) if traffic_key else None}}
+    e = {"w": workload, "k": kernels, "us": round(ms * 1e3, 2), "bound": bound, "ach": round(achieved, 1),
+         "frac": round(achieved / peak, 3)}
+    t = _traffic(traffic_key) if traffic_key else None
+    if t is not None:
+        e["traffic"] = t
     e.update(extra)
     return e
 
@@ -196,8 +202,8 @@ def main():
         else:
             ms_step, _ = _timed(step, iters, torch)
             ms_gemm, _ = _timed(gemm_only, iters, torch)
-            secondary.append(_entry(f"c2 a8w8 {name} M={M} K={K} N={N} bf16: GEMM", ms_gemm, "mfma", ops, k_gemm,
-                                    f"a8w8 {name}", us_quant_plus_gemm=round(ms_step * 1e3, 2)))
+            secondary.append(_entry(f"c2 a8w8 {name} M={M} K={K} N={N} bf16", ms_gemm, "mfma", ops, k_gemm,
+                                    f"a8w8 {name}", us_with_quant=round(ms_step * 1e3, 2)))
         del ws, xs, qs, ss, outs
         torch.cuda.empty_cache()
     gemm_tops = primary["ops"] / (primary["ms_gemm"] * 1e-3) / 1e12
@@ -290,26 +296,44 @@ def main():
     # ------------------------------------------------- c4: A16W4 group 128, K = 8192, N = 28672, bf16
     K4, N4 = workloads.A16W4_SHAPE
     packed, scale4, zp4, _, _ = workloads.int4_group_weights(N4, K4, 128)
-    if "c4" in legs:
-        pk = rotating(packed.to(dev), total_bytes=500e6)
-        n = len(pk)
-        sc = [scale4.to(dev).clone() for _ in range(n)]
-        zp = [zp4.to(dev).clone() for _ in range(n)]
-        wbytes = N4 * K4 / 2 + 2 * (K4 // 128) * N4 * 2
-        for m4 in (1, 4, 16, 64, 256):
-            act = workloads.activations(m4, K4, torch.bfloat16, seed=3).to(dev)
-            o4 = torch.empty(m4, N4, dtype=torch.bfloat16, device=dev)
-            f = lambda i: launchers.hip_gemm_a16w4_forward(o4, act, pk[i % n], sc[i % n], None, zp[i % n])
-            kern = kernel_of(f)
-            ms, _ = _timed(f, iters, torch)
-            extra = {"weight_GBps": round(wbytes / (ms * 1e-3) / 1e9, 1)}
-            if m4 >= 64:      # also as a matrix-core workload
-                extra["bf16_TFLOPs"] = round(2.0 * m4 * N4 * K4 / (ms * 1e-3) / 1e12, 1)
-                extra["frac_of_bf16_peak"] = round(2.0 * m4 * N4 * K4 / (ms * 1e-3) / 1e12 / PEAK_F16_TFLOPS, 4)
-            secondary.append(_entry(f"c4 a16w4 g128 M={m4} K={K4} N={N4} bf16", ms, "hbm",
-                                    wbytes + 2.0 * m4 * K4 + 2.0 * m4 * N4, kern, f"a16w4 g128 M={m4}", **extra))
-        del pk, sc, zp
-        torch.cuda.empty_cache()
+    # (M = 1 is the second half of the metric and always runs, on the reference layout and on the packed form)
+    pk = rotating(packed.to(dev), total_bytes=500e6)
+    n = len(pk)
+    sc = [scale4.to(dev).clone() for _ in range(n)]
+    zp = [zp4.to(dev).clone() for _ in range(n)]
+    wbytes = N4 * K4 / 2 + 2 * (K4 // 128) * N4 * 2
+    decode = {}
+    for m4 in (1, 4, 16, 64, 256) if "c4" in legs else (1,):
+        act = workloads.activations(m4, K4, torch.bfloat16, seed=3).to(dev)
+        o4 = torch.empty(m4, N4, dtype=torch.bfloat16, device=dev)
+        f = lambda i: launchers.hip_gemm_a16w4_forward(o4, act, pk[i % n], sc[i % n], None, zp[i % n])
+        kern = kernel_of(f)
+        ms, _ = _timed(f, iters, torch)
+        extra = {"weight_GBps": round(wbytes / (ms * 1e-3) / 1e9, 1)}
+        if m4 >= 64:      # also as a matrix-core workload
+            extra["bf16_TFLOPs"] = round(2.0 * m4 * N4 * K4 / (ms * 1e-3) / 1e12, 1)
+            extra["frac_of_bf16_peak"] = round(2.0 * m4 * N4 * K4 / (ms * 1e-3) / 1e12 / PEAK_F16_TFLOPS, 3)
+        e = _entry(f"c4 a16w4 g128 M={m4} K={K4} N={N4} bf16", ms, "hbm", wbytes + 2.0 * m4 * K4 + 2.0 * m4 * N4,
+                   kern, f"a16w4 g128 M={m4}", **extra)
+        secondary.append(e)
+        if m4 == 1:
+            decode["reference_layout"] = e
+    # the same decode on weights repacked once (GemmWeightOnly.prepack): the packed form holds exactly the
+    # bytes of the reference layout (nibbles, fp16 scales, fp16 zero points), so the algorithmic bytes are
+    # the bytes it reads
+    packs = [launchers.hip_a16w4_prepack(pk[i], sc[i], zp[i]) for i in range(n)]
+    act = workloads.activations(1, K4, torch.bfloat16, seed=3).to(dev)
+    o4 = torch.empty(1, N4, dtype=torch.bfloat16, device=dev)
+    f = lambda i: launchers.hip_gemm_a16w4_prepacked_forward(o4, act, packs[i % n])
+    kern = kernel_of(f)
+    ms, _ = _timed(f, max(iters, 100), torch)
+    e = _entry(f"c4 a16w4 g128 M=1 K={K4} N={N4} bf16, weights prepacked", ms, "hbm", wbytes + 2.0 * K4 + 2.0 * N4, kern,
+               "a16w4 g128 M=1 prepacked", weight_GBps=round(wbytes / (ms * 1e-3) / 1e9, 1),
+               packed_bytes=int(packs[0].buffer.numel()))
+    secondary.append(e)
+    decode["prepacked"] = e
+    del pk, sc, zp, packs
+    torch.cuda.empty_cache()
 
     # ------------------------------------------------------------ c3: A16W8 decode, fp16, per-channel
     if "c3" in legs:
@@ -488,6 +512,12 @@ def main():
                         "a16w4_decode_m1_ms": round(t_cpu4 * 1e3, 1),
                         "a16w4_decode_m1_weight_GBps": round((N4 * K4 / 2 + 4 * (K4 // 128) * N4) / t_cpu4 / 1e9, 3)}
 
+    # the second half of the metric, beside the first: A16W4 decode at M = 1 against the 8 TB/s of HBM3E, on
+    # the layout the reference's operator takes and on the packed form (bytes actually read = algorithmic bytes)
+    roofline["a16w4_decode_m1"] = {
+        name: {"kernel": e["k"], "bound": "hbm", "us_per_launch": e["us"], "achieved": e["ach"], "peak": PEAK_HBM_GBS,
+               "unit": "GB/s", "frac": e["frac"], "traffic": e.get("traffic")}
+        for name, e in decode.items()}
     value = primary["ops"] / (primary["ms_step"] * 1e-3) / 1e12
     result = {
         "metric": "a8w8_int8_tops_m2048", "value": round(value, 2), "unit": "TOPS", "n_gpus": 1,

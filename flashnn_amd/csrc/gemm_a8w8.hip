@@ -838,7 +838,7 @@ static SplitPlan plan_split(int64_t M, int64_t N, int64_t K, size_t ws_bytes) {
     for (int q = 2; q <= 8; ++q) {
         const int64_t units = t128 * q;
         const int slabs = split_chunk_slabs(KT, q);
-        if ((units <= 288 && slabs >= 8) || (units <= 512 && slabs >= 40)) parts = q;
+        if ((units <= 256 && slabs >= 8) || (units <= 512 && slabs >= 40)) parts = q;
     }
     // (a workspace too small for the best count takes the largest one it holds)
     for (; parts >= 2; --parts) {

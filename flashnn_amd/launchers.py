@@ -271,3 +271,60 @@ def hip_gemm_a16w4_forward(out, act, quant_w, scale_w, bias=None, zero_points=No
     quant_w is [N/2, K] with channel 2j in the low and 2j+1 in the high nibble of row j."""
     return _weight_only("fnn_gemm_a16w4", out, act, quant_w, scale_w, bias, zero_points,
                         quant_w.shape[0] * 2)
+
+
+class PrepackedInt4:
+    """int4 weights with groups of 128 in the library's packed form (see hip_a16w4_prepack): the buffer and
+    the shape it stands for."""
+
+    def __init__(self, buffer, n, k, group):
+        self.buffer, self.n, self.k, self.group = buffer, n, k, group
+
+
+def hip_a16w4_prepack(quant_w, scale_w, zero_points=None):
+    """Repack int4 weights in the reference layout (quant_w [N/2, K] int8 as GemmWeightOnly takes them,
+    flashnn/quant_gemm.py:174-204; scale_w and zero_points [K/128, N] fp16) into one stream for the decode
+    of one token.  Returns a PrepackedInt4; the originals are not modified and can be freed.  No
+    counterpart in the reference, whose launcher reads the layout above as it is (gemm_a16w4.py:336-406)."""
+    assert quant_w.dtype == torch.int8 and quant_w.dim() == 2 and quant_w.stride(1) == 1, "Weight must be int8 type"
+    assert scale_w.dim() == 2 and scale_w.dtype == torch.float16 and scale_w.is_contiguous(), \
+        "the packed form takes fp16 scales per group of 128"
+    _lib.require_gpu(quant_w, scale_w, zero_points)
+    lib = _lib.load()
+    K = quant_w.shape[1]
+    N = quant_w.shape[0] * 2
+    assert scale_w.shape[1] == N and scale_w.shape[0] * 128 == K, "the packed form takes groups of 128"
+    zp = None
+    if zero_points is not None:
+        zp = zero_points.reshape(scale_w.shape).to(torch.float16).contiguous()
+    size = int(lib.fnn_a16w4_prepacked_bytes(N, K, 128))
+    if size == 0:
+        raise _lib.FlashnnHipError(f"no packed form for N={N} K={K} (needs N % 16 == 0 and K % 1024 == 0)")
+    buf = torch.empty(size, dtype=torch.uint8, device=quant_w.device)
+    _lib.check(lib.fnn_a16w4_prepack(_lib.ptr(buf), _lib.ptr(quant_w), _lib.ptr(scale_w), _lib.ptr(zp), N, K,
+                                     quant_w.stride(0), 128, _lib.dtype_code(scale_w.dtype), _lib.FNN_F16,
+                                     _lib.current_stream(quant_w.device)))
+    return PrepackedInt4(buf, N, K, 128)
+
+
+def hip_gemm_a16w4_prepacked_forward(out, act, packed, bias=None):
+    """triton_gemm_a16w4_forward (flashnn/triton_kernels/gemm_a16w4.py:336-406) for one activation row on
+    weights packed by hip_a16w4_prepack."""
+    assert isinstance(packed, PrepackedInt4)
+    assert act.is_contiguous(), "Activation must be contiguous"
+    assert act.dim() == 2 and act.shape[1] == packed.k, "Matrix B must be transposed"
+    _lib.require_gpu(out, act, packed.buffer, bias)
+    lib = _lib.load()
+    M = act.shape[0]
+    assert out.shape == (M, packed.n) and out.stride(1) == 1
+    if bias is not None:
+        if bias.dim() != 1 or not bias.is_contiguous():
+            bias = bias.reshape(-1).contiguous()
+        assert bias.numel() == packed.n
+    _lib.check(lib.fnn_gemm_a16w4_prepacked(_lib.ptr(out), _lib.ptr(act), _lib.ptr(packed.buffer), _lib.ptr(bias), M,
+                                            packed.n, packed.k, act.stride(0) if M > 1 else packed.k,
+                                            out.stride(0) if M > 1 else packed.n, packed.group,
+                                            _lib.dtype_code(act.dtype), _lib.dtype_code(out.dtype),
+                                            _lib.dtype_code(bias.dtype) if bias is not None else 0,
+                                            _lib.current_stream(act.device)))
+    return out

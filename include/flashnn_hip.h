@@ -141,6 +141,35 @@ int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const void* scale
                    int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
                    void* stream);
 
+/*
+ * fnn_gemm_a16w4 for the decode of one token (M = 1) on weights repacked once by the caller.  The
+ * reference keeps int4 weights as [N/2, K] bytes with [K/group, N] tables beside them
+ * (flashnn/quant_gemm.py:174-204; its Triton launcher, flashnn/triton_kernels/gemm_a16w4.py:336-406, reads
+ * that layout as it is); a decode kernel then fetches rows K bytes apart plus two side tables.  The packed
+ * form is one stream: everything 16 channels need for 1024 values of K - 8 KB of nibbles, then the 8 x 16
+ * scales and the 8 x 16 zero points of those eight groups - is one contiguous unit of 8704 bytes, units in the
+ * order [channel tile][K range].  The bytes are exactly the reference layout's with fp16 tables,
+ * N K / 2 + 2 (K / 128) N 2; nothing is dropped or merged, zero points stay the caller's fp16 values.
+ * The unit's inner order is written out in flashnn_amd/csrc/gemm_wo_prepacked.hip and restated, with its
+ * inverse, in oracle/flashnn_oracle.py (prepack_a16w4 / unpack_prepacked_a16w4).
+ *   fnn_a16w4_prepacked_bytes(N, K, group)  size of the packed form; 0 if the shape has none (it needs
+ *                                           group = 128, N % 16 == 0, K % 1024 == 0 and K / 1024 in
+ *                                           {1, 2, 4} or at least 8)
+ *   fnn_a16w4_prepack(packed, qw, scale, zp, ...)   packed <- the reference layout (qw [N/2, K] with row stride
+ *                                           ldw, scale and zp [K/128, N] fp16, zp may be NULL = zeros);
+ *                                           a device-side copy, asynchronous on `stream`
+ *   fnn_gemm_a16w4_prepacked(out, act, packed, bias, ...)   out[0, n] as fnn_gemm_a16w4 computes it, within
+ *                                           rtol = atol = 1e-2 of the reference (group scales are applied in
+ *                                           fp32 to group sums); M > 1 is FNN_ERR_UNSUPPORTED
+ * Nothing repacks implicitly: fnn_gemm_a16w4 always reads the reference layout.
+ */
+size_t fnn_a16w4_prepacked_bytes(int64_t N, int64_t K, int64_t group);
+int fnn_a16w4_prepack(void* packed, const void* qw, const void* scale, const void* zp, int64_t N, int64_t K,
+                      int64_t ldw, int64_t group, int scale_dtype, int zp_dtype, void* stream);
+int fnn_gemm_a16w4_prepacked(void* out, const void* act, const void* packed, const void* bias, int64_t M,
+                             int64_t N, int64_t K, int64_t lda, int64_t ldc, int64_t group, int act_dtype,
+                             int out_dtype, int bias_dtype, void* stream);
+
 /* RMSNorm: out[m,k] = round_T(round_T(x[m,k] * rsqrt(mean_k(x^2) + eps)) * gamma[k]), T = x_dtype.
  * Replaces triton_rmsnorm_forward(x, weight, eps) (flashnn/triton_kernels/rms_norm.py:68-83) behind
  * RMSNorm (flashnn/norm.py:19-36); semantics of _torch_impl (:31-33) with the result in the input

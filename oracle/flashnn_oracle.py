@@ -235,6 +235,68 @@ def pack_int4(w: np.ndarray) -> np.ndarray:
     return (lo | (hi << 4)).astype(np.uint8).view(np.int8)
 
 
+# ---- the packed form of int4 weights for the one-token decode (no counterpart in the reference: these two
+# functions restate the layout that flashnn_amd/csrc/gemm_wo_prepacked.hip documents, one as array
+# reshapes, the other address by address, so that each checks the other and the kernel's repacking)
+PREPACK_UNIT_BYTES = 8 * 1024 + 2 * 256
+
+
+def prepack_a16w4(qw: np.ndarray, scale: np.ndarray, zp) -> np.ndarray:
+    """[N/2, K] packed bytes of the reference layout (flashnn/quant_gemm.py:175-190) plus [K/128, N] fp16
+    scales and zero points (None: zeros) -> the packed stream, as uint8.
+
+    Units in the order [tile of 16 channels][range of 1024 values of K]; a unit is 8 groups x (4 eighths x 16
+    channels x 4 words) 32-bit words of nibbles, then scales [channel][group], then zero points."""
+    u = (unpack_int4(qw).astype(np.int16) + 8).astype(np.uint32)          # the weight as 0..15
+    N, K = u.shape
+    assert N % 16 == 0 and K % 1024 == 0
+    T, KC = N // 16, K // 1024
+    scale = np.asarray(scale, dtype=np.float16)
+    zp = np.zeros_like(scale) if zp is None else np.asarray(zp, dtype=np.float16)
+    assert scale.shape == (K // 128, N) and zp.shape == scale.shape
+    v = u.reshape(T, 16, KC, 8, 4, 4, 8)                                  # tile, c, kc, b, i, g, j
+    word = np.zeros(v.shape[:-1], dtype=np.uint32)
+    for j in range(8):
+        word |= v[..., j] << np.uint32(4 * ((j >> 1) + 4 * (j & 1)))
+    nib = np.ascontiguousarray(word.transpose(0, 2, 3, 5, 1, 4)).astype("<u4")   # tile, kc, b, g, c, i
+    nib = nib.reshape(T, KC, 8 * 16 * 4 * 4).view(np.uint8)
+    def table(t):
+        t = t.reshape(KC, 8, T, 16).transpose(2, 0, 3, 1)                  # tile, kc, c, b
+        return np.ascontiguousarray(t).astype("<f2").reshape(T, KC, 128).view(np.uint8)
+    out = np.concatenate([nib, table(scale), table(zp)], axis=2)
+    assert out.shape == (T, KC, PREPACK_UNIT_BYTES)
+    return np.ascontiguousarray(out).reshape(-1)
+
+
+def unpack_prepacked_a16w4(buf: np.ndarray, N: int, K: int):
+    """The inverse of prepack_a16w4, walking the stream address by address: returns (qw [N/2, K] int8 in
+    the reference layout, scale [K/128, N] fp16, zp [K/128, N] fp16)."""
+    buf = np.asarray(buf, dtype=np.uint8)
+    T, KC = N // 16, K // 1024
+    assert buf.size == T * KC * PREPACK_UNIT_BYTES
+    w = np.zeros((N, K), dtype=np.int8)
+    scale = np.zeros((K // 128, N), dtype=np.float16)
+    zp = np.zeros((K // 128, N), dtype=np.float16)
+    for tile in range(T):
+        for kc in range(KC):
+            unit = buf[(tile * KC + kc) * PREPACK_UNIT_BYTES:][:PREPACK_UNIT_BYTES]
+            for b in range(8):
+                for piece in range(64):                     # 16 bytes of channel c, eighths g of four runs of 32
+                    g, c = piece >> 4, piece & 15
+                    raw = unit[1024 * b + 16 * piece:][:16].view("<u4")
+                    for i in range(4):
+                        k = 1024 * kc + 128 * b + 32 * i + 8 * g
+                        for j in range(8):
+                            nibble = (int(raw[i]) >> (4 * ((j >> 1) + 4 * (j & 1)))) & 0xF
+                            w[16 * tile + c, k + j] = nibble - 8
+            tabs = unit[8192:].view("<f2")
+            for c in range(16):
+                for b in range(8):
+                    scale[8 * kc + b, 16 * tile + c] = tabs[8 * c + b]
+                    zp[8 * kc + b, 16 * tile + c] = tabs[128 + 8 * c + b]
+    return pack_int4(w), scale, zp
+
+
 def dequantize_weights(w_nk, scale, zp, scale_dtype: str, group: int) -> np.ndarray:
     """Dequantised weights [K,N] as float32, with the reference's roundings.
 

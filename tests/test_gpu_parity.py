@@ -827,6 +827,88 @@ def test_a16w4_group128_config(M):
     np.testing.assert_allclose(o1[0].float().cpu().numpy(), col.bfloat16().float().numpy(), rtol=2.0 ** -7, atol=1e-6)
 
 
+def test_a16w4_prepacked_decode_config(hip_lib):
+    """The one-token decode on repacked weights at K=8192, N=28672: the device's repacking equals the
+    oracle's packed form byte for byte; the output stays within the tolerance of the oracle on three
+    bands of channels, equals a one-hot probe of every channel, and agrees with the reference-layout
+    kernel everywhere to the same tolerance."""
+    K, N = workloads.A16W4_SHAPE
+    packed, scale, zp_ref, u, zp = workloads.int4_group_weights(N, K, 128)
+    op = flashnn_amd.GemmWeightOnly(torch.bfloat16)
+    pk = op.prepack(packed.to(DEV), scale.to(DEV), zp_ref.to(DEV))
+    assert pk.buffer.numel() == hip_lib.fnn_a16w4_prepacked_bytes(N, K, 128) == N * K // 2 + 4 * (K // 128) * N
+    rows = slice(0, 64)                  # 128 channels = 8 tiles of the packed form, all of K
+    want_pk = O.prepack_a16w4(packed[rows].numpy(), O.to_np(scale[:, :128]), O.to_np(zp_ref[:, :128]))
+    assert np.array_equal(pk.buffer[:want_pk.size].cpu().numpy(), want_pk)
+    last = O.prepack_a16w4(packed[-8:].numpy(), O.to_np(scale[:, -16:]), O.to_np(zp_ref[:, -16:]))
+    assert np.array_equal(pk.buffer[-last.size:].cpu().numpy(), last)
+    act = workloads.activations(1, K, torch.bfloat16, seed=41)
+    out = op.forward_prepacked(act.to(DEV), pk)
+    assert _lib.last_kernel().startswith("gemv_w4_prepacked_kernel") and out.shape == (1, N)
+    for band in [slice(0, 64), slice(14336 - 32, 14336 + 32), slice(N - 64, N)]:
+        w_band = u[band].numpy().astype(np.int16) - 8
+        want = O.weight_only_gemm(O.to_np(act), w_band, O.to_np(scale[:, band]), O.to_np(zp_ref[:, band]), None,
+                                  O.F16, O.BF16, 128, True)
+        np.testing.assert_allclose(out[:, band].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    ref_layout = op(act.to(DEV), packed.to(DEV), scale.to(DEV), None, zp_ref.to(DEV))
+    np.testing.assert_allclose(out.float().cpu().numpy(), ref_layout.float().cpu().numpy(), rtol=RTOL, atol=ATOL)
+    k = 4321
+    e = torch.zeros(1, K, dtype=torch.bfloat16)
+    e[0, k] = 2.0
+    o1 = op.forward_prepacked(e.to(DEV), pk)
+    col = 2.0 * (u[:, k].float() - zp[k // 128].float()) * scale[k // 128].float()
+    np.testing.assert_allclose(o1[0].float().cpu().numpy(), col.bfloat16().float().numpy(), rtol=2.0 ** -7, atol=1e-6)
+
+
+@pytest.mark.parametrize("N,K,act_ty,with_zp,with_bias", [(16, 1024, torch.float16, True, False), (48, 2048, torch.bfloat16, True, True),
+                                                         (4096, 4096, torch.float16, False, True), (1040, 8192, torch.bfloat16, True, False),
+                                                         (12288, 11264, torch.float16, True, True), (8208, 16384, torch.bfloat16, True, False)])
+def test_a16w4_prepacked_shapes(hip_lib, N, K, act_ty, with_zp, with_bias):
+    """Other shapes of the packed decode: one to eleven K ranges (fewer ranges than waves: the waves split
+    the tiles; more: a wave walks several), tile counts that leave workgroups ragged, fp16 and bf16
+    activations with a wide range of magnitudes, with and without zero points and bias - against the
+    oracle, and the repacking against the oracle's byte for byte."""
+    g = torch.Generator().manual_seed(N + K)
+    w = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(K // 128, N).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(-8, 8, (K // 128, N), generator=g).half() if with_zp else None
+    bias = torch.randn(N, generator=g).to(act_ty) if with_bias else None
+    act = torch.randn(1, K, generator=g)
+    act[0, ::7] *= 300.0                 # a wide range of magnitudes inside every K range
+    act[0, 5::64] *= 1e-3
+    act = act.to(act_ty)
+    qw = torch.from_numpy(O.pack_int4(w.numpy()))
+    op = flashnn_amd.GemmWeightOnly(act_ty)
+    pk = op.prepack(qw.to(DEV), scale.to(DEV), None if zp is None else zp.to(DEV))
+    want_pk = O.prepack_a16w4(qw.numpy(), O.to_np(scale), None if zp is None else O.to_np(zp))
+    assert np.array_equal(pk.buffer.cpu().numpy(), want_pk)
+    out = op.forward_prepacked(act.to(DEV), pk, None if bias is None else bias.to(DEV))
+    cols = slice(0, N) if N * K <= 1 << 24 else slice(N - 512, N)
+    want = O.weight_only_gemm(O.to_np(act), w[cols].numpy(), O.to_np(scale[:, cols]), None if zp is None else O.to_np(zp[:, cols]),
+                              None if bias is None else O.to_np(bias[cols]), O.F16, O.tag_of(act), 128, True)
+    got = out[:, cols].float().cpu().numpy()
+    # (activations up to 1000 make outputs of the order of 10^3: the tolerance is the relative one)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL * max(1.0, float(np.abs(want).max()) / 50))
+    full = op(act.to(DEV), qw.to(DEV), scale.to(DEV), None if bias is None else bias.to(DEV), None if zp is None else zp.to(DEV))
+    np.testing.assert_allclose(out.float().cpu().numpy(), full.float().cpu().numpy(), rtol=RTOL,
+                               atol=ATOL * max(1.0, float(full.float().abs().max()) / 50))
+
+
+def test_a16w4_prepacked_argument_errors(hip_lib):
+    """Shapes without a packed form and calls with more than one row are refused, not served wrongly."""
+    f = hip_lib.fnn_a16w4_prepacked_bytes
+    assert f(28672, 8192, 128) == 28672 * 8192 // 2 + 4 * 64 * 28672
+    assert f(28672, 8192, 64) == 0 and f(28680, 8192, 128) == 0 and f(4096, 4224, 128) == 0 and f(4096, 3072, 128) == 0
+    qw = torch.zeros(8, 1024, dtype=torch.int8, device=DEV)
+    scale = torch.ones(8, 16, dtype=torch.float16, device=DEV)
+    pk = flashnn_amd.GemmWeightOnly.prepack(qw, scale)
+    act = torch.zeros(2, 1024, dtype=torch.float16, device=DEV)
+    with pytest.raises(_lib.FlashnnHipError, match="one token"):
+        flashnn_amd.GemmWeightOnly(torch.float16).forward_prepacked(act, pk)
+    with pytest.raises(AssertionError):
+        flashnn_amd.GemmWeightOnly.prepack(qw, scale.bfloat16())
+
+
 @pytest.mark.parametrize("bits,M,N,K", [(4, 1, 24576, 8192), (4, 2, 24576, 8192), (4, 3, 20480, 8192), (4, 4, 28672, 8192),
                                         (8, 1, 12288, 8192), (4, 2, 28672, 4096), (4, 1, 16384, 8192)])
 def test_weight_only_gemv_equal_chunks(bits, M, N, K):

@@ -262,6 +262,41 @@ def test_uint4_with_zero_point_maps_onto_signed_nibbles():
 
 
 # --------------------------------------------------------------------- rmsnorm + quant
+def test_prepacked_a16w4_layout_round_trip_and_addresses():
+    """The packed form of int4 weights: the array-reshape statement of the layout and the address-by-address
+    one are inverses of each other on random inputs; a weight, a scale and a zero point found by hand at
+    the byte the layout's formulas name; the size is the reference layout's; every nibble is used once."""
+    rng = np.random.default_rng(0)
+    for N, K in [(16, 1024), (32, 2048), (48, 4096), (16, 8192)]:
+        w = rng.integers(-8, 8, (N, K)).astype(np.int8)
+        qw = O.pack_int4(w)
+        scale = rng.uniform(1e-3, 1e-2, (K // 128, N)).astype(np.float16)
+        zp = rng.integers(-8, 8, (K // 128, N)).astype(np.float16)
+        buf = O.prepack_a16w4(qw, scale, zp)
+        assert buf.dtype == np.uint8 and buf.size == N * K // 2 + 2 * (K // 128) * N * 2
+        q2, s2, z2 = O.unpack_prepacked_a16w4(buf, N, K)
+        assert np.array_equal(q2, qw) and np.array_equal(s2, scale) and np.array_equal(z2, zp)
+        _, _, z0 = O.unpack_prepacked_a16w4(O.prepack_a16w4(qw, scale, None), N, K)
+        assert not z0.any()
+    # by hand (N = 32, K = 2048): channel 17 = tile 1, c = 1; k = 1485 = 1024 + 3 * 128 + 2 * 32 + 1 * 8 + 5, so
+    # unit (tile 1, kc 1) = number 1 * 2 + 1 = 3, group b = 3, word i = 2, eighth g = 1, value j = 5 at bits
+    # 4 * ((5 >> 1) + 4 * (5 & 1)) = 24: the low nibble of byte 3 of word 2 of the 16 bytes at 16 * (16 g + c)
+    N, K = 32, 2048
+    w = rng.integers(-8, 8, (N, K)).astype(np.int8)
+    scale = rng.uniform(1e-3, 1e-2, (K // 128, N)).astype(np.float16)
+    zp = rng.integers(-8, 8, (K // 128, N)).astype(np.float16)
+    buf = O.prepack_a16w4(O.pack_int4(w), scale, zp)
+    at = 3 * 8704 + 1024 * 3 + 16 * (16 * 1 + 1) + 4 * 2 + 3
+    assert (int(buf[at]) & 0xF) - 8 == int(w[17, 1485])
+    # its group is 8 * 1 + 3 = 11: scale at 8192 + 2 * (8 * c + b), zero point 256 bytes further
+    at = 3 * 8704 + 8192 + 2 * (8 * 1 + 3)
+    assert buf[at:at + 2].view(np.float16)[0] == scale[11, 17]
+    assert buf[at + 256:at + 258].view(np.float16)[0] == zp[11, 17]
+    # the very first word: channel 0, values 0..7, value j in nibble (j >> 1) + 4 (j & 1)
+    first = int(buf[:4].view("<u4")[0])
+    assert [((first >> (4 * ((j >> 1) + 4 * (j & 1)))) & 0xF) - 8 for j in range(8)] == [int(v) for v in w[0, :8]]
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(4, 128), (3, 32, 1024), (16, 8192)])
 def test_rmsnorm_dquant_matches_torch_ops(dtype, shape):
