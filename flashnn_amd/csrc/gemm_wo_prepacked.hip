@@ -176,7 +176,14 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemv_w4_prepacked_kernel(const 
             grp_c[b] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(-1024.f * S), 8 * b));
             grp_a[b] = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(A), 8 * b));
         }
-        // (LDS operations of one wave complete in order: what follows reads what was written above)
+        // The 32 activation operands of this lane (8 groups x 4 instructions; they depend on g alone) are
+        // read back once and stay in registers over all tiles: no LDS traffic inside the stream.  (LDS
+        // operations of one wave complete in order: the reads see what was written above.)
+        v4u areg[8][4];
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) areg[b][i] = *(const v4u*)(my_act + b * 256 + i * 64 + g * 16);
 
         // the fp16 pair (1024, 1024), kept in a register the compiler cannot see through: (w & m) | (k & ~m)
         // is then one bit-field insert instead of an and and an or with a literal each
@@ -209,8 +216,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemv_w4_prepacked_kernel(const 
                     const uint32_t wi = w[i], w8 = wi >> 8;
                     const v4u x = v4u{(wi & 0x000F000Fu) | (k1024 & ~0x000F000Fu), (wi & 0x00F000F0u) | (k1024 & ~0x00F000F0u),
                                       (w8 & 0x000F000Fu) | (k1024 & ~0x000F000Fu), (w8 & 0x00F000F0u) | (k1024 & ~0x00F000F0u)};
-                    const v4u a = *(const v4u*)(my_act + b * 256 + i * 64 + g * 16);
-                    d = MfmaT<FNN_F16>::mma(a, x, d);
+                    d = MfmaT<FNN_F16>::mma(areg[b][i], x, d);
                 }
                 const float sb = f16_bits_to_f32((sraw[b >> 1] >> (16 * (b & 1))) & 0xFFFFu);
                 const float z8 = 8.f + f16_bits_to_f32((zraw[b >> 1] >> (16 * (b & 1))) & 0xFFFFu);
