@@ -81,8 +81,9 @@ struct OptionalStage<false, BYTES> {
 // zero whenever no call is in flight.
 template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2, bool SPLIT = false>
 __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Args p) {
-    // WGM x 2 waves.  WGM = 4 puts two waves on every SIMD (at most 256 registers each): one can issue
-    // MFMAs while the other waits for LDS fragments, a copy or the barrier.
+    // WGM x 2 waves.  Only WGM = 2 (one wave per SIMD) is instantiated: with WGM = 4 the two waves of a SIMD
+    // meet at the same barrier every slab and never filled each other's gaps (256x192: 81.6 us with four
+    // waves, 83.9 with eight; never faster on any shape tried).
     constexpr int NWAVES = WGM * 2, NT = NWAVES * 64;
     constexpr int WTM = BM / WGM, WTN = BN / 2;
     constexpr int FM = WTM / 16, FN = WTN / 16;   // 16x16 fragments per wave tile
@@ -777,18 +778,12 @@ static bool valid_tile(int bm, int bn, int waves) {
     if (bm == 0 && bn == 0) return waves == 0;
     if (waves == 0 || waves == 4)
         return (bm == 256 && (bn == 256 || bn == 192 || bn == 128)) || (bm == 128 && bn == 128) || (bm == 64 && bn == 128);
-    if (waves == 8) return bm == 256 && (bn == 256 || bn == 192 || bn == 128);
     return false;
 }
 
 template <int MODE>
 static void launch_tile(A8W8Args& p, hipStream_t st, int bm, int bn, int waves) {
-    if (waves == 8) {
-        if (bn == 256) launch_mfma<256, 256, MODE, false, 4>(p, st);
-        else if (bn == 192) launch_mfma<256, 192, MODE, false, 4>(p, st);
-        else launch_mfma<256, 128, MODE, false, 4>(p, st);
-    }
-    else if (bm == 256 && bn == 192) launch_mfma<256, 192, MODE>(p, st);
+    if (bm == 256 && bn == 192) launch_mfma<256, 192, MODE>(p, st);
     else if (bm == 256 && bn == 256) launch_mfma<256, 256, MODE>(p, st);
     else if (bm == 256 && bn == 128) launch_mfma<256, 128, MODE>(p, st);
     else if (bm == 64 && bn == 128) launch_mfma<64, 128, MODE>(p, st);

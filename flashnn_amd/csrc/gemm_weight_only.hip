@@ -1517,7 +1517,10 @@ static int run_wo(const char* fn, void* out, const void* act, const void* qw, co
         set_error("%s: scale / zero-point / bias type must be fp16, bf16 or fp32", fn);
         return FNN_ERR_UNSUPPORTED;
     }
-    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) { set_error("%s: shape too large", fn); return FNN_ERR_UNSUPPORTED; }
+    if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30) || lda > (1LL << 30) || ldw > (1LL << 30)) {
+        set_error("%s: shape or row stride too large", fn);
+        return FNN_ERR_UNSUPPORTED;
+    }
     if (M == 0 || N == 0) return FNN_OK;
     WoArgs p{};
     p.act = act; p.qw = (const int8_t*)qw; p.scale = scale; p.zp = zp; p.bias = bias; p.out = out;

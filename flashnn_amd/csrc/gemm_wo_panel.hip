@@ -674,6 +674,9 @@ bool launch_wo_panel_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t
 }
 
 bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st) {
+    // the kernel addresses the up to 64 rows of a pass and the 8 weight rows of a load with 32-bit offsets
+    // from a 64-bit base: strides that do not fit go to the other kernels
+    if (64 * p.lda * 2 >= (1LL << 32) || 8 * p.ldw >= (1LL << 32)) return false;
     if (wbits == 4) return act_dtype == FNN_F16 ? launch_panel_t<4, FNN_F16>(p, st) : launch_panel_t<4, FNN_BF16>(p, st);
     return act_dtype == FNN_F16 ? launch_panel_t<8, FNN_F16>(p, st) : launch_panel_t<8, FNN_BF16>(p, st);
 }

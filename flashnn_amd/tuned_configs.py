@@ -11,7 +11,7 @@ recorded configurations are still honoured; shapes without one take the library'
 
 File format (the reference's, triton_utils.py:38-57): {method_name: [kwargs, launch_options]} with
 kwargs = {"BLOCK_M": .., "BLOCK_N": ..} ((0, 0) = the library's own choice) and launch_options =
-{"num_warps": 4 or 8} (absent = the tile's default), the reference's own option names (gemm_a8w8.py:17-50).
+{"num_warps": 4} (absent = the tile's default; every tile runs four waves), the reference's own option names (gemm_a8w8.py:17-50).
 The file lives at $FLASHNN_AMD_TUNED_CONFIGS or flashnn_amd/configs/hip_autotune_best_configs.json.
 FORECE_RE_TUNE_TRITON_KERNELS (the reference's spelling, triton_utils.py:22-24) lists method-name
 prefixes, separated by ';', that are tuned again even if recorded.
@@ -24,8 +24,7 @@ JSON_FILENAME = "hip_autotune_best_configs.json"
 
 # candidate (rows, columns, waves) of the A8W8 MFMA kernel; (0, 0, 0) = static choice (which may be a
 # few-row kernel); waves = 0 is the tile's default (four)
-A8W8_CANDIDATES = [(0, 0, 0), (256, 256, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0),
-                   (256, 256, 8), (256, 192, 8), (256, 128, 8)]
+A8W8_CANDIDATES = [(0, 0, 0), (256, 256, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0)]
 
 
 def json_file_path():

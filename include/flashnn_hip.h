@@ -196,9 +196,8 @@ int fnn_layernorm_dquant(void* q, void* scale, const void* x, const void* gamma,
 
 /*
  * fnn_gemm_a8w8 with the output tile of the MFMA kernel chosen by the caller: (tile_m, tile_n, waves) with
- * waves = 4 (or 0: the tile's default) and the tile one of 256x256, 256x192, 256x128, 128x128, 64x128, or waves = 8
- * (two wavefronts on every SIMD) and the tile one of 256x256, 256x192, 256x128; (0, 0, 0) is the library's
- * own choice.  A named tile also bypasses the few-row kernels.  This is what a shape-keyed
+ * waves = 4 (or 0: the tile's default) and the tile one of 256x256, 256x192, 256x128, 128x128, 64x128; (0, 0, 0)
+ * is the library's own choice.  A named tile also bypasses the few-row kernels.  This is what a shape-keyed
  * tuned-configuration cache calls - the role that compile_and_cache_kernels and its JSON file play in the
  * reference (flashnn/triton_kernels/triton_utils.py:84-151; method name "gemm_a8w8_M_N_K",
  * gemm_a8w8.py:199; `waves` is the num_warps of its launch options, gemm_a8w8.py:17-50).

@@ -107,8 +107,7 @@ def _rand_i8(shape, seed, lo=-128, hi=128):
 
 
 # every tile of the MFMA kernel: (rows, columns, waves); (0, 0, 0) = the library's own choice
-TILES = [(0, 0, 0), (256, 256, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0), (256, 256, 8),
-         (256, 192, 8), (256, 128, 8)]
+TILES = [(0, 0, 0), (256, 256, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0), (256, 256, 4)]
 
 
 def _scaled(out_ty, a, b, ar, ac, tile):
@@ -147,8 +146,7 @@ def test_a8w8_partial_last_slab_bit_exact(tile, mnk):
 @pytest.mark.parametrize("tile,mn", [((64, 128, 0), (720, 773)), ((64, 128, 0), (1100, 300)),
                                      ((128, 128, 0), (1290, 650)), ((256, 128, 0), (2310, 1100)),
                                      ((256, 192, 0), (2400, 1000)), ((256, 192, 0), (2600, 200)),
-                                     ((256, 192, 8), (2400, 1000)), ((256, 256, 8), (2600, 1300)),
-                                     ((256, 128, 8), (2310, 1100))])
+                                     ((256, 256, 0), (2600, 1300))])
 def test_a8w8_tile_numbering_many_tile_rows(tile, mn):
     """More than 8 tile rows and a number of tile columns that is no multiple of 4: the tiles are numbered
     in groups of 4 tile columns, and the last group is narrower."""

@@ -57,6 +57,22 @@ def test_argument_errors_are_reported_without_a_gpu(hip_lib):
     assert rc == -1 and b"even" in hip_lib.fnn_last_error()
     rc = hip_lib.fnn_gemm_a16w8(one, one, one, one, null, null, 1, 8, 100, 100, 100, 8, 64, 0, 0, 0, 0, 0, null)
     assert rc == -1 and b"multiple of the group" in hip_lib.fnn_last_error()
+    # row strides the kernels' 32-bit row offsets cannot reach are refused, not wrapped
+    rc = hip_lib.fnn_gemm_a16w8(one, one, one, one, null, null, 4, 64, 1024, 1 << 31, 1024, 64, 0, 0, 0, 0, 0, 0, null)
+    assert rc == -2 and b"row stride too large" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a16w4(one, one, one, one, null, null, 4, 64, 1024, 1024, 1 << 31, 64, 0, 0, 0, 0, 0, 0, null)
+    assert rc == -2 and b"row stride too large" in hip_lib.fnn_last_error()
+    # the packed int4 form: shapes without one, more than one row, and bad table types are refused
+    assert hip_lib.fnn_a16w4_prepacked_bytes(28672, 8192, 128) == 28672 * 8192 // 2 + 4 * 64 * 28672
+    assert hip_lib.fnn_a16w4_prepacked_bytes(28672, 8192, 64) == 0 and hip_lib.fnn_a16w4_prepacked_bytes(24, 8192, 128) == 0
+    assert hip_lib.fnn_a16w4_prepacked_bytes(4096, 3072, 128) == 0 and hip_lib.fnn_a16w4_prepacked_bytes(4096, 4000, 128) == 0
+    rc = hip_lib.fnn_a16w4_prepack(one, one, one, null, 64, 1024, 1024, 128, 1, 0, null)       # bf16 scales
+    assert rc == -2 and b"fp16 scales" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_a16w4_prepack(one, one, one, null, 64, 1000, 1000, 128, 0, 0, null)
+    assert rc == -2 and b"packed form needs" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a16w4_prepacked(one, one, one, null, 2, 64, 1024, 1024, 64, 128, 0, 0, 0, null)
+    assert rc == -2 and b"one token" in hip_lib.fnn_last_error()
+    assert hip_lib.fnn_gemm_a16w4_prepacked(null, null, null, null, 0, 64, 1024, 1024, 64, 128, 0, 0, 0, null) == 0
     # empty problems are a no-op
     assert hip_lib.fnn_gemm_a8w8_i32(one, one, one, 0, 4, 128, 128, 128, 4, null) == 0
 
@@ -154,14 +170,14 @@ def test_tuned_config_file_format_and_lookup(tmp_path, monkeypatch):
     monkeypatch.delenv("FORECE_RE_TUNE_TRITON_KERNELS", raising=False)
     cache = TC.TunedConfigs()
     assert cache.lookup("gemm_a8w8_2048_12288_4096") is None
-    cache.record("gemm_a8w8_2048_12288_4096", (256, 192, 8))
+    cache.record("gemm_a8w8_2048_12288_4096", (256, 192, 4))
     cache.record("gemm_a8w8_16_4096_4096", (0, 0, 0))
     data = json.load(open(path))
-    assert data == {"gemm_a8w8_2048_12288_4096": [{"BLOCK_M": 256, "BLOCK_N": 192}, {"num_warps": 8}],
+    assert data == {"gemm_a8w8_2048_12288_4096": [{"BLOCK_M": 256, "BLOCK_N": 192}, {"num_warps": 4}],
                     "gemm_a8w8_16_4096_4096": [{"BLOCK_M": 0, "BLOCK_N": 0}, {}]}
     # a fresh view (another process) reads the file back
     other = TC.TunedConfigs()
-    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 192, 8) and other.lookup("gemm_a8w8_1_1_1") is None
+    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 192, 4) and other.lookup("gemm_a8w8_1_1_1") is None
     # forced re-tune by method-name prefix, once per process
     monkeypatch.setenv("FORECE_RE_TUNE_TRITON_KERNELS", "gemm_a8w8_2048;fuse_moe")
     assert TC.force_re_tune("gemm_a8w8_2048_12288_4096") and not TC.force_re_tune("gemm_a8w8_16_4096_4096")
@@ -178,7 +194,7 @@ def test_tuned_config_file_format_and_lookup(tmp_path, monkeypatch):
     assert other.shape_tile("gemm_a8w8", 1, 1, 1) is None
     assert TC.serialize_best_config((128, 128)) == [{"BLOCK_M": 128, "BLOCK_N": 128}, {}]
     assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 192}, {}]) == (256, 192, 0)
-    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 256}, {"num_warps": 8}]) == (256, 256, 8)
+    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 256}, {"num_warps": 4}]) == (256, 256, 4)
 
 
 def test_tiled_entry_rejects_unknown_tiles(hip_lib):
@@ -190,6 +206,8 @@ def test_tiled_entry_rejects_unknown_tiles(hip_lib):
     assert rc == -1 and b"no such tile 128x128 with 8 waves" in hip_lib.fnn_last_error()
     rc = hip_lib.fnn_gemm_a8w8_i32_tiled(one, one, one, 4, 4, 128, 128, 128, 4, 64, 128, 8, null)
     assert rc == -1 and b"no such tile 64x128 with 8 waves" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a8w8_tiled(one, one, one, one, one, 4, 4, 128, 128, 128, 4, 0, 0, 0, 256, 192, 8, null)
+    assert rc == -1 and b"no such tile 256x192 with 8 waves" in hip_lib.fnn_last_error()
 
 
 def test_a8w8_rejects_row_strides_beyond_the_band_logic(hip_lib):
