@@ -34,6 +34,9 @@ _SIGNATURES = {
     "fnn_gemm_a8w8_i32_tiled": [_ptr] * 3 + [_i64] * 6 + [_int] * 3 + [_ptr],
     "fnn_gemm_a16w8": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],
     "fnn_gemm_a16w4": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr],
+    "fnn_gemm_weight_only_workspace_bytes": [_i64] * 4 + [_int] * 2,
+    "fnn_gemm_a16w8_ws": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr, _size, _ptr],
+    "fnn_gemm_a16w4_ws": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr, _size, _ptr],
     "fnn_a16w4_prepacked_bytes": [_i64] * 3,
     "fnn_a16w4_prepack": [_ptr] * 4 + [_i64] * 4 + [_int] * 2 + [_ptr],
     "fnn_gemm_a16w4_prepacked": [_ptr] * 4 + [_i64] * 6 + [_int] * 3 + [_ptr],
@@ -41,7 +44,8 @@ _SIGNATURES = {
     "fnn_fused_moe_a16w4": [_ptr] * 9 + [_i64] * 14 + [_int] * 8 + [_ptr],
 }
 _RESTYPE = {"fnn_last_error": ctypes.c_char_p, "fnn_last_kernel": ctypes.c_char_p,
-            "fnn_gemm_a8w8_workspace_bytes": ctypes.c_size_t, "fnn_a16w4_prepacked_bytes": ctypes.c_size_t}
+            "fnn_gemm_a8w8_workspace_bytes": ctypes.c_size_t, "fnn_a16w4_prepacked_bytes": ctypes.c_size_t,
+            "fnn_gemm_weight_only_workspace_bytes": ctypes.c_size_t}
 
 _lib = None
 

@@ -1462,6 +1462,65 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
     return true;
 }
 
+// ---- bf16 activation rows -> fp16 rows (for the kernels that round every weight as the reference does)
+// One 256-thread workgroup per row.  The row's largest magnitude is brought to [2^13, 2^14) by a power of two,
+// so every bf16 value (8 significant bits) whose magnitude is within 2^-30 of the row's largest becomes an
+// fp16 value without loss and nothing overflows; smaller ones lose low bits that could not move the output.
+// The inverse power goes to unscale[row]; rows of zeros or with non-finite values are left unscaled.
+__global__ __launch_bounds__(256) void act_bf16_to_f16_kernel(uint16_t* dst, float* unscale, const uint16_t* src, int K,
+                                                              int64_t lda) {
+    __shared__ uint32_t smax[4];
+    const int row = blockIdx.x;
+    const uint16_t* in = src + (int64_t)row * lda;
+    uint16_t* out = dst + (int64_t)row * K;
+    uint32_t mx = 0;            // magnitudes compare like their bit patterns
+    for (int k = threadIdx.x * 8; k < K; k += 256 * 8) {
+        const v4u v = *(const v4u*)(in + k);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            mx = max(mx, v[i] & 0x7FFFu);
+            mx = max(mx, (v[i] >> 16) & 0x7FFFu);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o, 64));
+    if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = max(max(smax[0], smax[1]), max(smax[2], smax[3]));
+    const int ex = (int)(mx >> 7);
+    const int sh = (ex == 0 || ex == 255) ? 0 : max(-100, min(100, 13 - (ex - 127)));
+    const float up = __uint_as_float((uint32_t)(127 + sh) << 23);
+    if (threadIdx.x == 0) unscale[row] = __uint_as_float((uint32_t)(127 - sh) << 23);
+    for (int k = threadIdx.x * 8; k < K; k += 256 * 8) {
+        const v4u v = *(const v4u*)(in + k);
+        v4u o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = __uint_as_float(v[i] << 16) * up, hi = __uint_as_float(v[i] & 0xFFFF0000u) * up;
+            o[i] = f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+        }
+        *(v4u*)(out + k) = o;
+    }
+}
+
+size_t act_f16_ws_bytes(int64_t M, int64_t K) { return (size_t)((M * K * 2 + 255) / 256 * 256) + (size_t)M * sizeof(float); }
+
+bool convert_act_to_f16(const WoArgs& p, WoArgs& q, hipStream_t st) {
+    if (!p.cvt_ws || p.cvt_ws_bytes < act_f16_ws_bytes(p.M, p.K) || ((uintptr_t)p.cvt_ws % 16) != 0) return false;
+    if (p.scale_dtype != FNN_F16 || (p.zp && p.zp_dtype != FNN_F16) || (p.group != 0 && p.group != 128)) return false;
+    if (p.K % 8 != 0 || p.lda % 8 != 0 || ((uintptr_t)p.act % 16) != 0 || p.m_base != 0) return false;
+    q = p;
+    q.act = p.cvt_ws;
+    q.lda = p.K;
+    q.act_unscale = (const float*)((char*)p.cvt_ws + (size_t)(((int64_t)p.M * p.K * 2 + 255) / 256 * 256));
+    q.cvt_ws = nullptr;
+    q.cvt_ws_bytes = 0;
+    note_kernel("act_bf16_to_f16_kernel");
+    act_bf16_to_f16_kernel<<<dim3(p.M), dim3(256), 0, st>>>((uint16_t*)p.cvt_ws, (float*)q.act_unscale,
+                                                            (const uint16_t*)p.act, p.K, p.lda);
+    return true;
+}
+
 template <int WBITS, int ADT>
 static void dispatch_wo(WoArgs& p, hipStream_t st) {
     const bool aligned = p.K % 64 == 0 && p.ldw % 16 == 0 && p.lda % 8 == 0 && ((uintptr_t)p.qw % 16) == 0 &&
@@ -1501,7 +1560,8 @@ template <int WBITS>
 static int run_wo(const char* fn, void* out, const void* act, const void* qw, const void* scale,
                   const void* bias, const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldw, int64_t ldc, int64_t group, int act_dtype, int out_dtype,
-                  int scale_dtype, int zp_dtype, int bias_dtype, void* stream) {
+                  int scale_dtype, int zp_dtype, int bias_dtype, void* stream, void* workspace = nullptr,
+                  size_t ws_bytes = 0) {
     // an empty tensor has no address: pointers are only required when there is something to compute
     if (M != 0 && N != 0 && (!out || !act || !qw || !scale)) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
     if (M < 0 || N < 0 || K <= 0 || lda < K || ldw < K || ldc < N || group < 0) {
@@ -1526,6 +1586,8 @@ static int run_wo(const char* fn, void* out, const void* act, const void* qw, co
     p.act = act; p.qw = (const int8_t*)qw; p.scale = scale; p.zp = zp; p.bias = bias; p.out = out;
     p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = lda; p.ldw = ldw; p.ldc = ldc; p.group = (int)group;
     p.out_dtype = out_dtype; p.scale_dtype = scale_dtype; p.zp_dtype = zp_dtype; p.bias_dtype = bias_dtype;
+    if (ws_bytes > 0 && !workspace) { set_error("%s: a workspace size without a workspace", fn); return FNN_ERR_ARG; }
+    p.cvt_ws = workspace; p.cvt_ws_bytes = ws_bytes;
     const Call call(fn);
     if (act_dtype == FNN_F16) dispatch_wo<WBITS, FNN_F16>(p, (hipStream_t)stream);
     else dispatch_wo<WBITS, FNN_BF16>(p, (hipStream_t)stream);
@@ -1552,6 +1614,31 @@ extern "C" int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const 
                               void* stream) {
     return run_wo<4>("fnn_gemm_a16w4", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group,
                      act_dtype, out_dtype, scale_dtype, zp_dtype, bias_dtype, stream);
+}
+
+extern "C" size_t fnn_gemm_weight_only_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int act_dtype,
+                                                       int scale_dtype) {
+    // bf16 activations with fp16 tables, more than 64 rows (the tiled kernel): the rows are converted to fp16
+    // once, so that every weight can be rounded as the reference rounds it
+    if (M <= 64 || N <= 0 || K <= 0 || K % 8 != 0 || M > (1 << 30) || K > (1 << 30)) return 0;
+    if (act_dtype != FNN_BF16 || scale_dtype != FNN_F16 || (group != 0 && group != 128)) return 0;
+    return act_f16_ws_bytes(M, K);
+}
+
+extern "C" int fnn_gemm_a16w8_ws(void* out, const void* act, const void* qw, const void* scale, const void* bias,
+                                 const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                                 int64_t group, int act_dtype, int out_dtype, int scale_dtype, int zp_dtype,
+                                 int bias_dtype, void* workspace, size_t ws_bytes, void* stream) {
+    return run_wo<8>("fnn_gemm_a16w8_ws", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group, act_dtype,
+                     out_dtype, scale_dtype, zp_dtype, bias_dtype, stream, workspace, ws_bytes);
+}
+
+extern "C" int fnn_gemm_a16w4_ws(void* out, const void* act, const void* qw, const void* scale, const void* bias,
+                                 const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                                 int64_t group, int act_dtype, int out_dtype, int scale_dtype, int zp_dtype,
+                                 int bias_dtype, void* workspace, size_t ws_bytes, void* stream) {
+    return run_wo<4>("fnn_gemm_a16w4_ws", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group, act_dtype,
+                     out_dtype, scale_dtype, zp_dtype, bias_dtype, stream, workspace, ws_bytes);
 }
 
 // ------------------------------------------------------------------ mixture of experts, int4 weights

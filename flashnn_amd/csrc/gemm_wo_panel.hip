@@ -44,7 +44,12 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // single pass over the weights.
 // REFQ (1, or 2 with zero points; fp16 activations, per-channel fp16 scales and zero points): every weight is dequantised and rounded to
 // fp16 as the reference's torch path does before the dot product (ref_dq_f16 in wo_common.h); the MFMAs
-// against ones and the fold at the end are then not needed.
+// against ones and the fold at the end are then not needed.  (The same with tables per group of 128 - a
+// lane fetching its row's scale and zero point slab by slab, bf16 rows converted to fp16 by a pass of their
+// own - was built and measured on A16W4, K = 8192, N = 28672: 16 rows 28.0 -> 38.5 us, 64 rows 52.5 -> 56.5 us.
+// Three more instructions per pair of weights where the fold costs two per output and slab: at these row
+// counts the kernel streams weights, and the vector unit has no room for it.  Not kept; the tiled kernel for
+// more than 64 rows has it.)
 template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL, bool MOE = false, int REFQ = 0>
 __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, const int passes, const MoeArgs q) {
     static_assert(!REFQ || (ADT == FNN_F16 && !G128 && !MOE), "reference rounding: fp16, per-channel");

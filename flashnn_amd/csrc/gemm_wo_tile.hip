@@ -35,8 +35,16 @@ namespace fnn {
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
-template <int WBITS, int ADT, bool G128, int SDT, int BM>
+// REFQ (1, or 2 with zero points; fp16 activations, fp16 scales and zero points, per channel or per group of
+// 128): every weight is dequantised and rounded to fp16 as the reference's torch path does before the dot
+// product, (q - zp) * s with both operations rounded (ref_dq_f16 in wo_common.h; flashnn/quant_gemm.py:14-36).
+// The accumulators then run over all of K: no MFMAs against ones, no fold per slab, no second accumulator
+// set, and the result differs from the reference's only by the order of the fp32 additions.  bf16
+// activations reach this form through the conversion pass of gemm_weight_only.hip (rows scaled by a power
+// of two, p.act_unscale undoes it).
+template <int WBITS, int ADT, bool G128, int SDT, int BM, int REFQ = 0>
 __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const int tiles_m, const int tiles) {
+    static_assert(!REFQ || (ADT == FNN_F16 && SDT == FNN_F16), "reference rounding: fp16 activations and tables");
     typedef MfmaT<ADT> MT;
     static_assert(WBITS == 4 || BM == 128, "three stages of 128 int8 weight rows leave room for 128 activation rows");
     constexpr int NH = WBITS == 4 ? 2 : 1;          // channels per weight row
@@ -157,6 +165,18 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     const float zmul = has_zp ? 1.f : 0.f;
     typedef typename std::conditional<NH == 2, v4u, v2u>::type tab_t;
 
+    // REFQ with per-channel tables: the scale and zero point of the channels this lane's operand rows hold
+    const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
+    v2h rq_s[NA], rq_z[NA];
+    if constexpr (REFQ != 0 && !G128) {
+#pragma unroll
+        for (int a = 0; a < NA; ++a) {
+            const int n = n0 + wn * WTN + (a / NH) * 16 * NH + NH * row16 + (a % NH);
+            rq_s[a] = pair_of_f16_bits(((const uint16_t*)p.scale)[n]);
+            rq_z[a] = pair_of_f16_bits(p.zp ? ((const uint16_t*)p.zp)[n] : 0u);
+        }
+    }
+
     // One slab.  All of the slab's weights are converted first (A operand a of k-step ks; int4: operand
     // 2 f + (0 even, 1 odd channel) of fragment f, int8: operand = fragment).  Then one activation fragment
     // at a time: its four k-steps against all operands (five independent MFMA chains, the fifth against
@@ -247,6 +267,113 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
         }
     };
 
+    if constexpr (REFQ != 0) {
+        // ---- per-weight rounding: a software pipeline over the slabs.  While the MFMAs of slab j run on
+        // operands that are already dequantised in registers, the weights of slab j + 1 are read from LDS,
+        // converted and dequantised into a second set - vector instructions placed between the MFMAs, two
+        // per MFMA - so that the matrix cores and the vector unit of a SIMD work at the same time although
+        // both waves of the SIMD cross the same barrier every slab.  The weight stage of slab j is free
+        // from barrier j on (its operands were formed during slab j - 1), so the weights are copied three
+        // slabs ahead into three stages, the tables two ahead.
+        v4u A0[4][NA], A1[4][NA];
+        auto dequant_slab = [&](v4u(&A)[4][NA], const char* sw, const char* stg) {
+            if constexpr (G128) {
+#pragma unroll
+                for (int a = 0; a < NA; ++a) {
+                    const int ch = wn * WTN + (a / NH) * 16 * NH + NH * row16 + (a % NH);
+                    rq_s[a] = pair_of_f16_bits(*(const uint16_t*)(stg + ch * 2));
+                    rq_z[a] = pair_of_f16_bits(REFQ == 2 ? *(const uint16_t*)(stg + 256 + ch * 2) : 0u);
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int f = 0; f < NF; ++f) {
+                    const v4u w = *(const v4u*)(sw + w_rd[h] + f * 16 * 128);
+                    if constexpr (WBITS == 4)
+                        convert_w4_nat<ADT>(w, A[2 * h][2 * f], A[2 * h + 1][2 * f], A[2 * h][2 * f + 1], A[2 * h + 1][2 * f + 1]);
+                    else
+                        convert_w8<ADT>(w, A[2 * h][f], A[2 * h + 1][f]);
+                }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int a = 0; a < NA; ++a) A[ks][a] = ref_dq_f16<REFQ == 2>(A[ks][a], rq_c, rq_z[a], rq_s[a]);
+        };
+        auto mfma_slab = [&](const v4u(&A)[4][NA], const char* sa) {
+#pragma unroll
+            for (int b = 0; b < FB; ++b) {
+                v4u B[4];
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) B[ks] = *(const v4u*)(sa + a_rd[ks >> 1][ks & 1] + b * 16 * 256);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                    for (int a = 0; a < NA; ++a) outv[a][b] = MT::mma(A[ks][a], B[ks], outv[a][b]);
+            }
+        };
+        // the order asked of the scheduler: per activation fragment its four LDS reads, then each of its MFMAs
+        // followed by two vector instructions of the dequantisation (what is left of those comes last)
+        auto interleave = [&]() {
+            // (first the LDS reads of the dequantisation: 2 NF weight pieces and, with group tables, 2 NA entries)
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * NF + (G128 ? 2 * NA : 0), 0);
+#pragma unroll
+            for (int b = 0; b < FB; ++b) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+                for (int q = 0; q < 4 * NA; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                }
+            }
+        };
+#define FNN_RQ_ITER(CUR, NXT, CA, CWN, CTN, FA, FW, FT, J)                \
+    do {                                                                  \
+        wait_barrier();                                                   \
+        copy_a(FA, (J) + 1);                                              \
+        copy_t(FT, (J) + 2);                                              \
+        copy_w(FW, (J) + 3);                                              \
+        __builtin_amdgcn_sched_barrier(0);                                \
+        dequant_slab(NXT, CWN, CTN);                                      \
+        mfma_slab(CUR, CA);                                               \
+        interleave();                                                     \
+        __builtin_amdgcn_sched_barrier(0);                                \
+    } while (0)
+        // prologue: the weights and tables of slab 0 first (they are waited for at once), then what the loop
+        // would have issued before its first barrier
+        copy_w(sw0, 0);
+        copy_t(st0, 0);
+        copy_a(sa0, 0);
+        copy_t(st1, 1);
+        copy_w(sw1, 1);
+        copy_w(sw2, 2);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0070 | ((NCA + NCT + 2 * NCW) & 15) | (((NCA + NCT + 2 * NCW) >> 4) << 14));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        dequant_slab(A0, sw0, st0);
+        __builtin_amdgcn_sched_barrier(0);
+        int j = 0;
+        for (; j + 6 <= KT; j += 6) {
+            FNN_RQ_ITER(A0, A1, sa0, sw1, st1, sa1, sw0, st2, j);
+            FNN_RQ_ITER(A1, A0, sa1, sw2, st2, sa0, sw1, st0, j + 1);
+            FNN_RQ_ITER(A0, A1, sa0, sw0, st0, sa1, sw2, st1, j + 2);
+            FNN_RQ_ITER(A1, A0, sa1, sw1, st1, sa0, sw0, st2, j + 3);
+            FNN_RQ_ITER(A0, A1, sa0, sw2, st2, sa1, sw1, st0, j + 4);
+            FNN_RQ_ITER(A1, A0, sa1, sw0, st0, sa0, sw2, st1, j + 5);
+        }
+        // (KT is a multiple of 2: the remaining slabs come in pairs and the operand sets line up)
+        if (j < KT) {
+            FNN_RQ_ITER(A0, A1, sa0, sw1, st1, sa1, sw0, st2, j);
+            FNN_RQ_ITER(A1, A0, sa1, sw2, st2, sa0, sw1, st0, j + 1);
+        }
+        if (j + 2 < KT) {
+            FNN_RQ_ITER(A0, A1, sa0, sw0, st0, sa1, sw2, st1, j + 2);
+            FNN_RQ_ITER(A1, A0, sa1, sw1, st1, sa0, sw0, st2, j + 3);
+        }
+#undef FNN_RQ_ITER
+    } else {
 #define FNN_TILE_ITER(CA, CW, CT, FA, FW, FT, J)                          \
     do {                                                                  \
         wait_barrier();                                                   \
@@ -280,8 +407,9 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     if (j + 2 < KT) { FNN_TILE_ITER(sa0, sw2, st2, sa1, sw1, st0, j + 2); }
     if (j + 3 < KT) { FNN_TILE_ITER(sa1, sw0, st0, sa0, sw2, st1, j + 3); }
 #undef FNN_TILE_ITER
+    }
     // ---- per-channel scales: one fold at the end
-    if constexpr (!G128) {
+    if constexpr (!G128 && REFQ == 0) {
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
             float sc[4], zc[4];
@@ -312,12 +440,14 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
         for (int b = 0; b < FB; ++b) {
             const int m = m0 + wm * WTM + b * 16 + row16;
             if (m >= p.M) continue;
+            // (rows converted from bf16 were scaled by a power of two: the exact inverse)
+            const float un = REFQ != 0 && p.act_unscale ? p.act_unscale[m] : 1.f;
             uint32_t pk[2 * NH];
 #pragma unroll
             for (int c = 0; c < 4 * NH; c += 2) {
                 // channel c of the lane: int4: register c >> 1 of operand 2 f + (c & 1); int8: register c of operand f
-                const float v0 = (NH == 2 ? outv[2 * f][b][c >> 1] : outv[f][b][c]) + bias[c];
-                const float v1 = (NH == 2 ? outv[2 * f + 1][b][c >> 1] : outv[f][b][c + 1]) + bias[c + 1];
+                const float v0 = (NH == 2 ? outv[2 * f][b][c >> 1] : outv[f][b][c]) * un + bias[c];
+                const float v1 = (NH == 2 ? outv[2 * f + 1][b][c >> 1] : outv[f][b][c + 1]) * un + bias[c + 1];
                 const uint32_t b0 = out_f16 ? f32_to_f16_bits(v0) : f32_to_bf16_bits(v0);
                 const uint32_t b1 = out_f16 ? f32_to_f16_bits(v1) : f32_to_bf16_bits(v1);
                 pk[c >> 1] = (b0 & 0xFFFFu) | (b1 << 16);
@@ -348,26 +478,41 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
                               ((uintptr_t)p.scale % 16) == 0 && (!p.zp || ((uintptr_t)p.zp % 16) == 0);
         if (!tables16) return false;
     }
+    if constexpr (ADT == FNN_BF16) {
+        // bf16 rows become fp16 rows where scratch was given: the weights are then rounded as the reference does
+        WoArgs q;
+        if (convert_act_to_f16(p, q, st) && launch_tile_t<WBITS, FNN_F16>(q, st)) return true;
+    }
     const int bm = (p.M <= 128 || WBITS == 8) ? 128 : 256;
     const int tiles_m = (p.M + bm - 1) / bm;
     const int tiles = tiles_m * (p.N / 128);
     const dim3 grid(((tiles + 7) / 8) * 8);   // (workgroups beyond the last tile return at once)
-    note_kernel("gemm_wo_tile_kernel", WBITS, bm, 128);
-#define FNN_TILE(G, SDTV)                                                                                \
+    // fp16 activations with fp16 tables: every weight rounded as the reference rounds it
+    const bool refq = ADT == FNN_F16 && p.scale_dtype == FNN_F16 && (!p.zp || p.zp_dtype == FNN_F16) &&
+                      (p.group == 128 || ((uintptr_t)p.scale % 2) == 0);
+    note_kernel(refq ? "gemm_wo_tile_kernel(per-weight rounding)" : "gemm_wo_tile_kernel", WBITS, bm, 128);
+#define FNN_TILE(G, SDTV, RQ)                                                                            \
     do {                                                                                                 \
         if constexpr (WBITS == 4) {                                                                      \
             if (bm == 256) {                                                                             \
-                gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 256><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles); \
+                gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 256, RQ><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles); \
                 break;                                                                                   \
             }                                                                                            \
         }                                                                                                \
-        gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 128><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles);    \
+        gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 128, RQ><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles); \
     } while (0)
+    if constexpr (ADT == FNN_F16) {
+        if (refq) {
+            if (p.group == 128) { if (p.zp) FNN_TILE(true, FNN_F16, 2); else FNN_TILE(true, FNN_F16, 1); }
+            else { if (p.zp) FNN_TILE(false, FNN_F16, 2); else FNN_TILE(false, FNN_F16, 1); }
+            return true;
+        }
+    }
     if (p.group == 128) {
-        if (p.scale_dtype == FNN_F16) FNN_TILE(true, FNN_F16);
-        else FNN_TILE(true, FNN_BF16);
+        if (p.scale_dtype == FNN_F16) FNN_TILE(true, FNN_F16, 0);
+        else FNN_TILE(true, FNN_BF16, 0);
     } else {
-        FNN_TILE(false, FNN_F16);
+        FNN_TILE(false, FNN_F16, 0);
     }
 #undef FNN_TILE
     return true;

@@ -19,6 +19,10 @@ struct WoArgs {
     int group;            // 0 = per channel
     int out_dtype, scale_dtype, zp_dtype, bias_dtype;
     int m_base;           // first activation row handled by this launch
+    void* cvt_ws;         // scratch for bf16 activations converted to fp16 (NULL: none), cvt_ws_bytes of it
+    size_t cvt_ws_bytes;
+    const float* act_unscale;   // per activation row: what the output is multiplied by (NULL: nothing); set where
+                                // the rows were scaled by a power of two on their way from bf16 to fp16
 };
 
 constexpr int kWoWaves = 8;
@@ -150,6 +154,12 @@ __device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4
 }
 
 
+// gemm_weight_only.hip: where the caller gave scratch and the tables are fp16 (per channel or per group of
+// 128), converts the bf16 activation rows of p to fp16 rows in the scratch, each row scaled by a power of two
+// so that every value is representable, and fills q with the same problem on those rows (q.act_unscale
+// holding the inverse scales); false, with nothing launched, if that does not apply
+bool convert_act_to_f16(const WoArgs& p, WoArgs& q, hipStream_t st);
+size_t act_f16_ws_bytes(int64_t M, int64_t K);
 // gemm_wo_panel.hip: 9 .. a few hundred activation rows; false if the shape does not suit it
 bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
 // gemm_wo_tile.hip: more than 64 activation rows, tiled MFMA kernel; false if the shape does not suit it

@@ -248,14 +248,23 @@ def _weight_only(fn_name, out, act, quant_w, scale_w, bias, zero_points, n_out):
         if bias.dim() != 1 or not bias.is_contiguous():
             bias = bias.reshape(-1).contiguous()
         assert bias.numel() == N
-    fn = getattr(lib, fn_name)
-    _lib.check(fn(_lib.ptr(out), _lib.ptr(act), _lib.ptr(quant_w), _lib.ptr(scale_w), _lib.ptr(bias),
-                  _lib.ptr(zp), M, N, K, act.stride(0) if M > 1 else K, K,
-                  out.stride(0) if M > 1 else N, group, _lib.dtype_code(act.dtype),
-                  _lib.dtype_code(out.dtype), _lib.dtype_code(scale_w.dtype),
-                  _lib.dtype_code(zp.dtype) if zp is not None else 0,
-                  _lib.dtype_code(bias.dtype) if bias is not None else 0,
-                  _lib.current_stream(act.device)))
+    args = (_lib.ptr(out), _lib.ptr(act), _lib.ptr(quant_w), _lib.ptr(scale_w), _lib.ptr(bias),
+            _lib.ptr(zp), M, N, K, act.stride(0) if M > 1 else K, K,
+            out.stride(0) if M > 1 else N, group, _lib.dtype_code(act.dtype),
+            _lib.dtype_code(out.dtype), _lib.dtype_code(scale_w.dtype),
+            _lib.dtype_code(zp.dtype) if zp is not None else 0,
+            _lib.dtype_code(bias.dtype) if bias is not None else 0)
+    # scratch for bf16 rows converted to fp16 (so that every weight is rounded as the reference rounds it): taken
+    # from torch's caching allocator per call, which hands it to later calls on this stream in stream order
+    need = 0
+    if M > 64 and act.dtype == torch.bfloat16:
+        need = int(lib.fnn_gemm_weight_only_workspace_bytes(M, N, K, group, _lib.dtype_code(act.dtype),
+                                                            _lib.dtype_code(scale_w.dtype)))
+    if need:
+        ws = torch.empty(need, dtype=torch.uint8, device=act.device)
+        _lib.check(getattr(lib, fn_name + "_ws")(*args, ws.data_ptr(), need, _lib.current_stream(act.device)))
+    else:
+        _lib.check(getattr(lib, fn_name)(*args, _lib.current_stream(act.device)))
     return out
 
 

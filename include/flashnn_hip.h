@@ -142,6 +142,32 @@ int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const void* scale
                    void* stream);
 
 /*
+ * fnn_gemm_a16w8 / fnn_gemm_a16w4 with scratch memory for the activations.  The reference's torch path
+ * rounds every dequantised weight to fp16 before the dot product, (q - zp) * s with both operations rounded
+ * (flashnn/quant_gemm.py:14-36); the tiled kernel for more than 64 rows does the same where activations and
+ * tables are fp16 (so do the few-row kernels with per-channel tables), and the result then differs from the
+ * reference's only by the order of the fp32 additions.  bf16 activations (more than 64 rows, fp16 tables
+ * per channel or per group of 128) reach that form through
+ * one conversion pass: every row becomes an fp16 row in the workspace, scaled by a power of two that makes
+ * every value representable (undone exactly on the output).  Without a workspace, or with less than
+ *   fnn_gemm_weight_only_workspace_bytes(M, N, K, group, act_dtype, scale_dtype)   (0: the call would not use one)
+ * the call is fnn_gemm_a16w8 / fnn_gemm_a16w4: the same kernels scaling group sums in fp32, which agrees with
+ * the reference within rtol = atol = 1e-2 on the configured shapes but is not its rounding.  The workspace
+ * needs no initialisation, is 16-byte aligned, and belongs to the call while it runs (calls that overlap
+ * in time need one each).
+ */
+size_t fnn_gemm_weight_only_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int act_dtype,
+                                            int scale_dtype);
+int fnn_gemm_a16w8_ws(void* out, const void* act, const void* qw, const void* scale, const void* bias,
+                      const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                      int64_t group, int act_dtype, int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
+                      void* workspace, size_t ws_bytes, void* stream);
+int fnn_gemm_a16w4_ws(void* out, const void* act, const void* qw, const void* scale, const void* bias,
+                      const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                      int64_t group, int act_dtype, int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
+                      void* workspace, size_t ws_bytes, void* stream);
+
+/*
  * fnn_gemm_a16w4 for the decode of one token (M = 1) on weights repacked once by the caller.  The
  * reference keeps int4 weights as [N/2, K] bytes with [K/group, N] tables beside them
  * (flashnn/quant_gemm.py:174-204; its Triton launcher, flashnn/triton_kernels/gemm_a16w4.py:336-406, reads

@@ -607,20 +607,33 @@ def _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp, with_bias, seed)
     return act, w, qw, scale, zp, bias
 
 
-WO_BREACHES = []   # (test id, outputs beyond the stated tolerance, outputs) of the cases that had any
+WO_BREACHES = []   # (case, outputs beyond the stated tolerance, outputs) of the cases that had any
+
+# The kernels that scale channel or group sums in fp32 where the reference rounds every dequantised weight to
+# the table type (flashnn/quant_gemm.py:14-36).  The reference's rounding moves an output by about
+# 2^-11 |w| sqrt(K) (2^-8 with bf16 tables), which on outputs near zero of long dot products exceeds
+# rtol = atol = 1e-2 although the kernel is the more accurate of the two.  Only these kernels may leave the
+# stated tolerance, only on a bounded share of the outputs, and only towards the float64 value; every kernel
+# that says it rounds per weight - the tiled kernel for more than 64 rows and the few-row kernels with
+# per-channel tables, on fp16 tables - is held to the tolerance without exception.
+FP32_SCALING_KERNELS = {"gemm_wo_panel_kernel", "gemm_wo_stream_kernel", "gemm_wo_any_kernel", "gemm_wo_decode_kernel",
+                        "gemm_wo_decode_lds_kernel", "gemm_wo_gemv_kernel", "gemm_wo_gemv_flat_kernel",
+                        "gemm_wo_tile_kernel"}
+BREACH_SHARE = {"f16": 0.005, "bf16": 0.10, "f32": 0.005}     # by table type
 
 
 def _wo_check(act, w, qw, scale, zp, bias, group, bits, out_ty, strict=False):
     """The stated tolerance, unscaled: |got - oracle| <= 1e-2 + 1e-2 |oracle|, the oracle being the reference's
-    torch path with its per-weight rounding of the dequantised weights to the scale type (fp16 for group
-    tables).  Where activations and per-channel scales are both fp16 the kernels round the same way and
-    `strict` demands that no output leaves the tolerance.  Elsewhere the kernels scale in fp32, which the
-    reference's rounding can leave by more than the tolerance on outputs near zero of long dot products;
-    such an output must then be at least as close to the float64 value as the oracle's is, and the count is
-    reported."""
+    torch path with its per-weight rounding of the dequantised weights to the table type (fp16 for group
+    tables).  A kernel that rounds the same way (it says so in its name, or the caller passes `strict`) must
+    keep every output inside.  The kernels listed in FP32_SCALING_KERNELS may leave it on at most
+    BREACH_SHARE of the outputs, each of which must then be at least as close to the float64 value as the
+    oracle's is; the cases and counts are reported."""
     d = lambda t: None if t is None else t.to(DEV)
     out = flashnn_amd.GemmWeightOnly(out_ty)(d(act), d(qw), d(scale), d(bias), d(zp))
     assert out.dtype == out_ty and out.shape == (act.shape[0], w.shape[0])
+    kernel = _lib.last_kernel()
+    strict = strict or "per-weight rounding" in kernel
     got = out.float().cpu().numpy()
     n = lambda t: None if t is None else O.to_np(t)
     want = O.weight_only_gemm(n(act), w.numpy(), n(scale), n(zp), n(bias), _tag(scale.dtype), _tag(out_ty),
@@ -630,8 +643,11 @@ def _wo_check(act, w, qw, scale, zp, bias, group, bits, out_ty, strict=False):
     if bad.any():
         import os
         case = os.environ.get("PYTEST_CURRENT_TEST", "?").split(" ")[0]
-        WO_BREACHES.append((case, int(bad.sum()), bad.size))
-        assert not strict, f"{int(bad.sum())} outputs beyond the stated tolerance on a reference-rounding path"
+        WO_BREACHES.append((f"{case} [{kernel}; act {_tag(act.dtype)}, tables {_tag(scale.dtype)}, "
+                            f"M={act.shape[0]} N={w.shape[0]} K={act.shape[1]} group={group}]", int(bad.sum()), bad.size))
+        assert not strict, f"{int(bad.sum())} outputs beyond the stated tolerance on a reference-rounding path ({kernel})"
+        assert kernel.split("<")[0] in FP32_SCALING_KERNELS, kernel
+        assert bad.mean() <= BREACH_SHARE[_tag(scale.dtype)], f"{bad.mean():.4f} of the outputs beyond the tolerance ({kernel})"
         assert (np.abs(got[bad] - exact[bad]) <= np.abs(want[bad] - exact[bad])).all()
     # ... and as close to the mathematical value as one output rounding (and fp32 accumulation) allows
     spread = max(1.0, float(np.sqrt(np.mean(want.astype(np.float64) ** 2))))
@@ -770,6 +786,46 @@ def test_weight_only_tiled_large_m(bits, group, M, N, K):
     scale_ty = torch.bfloat16 if M == 300 else torch.float16
     case = _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp=M != 128, with_bias=M in (65, 256), seed=700 + M)
     _wo_check(*case, group, bits, act_ty)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("group", [0, 128])
+def test_weight_only_bf16_rows_through_the_conversion_pass(hip_lib, bits, group):
+    """bf16 activations, fp16 tables, more than 64 rows: with scratch memory the rows become fp16 rows (scaled
+    by a power of two per row) and the tiled kernel rounds every weight as the reference does - no output
+    may leave the tolerance, with rows of magnitudes from 1e-20 to 1e20 among ordinary ones; the same call
+    without scratch runs the fp32-scaling kernel and stays within the tolerance of the first."""
+    M, N, K = 200, 256, 2048
+    act, w, qw, scale, zp, bias = _wo_inputs(M, N, K, group, bits, torch.bfloat16, torch.float16, True, True, seed=911)
+    act = act.float()
+    act[3] *= 1e20          # far beyond fp16's range
+    act[5] *= 1e-20         # far below it
+    act[7] = 0.0
+    act[9, ::2] *= 3e4
+    act = act.bfloat16()
+    d = lambda t: t.to(DEV)
+    out = flashnn_amd.GemmWeightOnly(torch.bfloat16)(d(act), d(qw), d(scale), d(bias), d(zp))
+    assert _lib.last_kernel().startswith("gemm_wo_tile_kernel(per-weight rounding)")
+    got = out.float().cpu().numpy()
+    want = O.weight_only_gemm(O.to_np(act), w.numpy(), O.to_np(scale), O.to_np(zp), O.to_np(bias), O.F16, O.BF16, group, bits == 4)
+    got, want = got.astype(np.float64), want.astype(np.float64)
+    scale_of_row = np.maximum(1.0, np.abs(want).max(axis=1, keepdims=True) / 50.0)      # rows of 1e20 have outputs of 1e20
+    assert (np.abs(got - want) <= (ATOL + RTOL * np.abs(want)) * scale_of_row).all()
+    assert not got[7].any() or np.allclose(got[7], O.to_np(bias).astype(np.float32), atol=1e-2)
+    # the plain entry point (no scratch): the fp32-scaling kernel, within the tolerance of the reference-rounding one
+    plain = torch.empty_like(out)
+    fn = hip_lib.fnn_gemm_a16w4 if bits == 4 else hip_lib.fnn_gemm_a16w8
+    a_d, q_d, s_d, z_d, b_d = d(act), d(qw), d(scale), d(zp), d(bias)
+    rc = fn(plain.data_ptr(), a_d.data_ptr(), q_d.data_ptr(), s_d.data_ptr(), b_d.data_ptr(), z_d.data_ptr(), M, N, K, K, K, N,
+            group, 1, 1, 0, 0, _lib.dtype_code(b_d.dtype), _lib.current_stream(a_d.device))
+    assert rc == 0 and _lib.last_kernel().startswith("gemm_wo_tile_kernel<")
+    p_np = plain.float().cpu().numpy().astype(np.float64)
+    assert (np.abs(p_np - got) <= (2 * ATOL + 2 * RTOL * np.abs(got)) * scale_of_row).all()
+    need = hip_lib.fnn_gemm_weight_only_workspace_bytes(M, N, K, group, 1, 0)
+    assert need == (M * K * 2 + 255) // 256 * 256 + 4 * M
+    assert hip_lib.fnn_gemm_weight_only_workspace_bytes(64, N, K, group, 1, 0) == 0        # few rows: other kernels
+    assert hip_lib.fnn_gemm_weight_only_workspace_bytes(M, N, K, group, 0, 0) == 0         # fp16 rows need no conversion
+    assert hip_lib.fnn_gemm_weight_only_workspace_bytes(M, N, K, group, 1, 1) == 0         # bf16 tables: fp32 scaling
 
 
 def test_weight_only_tiled_one_hot():
