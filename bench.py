@@ -453,6 +453,23 @@ def main():
             secondary.append(_entry(f"fused_moe_a8w8 tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={BMm} "
                                     f"({active} experts in use)", ms, "hbm",
                                     float(active) * Nm * Km + 2.0 * Mt * top_k * Nm, kern))
+        # a prompt's worth of tokens: the MFMA tiles over the sorted rows (one tile height per block size)
+        Mt = 4096
+        xm = workloads.activations(Mt, Km, torch.float16, seed=74, outlier_frac=0.01).to(dev)
+        am = torch.empty(Mt, Km, dtype=torch.int8, device=dev)
+        arm = torch.empty(Mt, dtype=torch.float16, device=dev)
+        launchers.hip_dynamic_quantize(am, xm, arm)
+        cm = torch.empty(Mt, top_k, Nm, dtype=torch.bfloat16, device=dev)
+        tw, tid = torch.topk(torch.softmax(torch.randn(Mt, E, generator=torch.Generator().manual_seed(8)), -1), top_k)
+        for blk in (64, 128, 256):
+            sid, eid, used = workloads.moe_align_block_size(tid, blk, E)
+            rows_padded = int(used[0])
+            twd, tidd, sid, eid, used = [t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used)]
+            f = lambda i: flashnn_amd.fused_moe_a8w8_forward(am, bm, cm, arm, acm, twd, tidd, sid, eid, used, True, top_k, blk)
+            kern = kernel_of(f)
+            ms, _ = _timed(f, 10, torch)
+            secondary.append(_entry(f"fused_moe_a8w8 tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={blk} "
+                                    f"({rows_padded} sorted rows)", ms, "mfma", 2.0 * Mt * top_k * Nm * Km, kern))
         del bm
         torch.cuda.empty_cache()
         # int4 expert weights of the same layer: per-channel tables, then tables per group of 128 ([E, N, K/128])

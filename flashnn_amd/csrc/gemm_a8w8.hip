@@ -79,8 +79,14 @@ struct OptionalStage<false, BYTES> {
 // count that chose it; nobody waits for anybody.  Integer sums do not depend on the order, so the result is
 // the unsplit kernel's bit for bit.  The unit that adds up sets the counter back to zero: the counters are
 // zero whenever no call is in flight.
-template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2, bool SPLIT = false>
-__global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Args p) {
+// MOE: the mixture-of-experts form for many routed rows per expert (flashnn/triton_kernels/fused_moe_a8w8.py:37-173).
+// The M dimension is the list of sorted routed rows (moe.EM of them, padded per expert to blocks of moe.block_m, a
+// multiple of BM): tile row r multiplies activation row sorted_ids[r] / top_k with the weight matrix of the
+// expert its block belongs to, and the result goes to output row sorted_ids[r], times the routing weight on
+// request.  Tiles beyond the rows in use return at once; padding rows read activation row 0 and store nothing.
+template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2, bool SPLIT = false, bool MOE = false>
+__global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Args p, const MoeArgs moe) {
+    static_assert(!MOE || (!SPLIT && MODE != OUT_I32), "the gathered form has no split and no raw output");
     // WGM x 2 waves.  Only WGM = 2 (one wave per SIMD) is instantiated: with WGM = 4 the two waves of a SIMD
     // meet at the same barrier every slab and never filled each other's gaps (256x192: 81.6 us with four
     // waves, 83.9 with eight; never faster on any shape tried).
@@ -125,7 +131,7 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
     const int t = SPLIT ? unit / p.kparts : unit;
     const int kpart = SPLIT ? unit - t * p.kparts : 0;
     const int8_t* const pa = SPLIT ? p.a + (int64_t)kpart * p.k_chunk : p.a;
-    const int8_t* const pb = SPLIT ? p.b + (int64_t)kpart * p.k_chunk : p.b;
+    const int8_t* pb = SPLIT ? p.b + (int64_t)kpart * p.k_chunk : p.b;
     // (the last part takes what the others leave: a few slabs more, so that it arrives last as a rule)
     const int Kl = SPLIT ? (kpart == p.kparts - 1 ? p.K - kpart * p.k_chunk : p.k_chunk) : p.K;
     // tiles are numbered in groups of GN tile columns, the column fastest within a group: the 32 workgroups
@@ -139,6 +145,15 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
     const int tile_m = rem / gw;
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
+    int expert = 0;
+    if constexpr (MOE) {
+        if (m0 >= moe.ntpp[0]) return;
+        expert = moe.expert_ids[m0 / moe.block_m];
+        pb += (int64_t)expert * moe.stride_be;
+    }
+    // the routed row of tile row r (MOE), and the activation row it reads: padding rows read row 0
+    auto routed = [&](int r) -> int { return moe.sorted_ids[min(m0 + r, moe.EM - 1)]; };
+    auto act_row = [&](int tok) -> int { return tok < moe.num_valid ? tok / moe.top_k : 0; };
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -156,7 +171,8 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
         for (int q = 0; q < NSC; ++q) {
             const int e = threadIdx.x + q * NT;
             const bool is_row = e < BM;
-            const int idx = is_row ? min(m0 + e, p.M - 1) : min(n0 + min(e - BM, BN - 1), p.N - 1);
+            int64_t idx = is_row ? min(m0 + e, p.M - 1) : min(n0 + min(e - BM, BN - 1), p.N - 1);
+            if constexpr (MOE) idx = is_row ? act_row(routed(e)) : idx + (int64_t)expert * moe.stride_scale_be;
             const void* base = is_row ? p.arow : p.acol;
             sc_raw[q] = (is_row ? p.arow_dtype : p.acol_dtype) == FNN_F32 ? ((const uint32_t*)base)[idx]
                                                                         : (uint32_t)((const uint16_t*)base)[idx];
@@ -169,8 +185,10 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
     const int lchunk = (lane & 7) ^ ((((wave & 1) << 2) + (lrow >> 1)) & 7);
     uint32_t goa[NLA], gob[NLB];
 #pragma unroll
-    for (int j = 0; j < NLA; ++j)
-        goa[j] = (uint32_t)min(m0 + (j * NWAVES + wave) * 8 + lrow, p.M - 1) * (uint32_t)p.lda + lchunk * 16;
+    for (int j = 0; j < NLA; ++j) {
+        const int r = (j * NWAVES + wave) * 8 + lrow;
+        goa[j] = (uint32_t)(MOE ? act_row(routed(r)) : min(m0 + r, p.M - 1)) * (uint32_t)p.lda + lchunk * 16;
+    }
 #pragma unroll
     for (int j = 0; j < NLB; ++j)
         gob[j] = (uint32_t)min(n0 + (j * NWAVES + wave) * 8 + lrow, p.N - 1) * (uint32_t)p.ldb + lchunk * 16;
@@ -566,6 +584,16 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
             if (is_row) sc_row[e] = v;
             else if (e < BM + BN) sc_col[e - BM] = v;
         }
+        // MOE: the routed row of every tile row (and its routing weight) behind the scales
+        int* const sc_tok = (int*)(sc_col + BN) + 4;
+        float* const sc_wr = (float*)(sc_tok + BM);
+        if constexpr (MOE) {
+            for (int e = threadIdx.x; e < BM; e += NT) {
+                const int tok = routed(e);
+                sc_tok[e] = tok;
+                sc_wr[e] = moe.mul_w && tok < moe.num_valid ? load_as_f32(moe.topk_w, tok, moe.topk_w_dtype) : 1.f;
+            }
+        }
         __syncthreads();
         const int nsel = (csel & 1) * 16 + (csel >> 1) * 8;   // column of this lane's 16 bytes within a fragment pair
         v4f ac[FN];
@@ -579,7 +607,14 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
 #pragma unroll
             for (int j = 0; j < FM; ++j) {
                 const float ar = sc_row[wm * WTM + j * 16 + frow];
-                const int m = wm0 + j * 16 + frow;
+                int m = wm0 + j * 16 + frow;
+                float wr = 1.f;
+                bool row_ok = true;
+                if constexpr (MOE) {        // the output row is the routed row; padding rows store nothing
+                    m = sc_tok[wm * WTM + j * 16 + frow];
+                    wr = sc_wr[wm * WTM + j * 16 + frow];
+                    row_ok = m < moe.num_valid;
+                }
 #pragma unroll
                 for (int i = 0; i < FN; i += 2) {
                     uint32_t lo[2], hi[2];
@@ -587,7 +622,12 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
                     for (int h = 0; h < 2; ++h) {
                         float v[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = ((float)acc[i + h][j][e] * ar) * ac[i + h][e];
+                        for (int e = 0; e < 4; ++e) {
+                            v[e] = ((float)acc[i + h][j][e] * ar) * ac[i + h][e];
+                            if constexpr (MOE) {
+                                if (moe.mul_w) v[e] = v[e] * wr;
+                            }
+                        }
                         if constexpr (MODE == OUT_BF16) {
                             lo[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2bf));
                             hi[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2bf));
@@ -603,7 +643,7 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
                         __builtin_nontemporal_store(val, (v4u*)(obase + (int64_t)(j * 16) * p.ldc + i * 16));
                     } else {
                         const int n = wn0 + i * 16 + nsel;
-                        if (m < p.M && n < p.N) {
+                        if ((MOE ? row_ok : m < p.M) && n < p.N) {
                             uint16_t* o = (uint16_t*)p.out + (int64_t)m * p.ldc + n;
                             if (n + 7 < p.N && (p.ldc & 7) == 0) {
                                 __builtin_nontemporal_store(val, (v4u*)o);
@@ -617,7 +657,7 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
                 }
             }
         };
-        if (inside) store_rows(std::false_type{});
+        if (inside && !MOE) store_rows(std::false_type{});
         else store_rows(std::true_type{});
     }
 }
@@ -759,7 +799,7 @@ static void launch_mfma(A8W8Args& p, hipStream_t st) {
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
     note_kernel("gemm_a8w8_ring_kernel", BM, BN, WGM * 2);
-    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, WGM><<<dim3(p.tiles_per_xcd * 8), dim3(WGM * 128), 0, st>>>(p);
+    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, WGM><<<dim3(p.tiles_per_xcd * 8), dim3(WGM * 128), 0, st>>>(p, MoeArgs{});
 }
 
 // The same tiles with K cut into p.kparts ranges (p.kparts, p.k_chunk, p.ws_count, p.ws_part set by the caller).
@@ -770,7 +810,7 @@ static void launch_mfma_split(A8W8Args& p, hipStream_t st) {
     const int units = p.tiles_m * p.tiles_n * p.kparts;
     p.tiles_per_xcd = (units + 7) / 8;
     note_kernel("gemm_a8w8_ring_kernel(split K)", BM, BN, p.kparts);
-    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, 2, true><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p);
+    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, 2, true><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p, MoeArgs{});
 }
 
 // The tiles that exist: (rows, columns, waves per workgroup).
@@ -935,6 +975,41 @@ static void dispatch(A8W8Args& p, hipStream_t st, int force_bm, int force_bn, in
             q = rows_from(q, m0, (int)(p.M - m0 < m_band ? p.M - m0 : m_band), MODE);
             dispatch_band<MODE>(q, st, aligned && ((uintptr_t)q.out % 16) == 0, force_bm, force_bn, force_waves);
         }
+}
+
+// Mixture of experts with many routed rows per expert: the MFMA tiles over the sorted rows.  A tile must lie
+// within one expert's rows, so its height divides block_m.  Returns false where this form does not apply (the
+// few-row kernels then take the call).
+template <int BM, int BN, int MODE, bool PAIR = false>
+static void launch_mfma_moe(A8W8Args& p, const MoeArgs& q, hipStream_t st) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    p.tiles_per_xcd = (p.tiles_m * p.tiles_n + 7) / 8;
+    note_kernel("gemm_a8w8_ring_kernel(moe)", BM, BN, 4);
+    gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, 2, false, true><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p, q);
+}
+
+template <int MODE>
+static bool launch_moe_tiled_t(A8W8Args& p, const MoeArgs& q, hipStream_t st) {
+    if (q.block_m % 256 == 0) launch_mfma_moe<256, 256, MODE>(p, q, st);
+    else if (q.block_m % 128 == 0) launch_mfma_moe<128, 128, MODE, true>(p, q, st);
+    else launch_mfma_moe<64, 128, MODE>(p, q, st);
+    return true;
+}
+
+static bool launch_a8w8_moe_tiled(A8W8Args& p, const MoeArgs& q, int mode, hipStream_t st) {
+    constexpr int64_t kLimit = (1LL << 31) - 1;
+    const int64_t rows = (q.num_valid + q.top_k - 1) / q.top_k;          // activation rows
+    const bool ok = q.block_m % 64 == 0 && q.EM % q.block_m == 0 && p.K % 32 == 0 && p.K >= 1024 &&
+                    p.lda % 16 == 0 && p.ldb % 16 == 0 && q.stride_be % 16 == 0 && ((uintptr_t)p.a % 16) == 0 &&
+                    ((uintptr_t)p.b % 16) == 0 && ((uintptr_t)p.out % 16) == 0 && rows * p.lda <= kLimit &&
+                    (int64_t)p.N * p.ldb <= kLimit && (int64_t)(p.M / 64) * ((p.N + 127) / 128) <= kLimit;
+    // The few-row kernel reads an expert's weights once per 64 sorted rows.  Measured on 8 experts of
+    // 28672 x 4096, 2 per token, microseconds over S sorted rows in use: few-row kernel 100 + 0.18 S; tiles of
+    // 64 rows 110 + 0.14 S, of 128 rows 105 + 0.10 S, of 256 rows 57 + 0.092 S.  Blocks of 128 rows or more
+    // always take the tiles; blocks of 64 from about 512 routed rows on.
+    if (!ok || (q.block_m % 128 != 0 && q.num_valid < 512)) return false;
+    return mode == OUT_F16 ? launch_moe_tiled_t<OUT_F16>(p, q, st) : launch_moe_tiled_t<OUT_BF16>(p, q, st);
 }
 
 static int check_args(const char* fn, const void* out, const void* a, const void* b, int64_t M,
@@ -1201,6 +1276,7 @@ extern "C" int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const v
     q.top_k = top_k; q.block_m = block_m; q.num_valid = (int)num_valid_tokens; q.EM = (int)EM;
     q.stride_be = stride_be; q.stride_scale_be = stride_scale_be;
     const Call call(fn);
-    launch_a8w8_moe(p, q, out_dtype == FNN_F16 ? OUT_F16 : OUT_BF16, (hipStream_t)stream);
+    const int mode = out_dtype == FNN_F16 ? OUT_F16 : OUT_BF16;
+    if (!launch_a8w8_moe_tiled(p, q, mode, (hipStream_t)stream)) launch_a8w8_moe(p, q, mode, (hipStream_t)stream);
     return call.done();
 }

@@ -545,6 +545,43 @@ def test_fused_moe_a8w8_bit_exact(shape, mul_w, out_ty):
             assert (want == 3.0).any()
 
 
+@pytest.mark.parametrize("out_ty", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [
+    # M, E, N, K, top_k, BM, tile rows: prompt-sized batches, which take the MFMA tiles over the sorted rows
+    (1024, 8, 1024, 1024, 2, 64, 64), (1500, 8, 384, 1056, 2, 128, 128), (1100, 4, 528, 2048, 2, 256, 256),
+    (2048, 8, 560, 1024, 1, 64, 64), (1300, 6, 1008, 1184, 3, 192, 64), (700, 2, 144, 4096, 2, 128, 128),
+    (40, 8, 272, 1024, 2, 128, 128)])
+def test_fused_moe_a8w8_many_rows_bit_exact(shape, out_ty):
+    """Many routed rows per expert: the tiled kernel gathers activation rows by the sorted list and scatters
+    the results; bit for bit against the oracle, with and without the routing weight, also when the list is
+    cut short (the tiles beyond it do nothing) and when some experts receive no rows."""
+    M, E, N, K, top_k, BM, tile_rows = shape
+    g = torch.Generator().manual_seed(M * 17 + E)
+    a = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g)
+    b = torch.randint(-128, 128, (E, N, K), dtype=torch.int8, generator=g)
+    ar = (torch.rand(M, generator=g) * 0.05).to(out_ty)
+    ac = (torch.rand(E, N, generator=g) * 0.05).float()
+    logits = torch.randn(M, E, generator=g)
+    if E >= 6:
+        logits[:, 1] = -1e9                 # an expert that nobody is routed to
+    w, ids = torch.topk(torch.softmax(logits, -1), top_k, dim=-1)
+    w = w.float().contiguous()
+    s, e, used = workloads.moe_align_block_size(ids, BM, E)
+    full = int(used[0])
+    for mul_w, cut in ((True, full), (False, full), (True, (full // BM // 2) * BM)):
+        used_c = torch.tensor([cut], dtype=torch.int32)
+        c = torch.full((M, top_k, N), 3.0, dtype=out_ty)
+        want = O.fused_moe_a8w8(a.numpy(), b.numpy(), c.float().reshape(M * top_k, N).numpy().copy(), O.to_np(ar),
+                                ac.numpy(), w.numpy(), s.numpy(), e.numpy(), used_c.numpy(), mul_w, top_k, BM, _tag(out_ty))
+        cd = c.to(DEV)
+        flashnn_amd.fused_moe_a8w8_forward(a.to(DEV), b.to(DEV), cd, ar.to(DEV), ac.to(DEV), w.to(DEV), ids.to(DEV),
+                                           s.to(DEV), e.to(DEV), used_c.to(DEV), mul_w, top_k, BM)
+        assert _lib.last_kernel() == f"gemm_a8w8_ring_kernel(moe)<{tile_rows},{256 if tile_rows == 256 else 128},4>"
+        assert np.array_equal(cd.float().cpu().reshape(M * top_k, N).numpy(), want)
+        if cut < full:
+            assert (want == 3.0).any()
+
+
 @pytest.mark.parametrize("act_ty", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("group,zp_kind", [(0, "float"), (0, None), (0, "int8"), (128, "float"), (128, None), (128, "int8"),
                                            (64, "int8")])
