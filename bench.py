@@ -490,6 +490,23 @@ def main():
                 secondary.append(_entry(f"fused_moe_a16w4 {label} tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} "
                                         f"block={BMm} ({active} experts in use)", ms, "hbm",
                                         float(active) * (N2 * Km + tables) + 2.0 * Mt * top_k * Nm, kern))
+        # a prompt's worth of tokens, per-channel tables: the tiled MFMA kernel over the sorted rows
+        sc4 = (torch.rand(E, Nm, device=dev, generator=g) * 9e-3 + 1e-3).to(torch.bfloat16)
+        zp4m = torch.randint(-3, 4, (E, Nm), device=dev, generator=g).to(torch.bfloat16)
+        Mt = 4096
+        a4 = workloads.activations(Mt, Km, torch.bfloat16, seed=75).to(dev)
+        cm = torch.empty(Mt, top_k, Nm, dtype=torch.bfloat16, device=dev)
+        tw, tid = torch.topk(torch.softmax(torch.randn(Mt, E, generator=torch.Generator().manual_seed(8)), -1), top_k)
+        for blk in (64, 256):
+            sid, eid, used = workloads.moe_align_block_size(tid, blk, E)
+            rows_padded = int(used[0])
+            twd, tidd, sid, eid, used = [t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used)]
+            f = lambda i: flashnn_amd.fused_moe_a16w4_forward(a4, b4, cm, sc4, zp4m, twd, tidd, sid, eid, used, True,
+                                                              top_k, blk)
+            kern = kernel_of(f)
+            ms, _ = _timed(f, 5, torch)
+            secondary.append(_entry(f"fused_moe_a16w4 per-channel tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={blk} "
+                                    f"({rows_padded} sorted rows)", ms, "mfma16", 2.0 * Mt * top_k * Nm * Km, kern))
         del b4
         torch.cuda.empty_cache()
 

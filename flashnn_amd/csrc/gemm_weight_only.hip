@@ -1728,7 +1728,7 @@ extern "C" int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const 
     // and the types)
     const bool fast = group == 0 || group == 128;
     const Call call(fn);
-    if (!(fast && launch_wo_panel_moe(p, q, act_dtype, st))) {
+    if (!(launch_wo_tile_moe(p, q, act_dtype, st) || (fast && launch_wo_panel_moe(p, q, act_dtype, st)))) {
         const dim3 grid((unsigned)EM, (unsigned)((2 * N + 255) / 256));
         note_kernel("moe_a16w4_any_kernel");
         if (act_dtype == FNN_F16) moe_a16w4_any_kernel<FNN_F16><<<grid, dim3(256), 0, st>>>(p, q);

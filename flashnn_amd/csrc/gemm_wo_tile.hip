@@ -42,9 +42,17 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // set, and the result differs from the reference's only by the order of the fp32 additions.  bf16
 // activations reach this form through the conversion pass of gemm_weight_only.hip (rows scaled by a power
 // of two, p.act_unscale undoes it).
-template <int WBITS, int ADT, bool G128, int SDT, int BM, int REFQ = 0>
-__global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const int tiles_m, const int tiles) {
+// MOE (per-channel tables, no REFQ): the mixture-of-experts form for many routed rows per expert
+// (flashnn/triton_kernels/fused_moe_a16w4.py:50-206).  The M dimension is the list of sorted routed rows,
+// padded per expert to blocks of q.block_m rows, a multiple of BM: tile row r multiplies activation row
+// sorted_ids[r] / top_k with the weights, scales and zero points of the expert its block belongs to, and the
+// result goes to output row sorted_ids[r], times the routing weight on request.  Tiles beyond the rows in
+// use return at once; padding rows read activation row 0 and store nothing.
+template <int WBITS, int ADT, bool G128, int SDT, int BM, int REFQ = 0, bool MOE = false>
+__global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const int tiles_m, const int tiles,
+                                                           const MoeArgs q) {
     static_assert(!REFQ || (ADT == FNN_F16 && SDT == FNN_F16), "reference rounding: fp16 activations and tables");
+    static_assert(!MOE || (!G128 && REFQ == 0 && WBITS == 4), "the gathered form: int4, per-channel tables");
     typedef MfmaT<ADT> MT;
     static_assert(WBITS == 4 || BM == 128, "three stages of 128 int8 weight rows leave room for 128 activation rows");
     constexpr int NH = WBITS == 4 ? 2 : 1;          // channels per weight row
@@ -81,6 +89,11 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     const int tile_n = t / tiles_m, tile_m = t - tile_n * tiles_m;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int KT = p.K / 128;
+    int expert = 0;
+    if constexpr (MOE) {
+        if (m0 >= q.ntpp[0]) return;
+        expert = q.expert_ids[m0 / q.block_m];
+    }
 
     // ---- copies.  A wave instruction writes 1 KB of LDS, linear in the lane id; the swizzle is applied
     // on the global side.  Activations: instruction i of a wave covers rows (i * 8 + wave) * 4 .. + 3,
@@ -92,12 +105,20 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     const int ar_max = p.M - 1 - m0;                 // rows beyond M read the last row (and are not stored)
     const uint32_t a_chunk = (((lane & 15) ^ (ar0 & 15)) << 4);
     const uint32_t lda2 = (uint32_t)(p.lda * 2);
-    const char* const a_base = (const char*)p.act + (int64_t)m0 * p.lda * 2;
+    const char* const a_base = (const char*)p.act + (MOE ? 0 : (int64_t)m0 * p.lda * 2);
+    uint32_t a_off[MOE ? NCA : 1];                   // MOE: the gathered rows' offsets are kept
+    if constexpr (MOE) {
+#pragma unroll
+        for (int i = 0; i < NCA; ++i) {
+            const int tok = q.sorted_ids[m0 + ar0 + 32 * i];
+            a_off[i] = (uint32_t)(tok < q.num_valid ? tok / q.top_k : 0) * lda2 + a_chunk;
+        }
+    }
     auto copy_a = [&](char* stage, int j) {
         const char* src = a_base + (int64_t)min(j, KT - 1) * 256;        // scalar
 #pragma unroll
         for (int i = 0; i < NCA; ++i) {
-            const uint32_t off = (uint32_t)min(ar0 + 32 * i, ar_max) * lda2 + a_chunk;
+            const uint32_t off = MOE ? a_off[i] : (uint32_t)min(ar0 + 32 * i, ar_max) * lda2 + a_chunk;
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + off), (lds_ptr_t)(stage + (i * 8 + wave) * 1024), 16, 0, 0);
         }
         // (the compiler keeps these offsets in registers where it has them to spare)
@@ -111,7 +132,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
         const int r = (i * 8 + wave) * 8 + (lane >> 3);
         gw[i] = (uint32_t)r * (uint32_t)p.ldw + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
     }
-    const char* const w_base = (const char*)p.qw + (int64_t)(n0 / NH) * p.ldw;
+    const char* const w_base = (const char*)p.qw + (int64_t)(n0 / NH) * p.ldw + (MOE ? (int64_t)expert * q.stride_be : 0);
     auto copy_w = [&](char* stage, int j) {
         const char* src = w_base + (int64_t)min(j, KT - 1) * 128;
 #pragma unroll
@@ -416,8 +437,8 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int n = n0 + wn * WTN + (NH == 2 ? (a >> 1) * 32 + 2 * (4 * g + r) + (a & 1) : a * 16 + 4 * g + r);
-                sc[r] = load_as_f32(p.scale, n, p.scale_dtype);
-                zc[r] = c_off + (has_zp ? load_as_f32(p.zp, n, p.zp_dtype) : 0.f);
+                sc[r] = load_as_f32(p.scale, (MOE ? (int64_t)expert * q.stride_scale_be : 0) + n, p.scale_dtype);
+                zc[r] = c_off + (has_zp ? load_as_f32(p.zp, (MOE ? (int64_t)expert * q.stride_zp_be : 0) + n, p.zp_dtype) : 0.f);
             }
 #pragma unroll
             for (int b = 0; b < FB; ++b)
@@ -438,10 +459,16 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
         for (int c = 0; c < 4 * NH; ++c) bias[c] = p.bias ? load_as_f32(p.bias, nb + c, p.bias_dtype) : 0.f;
 #pragma unroll
         for (int b = 0; b < FB; ++b) {
-            const int m = m0 + wm * WTM + b * 16 + row16;
-            if (m >= p.M) continue;
+            int m = m0 + wm * WTM + b * 16 + row16;
+            if (!MOE && m >= p.M) continue;
             // (rows converted from bf16 were scaled by a power of two: the exact inverse)
-            const float un = REFQ != 0 && p.act_unscale ? p.act_unscale[m] : 1.f;
+            float un = 1.f;
+            if constexpr (REFQ != 0) un = p.act_unscale ? p.act_unscale[m] : 1.f;
+            if constexpr (MOE) {       // the output row is the routed row; `un` carries the routing weight
+                m = q.sorted_ids[m];
+                if (m >= q.num_valid) continue;
+                if (q.mul_w) un = load_as_f32(q.topk_w, m, q.topk_w_dtype);
+            }
             uint32_t pk[2 * NH];
 #pragma unroll
             for (int c = 0; c < 4 * NH; c += 2) {
@@ -495,11 +522,11 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
     do {                                                                                                 \
         if constexpr (WBITS == 4) {                                                                      \
             if (bm == 256) {                                                                             \
-                gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 256, RQ><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles); \
+                gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 256, RQ><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, MoeArgs{}); \
                 break;                                                                                   \
             }                                                                                            \
         }                                                                                                \
-        gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 128, RQ><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles); \
+        gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 128, RQ><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, MoeArgs{}); \
     } while (0)
     if constexpr (ADT == FNN_F16) {
         if (refq) {
@@ -516,6 +543,32 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
     }
 #undef FNN_TILE
     return true;
+}
+
+// Mixture of experts, int4 weights with per-channel tables, many routed rows per expert; false where this
+// form does not apply.
+template <int ADT>
+static bool launch_tile_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
+    const int bm = q.block_m % 256 == 0 ? 256 : 128;
+    const int tiles_m = p.M / bm;
+    const int tiles = tiles_m * (p.N / 128);
+    const dim3 grid(((tiles + 7) / 8) * 8);
+    note_kernel("gemm_wo_tile_kernel(moe)", 4, bm, 128);
+    if (bm == 256) gemm_wo_tile_kernel<4, ADT, false, FNN_F16, 256, 0, true><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, q);
+    else gemm_wo_tile_kernel<4, ADT, false, FNN_F16, 128, 0, true><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, q);
+    return true;
+}
+
+bool launch_wo_tile_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t st) {
+    const int64_t rows = (q.num_valid + q.top_k - 1) / q.top_k;          // activation rows
+    const bool ok = p.group == 0 && q.block_m % 128 == 0 && q.EM % q.block_m == 0 && p.N % 128 == 0 &&
+                    p.K % 256 == 0 && p.K >= 512 && p.lda % 8 == 0 && p.ldw % 16 == 0 &&
+                    q.stride_be % 16 == 0 && ((uintptr_t)p.qw % 16) == 0 && ((uintptr_t)p.act % 16) == 0 &&
+                    rows * p.lda * 2 < (1LL << 32) && (int64_t)64 * p.ldw < (1LL << 31) &&
+                    q.stride_scale_n == 1 && (!p.zp || (q.stride_zp_n == 1 && p.zp_dtype != FNN_I8)) &&
+                    (int64_t)(p.M / 128) * (p.N / 128) < (1LL << 31);
+    if (!ok) return false;
+    return act_dtype == FNN_F16 ? launch_tile_moe_t<FNN_F16>(p, q, st) : launch_tile_moe_t<FNN_BF16>(p, q, st);
 }
 
 bool launch_wo_tile(WoArgs& p, int wbits, int act_dtype, hipStream_t st) {

@@ -164,6 +164,8 @@ size_t act_f16_ws_bytes(int64_t M, int64_t K);
 bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
 // gemm_wo_tile.hip: more than 64 activation rows, tiled MFMA kernel; false if the shape does not suit it
 bool launch_wo_tile(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
+// ... its mixture-of-experts form (int4, per-channel tables, blocks of 128 rows or more); false otherwise
+bool launch_wo_tile_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t st);
 // the int4 per-channel kernel over gathered rows of a mixture of experts; false if the shape does not suit it
 bool launch_wo_panel_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t st);
 

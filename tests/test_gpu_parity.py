@@ -630,6 +630,46 @@ def test_fused_moe_a16w4_close(shape, group, zp_kind, act_ty):
     assert bool((got2[rest] == 3.0).all()) and not bool((got2[first] == 3.0).all())
 
 
+@pytest.mark.parametrize("act_ty", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("zp_kind", ["float", None])
+@pytest.mark.parametrize("shape", [
+    # M, E, packed rows (half the output channels), K, top_k, BM, tile rows
+    (1024, 8, 256, 1024, 2, 128, 128), (1100, 4, 192, 2048, 2, 256, 256), (40, 8, 128, 1280, 2, 128, 128),
+    (1500, 6, 64, 4096, 1, 384, 128)])
+def test_fused_moe_a16w4_many_rows_close(shape, zp_kind, act_ty):
+    """Many routed rows per expert, per-channel tables: the tiled MFMA kernel gathers activation rows by the
+    sorted list and scatters the results; the tolerance of 16-bit GEMM outputs against the oracle, with the
+    routing weight and without, the list whole and cut short, one expert without rows."""
+    M, E, N2, K, top_k, BM, tile_rows = shape
+    g = torch.Generator().manual_seed(M * 19 + E)
+    a = torch.randn(M, K, generator=g).to(act_ty)
+    w = torch.randint(-8, 8, (E, 2 * N2, K), dtype=torch.int8, generator=g)
+    packed = torch.stack([torch.from_numpy(O.pack_int4(w[e].numpy())) for e in range(E)])
+    scale = torch.empty(E, 2 * N2).uniform_(1e-3, 1e-2, generator=g).to(act_ty)
+    zp = None if zp_kind is None else torch.randint(-3, 4, (E, 2 * N2), generator=g).to(act_ty)
+    logits = torch.randn(M, E, generator=g)
+    if E >= 6:
+        logits[:, 1] = -1e9
+    tw, ids = torch.topk(torch.softmax(logits, -1), top_k, dim=-1)
+    tw = tw.float().contiguous()
+    s, e, used = workloads.moe_align_block_size(ids, BM, E)
+    full = int(used[0])
+    for mul_w, cut in ((True, full), (False, full), (True, (full // BM // 2) * BM)):
+        used_c = torch.tensor([cut], dtype=torch.int32)
+        c = torch.full((M, top_k, 2 * N2), 3.0, dtype=act_ty)
+        want = O.fused_moe_a16w4(O.to_np(a), packed.numpy(), c.float().reshape(M * top_k, 2 * N2).numpy().copy(),
+                                 O.to_np(scale), None if zp is None else O.to_np(zp.float()), tw.numpy(), s.numpy(),
+                                 e.numpy(), used_c.numpy(), mul_w, top_k, BM, _tag(act_ty), _tag(act_ty))
+        cd = c.to(DEV)
+        flashnn_amd.fused_moe_a16w4_forward(a.to(DEV), packed.to(DEV), cd, scale.to(DEV), None if zp is None else zp.to(DEV),
+                                            tw.to(DEV), ids.to(DEV), s.to(DEV), e.to(DEV), used_c.to(DEV), mul_w, top_k, BM)
+        assert _lib.last_kernel() == f"gemm_wo_tile_kernel(moe)<4,{tile_rows},128>"
+        got = cd.float().cpu().reshape(M * top_k, 2 * N2).numpy()
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+        if cut < full:
+            assert (want == 3.0).any() and np.array_equal(got == 3.0, want == 3.0)
+
+
 # ------------------------------------------------------------------ weight-only GEMM
 def _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp, with_bias, seed):
     g = torch.Generator().manual_seed(seed)
