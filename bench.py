@@ -469,7 +469,8 @@ def main():
             kern = kernel_of(f)
             ms, _ = _timed(f, 10, torch)
             secondary.append(_entry(f"fused_moe_a8w8 tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={blk} "
-                                    f"({rows_padded} sorted rows)", ms, "mfma", 2.0 * Mt * top_k * Nm * Km, kern))
+                                    f"({rows_padded} sorted rows)", ms, "mfma", 2.0 * Mt * top_k * Nm * Km, kern,
+                                    f"moe a8w8 {Mt} tokens block {blk}"))
         del bm
         torch.cuda.empty_cache()
         # int4 expert weights of the same layer: per-channel tables, then tables per group of 128 ([E, N, K/128])
@@ -506,7 +507,8 @@ def main():
             kern = kernel_of(f)
             ms, _ = _timed(f, 5, torch)
             secondary.append(_entry(f"fused_moe_a16w4 per-channel tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={blk} "
-                                    f"({rows_padded} sorted rows)", ms, "mfma16", 2.0 * Mt * top_k * Nm * Km, kern))
+                                    f"({rows_padded} sorted rows)", ms, "mfma16", 2.0 * Mt * top_k * Nm * Km, kern,
+                                    f"moe a16w4 {Mt} tokens block {blk}"))
         del b4
         torch.cuda.empty_cache()
 
