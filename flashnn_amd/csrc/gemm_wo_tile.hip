@@ -82,11 +82,18 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     const int wm = wave % WGM, wn = wave / WGM;
     const int row16 = lane & 15, g = lane >> 4;
 
-    // workgroups id, id + 8, .. share an XCD: the row tiles of one channel tile follow each other there
+    // workgroups id, id + 8, .. share an XCD and take consecutive tile numbers
     const int per_xcd = gridDim.x >> 3;
     const int t = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (t >= tiles) return;
-    const int tile_n = t / tiles_m, tile_m = t - tile_n * tiles_m;
+    // tiles are numbered in groups of four channel tiles, the channel tile fastest within a group: the 32
+    // workgroups an XCD runs at a time then cover 8 row tiles x 4 channel tiles, and the activation rows are
+    // fetched into its L2 once per group instead of once per channel tile
+    constexpr int GN = 4;
+    const int tiles_n = tiles / tiles_m;
+    const int grp = t / (GN * tiles_m), rem = t - grp * (GN * tiles_m);
+    const int gcols = min(GN, tiles_n - grp * GN);
+    const int tile_n = grp * GN + rem % gcols, tile_m = rem / gcols;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int KT = p.K / 128;
     int expert = 0;

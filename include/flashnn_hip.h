@@ -319,6 +319,9 @@ int fnn_gemm_a8w8_i32_tiled(int32_t* acc, const void* a, const void* b, int64_t 
  * are left untouched.  sorted_token_ids [EM], expert_ids and num_tokens_post_padded [1] are int32 device
  * arrays.  The weight-streaming kernel takes N % 16 == 0, K % 32 == 0, K >= 1024, block_m % 16 == 0,
  * EM % block_m == 0 and 16-byte aligned rows; anything else takes a slow guarded kernel.
+ * Many routed rows per expert: with block_m a multiple of 128 (or of 64, from 512 routed rows on) and
+ * K >= 1024 the call runs MFMA tiles over the sorted rows (tile height 64, 128 or 256 = the largest of those
+ * that divides block_m) instead of streaming an expert's weights once per 64 rows; same arithmetic, same bits.
  */
 int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const void* alpha_row,
                        const void* alpha_col, const void* topk_weights,
@@ -348,7 +351,9 @@ int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const void* alpha_
  * N % 16 == 0, K >= 1024, block_m % 16 == 0, EM % block_m == 0 and 16-byte aligned rows; anything else
  * takes a slow guarded kernel.  The reference multiplies the dequantised weights of a K block by their scale
  * before the dot product and rounds them to the scale type; here the block's dot product is scaled
- * afterwards, in fp32.
+ * afterwards, in fp32.  Many routed rows per expert: with group = 0, floating zero points, block_m a multiple
+ * of 128, 2N % 128 == 0 and K % 256 == 0 the call runs the tiled MFMA kernel over the sorted rows (128 or 256
+ * rows x 128 channels per workgroup).
  */
 int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const void* scale_b,
                         const void* zero_points, const void* topk_weights,
