@@ -51,8 +51,13 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 template <int WBITS, int ADT, bool G128, int SDT, int BM, int REFQ = 0, bool MOE = false>
 __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const int tiles_m, const int tiles,
                                                            const MoeArgs q) {
-    static_assert(!REFQ || (ADT == FNN_F16 && SDT == FNN_F16), "reference rounding: fp16 activations and tables");
-    static_assert(!MOE || (!G128 && REFQ == 0 && WBITS == 4), "the gathered form: int4, per-channel tables");
+    // REFQ = 3: the same software pipeline over the slabs without the per-weight rounding, for per-channel
+    // tables of any type: the operands are the converted integers, the activation sums come from MFMAs
+    // against ones and scale and zero point are applied once at the end.
+    constexpr bool ROUNDQ = REFQ == 1 || REFQ == 2;
+    static_assert(!ROUNDQ || (ADT == FNN_F16 && SDT == FNN_F16), "reference rounding: fp16 activations and tables");
+    static_assert(REFQ != 3 || !G128, "the pipeline without rounding: per-channel tables");
+    static_assert(!MOE || (!G128 && (REFQ == 0 || REFQ == 3) && WBITS == 4), "the gathered form: int4, per-channel tables");
     typedef MfmaT<ADT> MT;
     static_assert(WBITS == 4 || BM == 128, "three stages of 128 int8 weight rows leave room for 128 activation rows");
     constexpr int NH = WBITS == 4 ? 2 : 1;          // channels per weight row
@@ -113,19 +118,22 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     const uint32_t a_chunk = (((lane & 15) ^ (ar0 & 15)) << 4);
     const uint32_t lda2 = (uint32_t)(p.lda * 2);
     const char* const a_base = (const char*)p.act + (MOE ? 0 : (int64_t)m0 * p.lda * 2);
-    uint32_t a_off[MOE ? NCA : 1];                   // MOE: the gathered rows' offsets are kept
+    // MOE: the activation row of every tile row, staged once in the first table stage (per-channel tables
+    // leave the table stages unused); a copy reads its rows from there instead of keeping NCA offsets in registers
+    int* const a_rows = (int*)st0;
     if constexpr (MOE) {
-#pragma unroll
-        for (int i = 0; i < NCA; ++i) {
-            const int tok = q.sorted_ids[m0 + ar0 + 32 * i];
-            a_off[i] = (uint32_t)(tok < q.num_valid ? tok / q.top_k : 0) * lda2 + a_chunk;
+        static_assert(BM * 4 <= TSTG, "the tile's row numbers fit a table stage");
+        for (int r = threadIdx.x; r < BM; r += 512) {
+            const int tok = q.sorted_ids[m0 + r];
+            a_rows[r] = tok < q.num_valid ? tok / q.top_k : 0;
         }
+        __syncthreads();
     }
     auto copy_a = [&](char* stage, int j) {
         const char* src = a_base + (int64_t)min(j, KT - 1) * 256;        // scalar
 #pragma unroll
         for (int i = 0; i < NCA; ++i) {
-            const uint32_t off = MOE ? a_off[i] : (uint32_t)min(ar0 + 32 * i, ar_max) * lda2 + a_chunk;
+            const uint32_t off = (uint32_t)(MOE ? a_rows[ar0 + 32 * i] : min(ar0 + 32 * i, ar_max)) * lda2 + a_chunk;
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + off), (lds_ptr_t)(stage + (i * 8 + wave) * 1024), 16, 0, 0);
         }
         // (the compiler keeps these offsets in registers where it has them to spare)
@@ -196,7 +204,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     // REFQ with per-channel tables: the scale and zero point of the channels this lane's operand rows hold
     const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
     v2h rq_s[NA], rq_z[NA];
-    if constexpr (REFQ != 0 && !G128) {
+    if constexpr (ROUNDQ && !G128) {
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
             const int n = n0 + wn * WTN + (a / NH) * 16 * NH + NH * row16 + (a % NH);
@@ -323,10 +331,12 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
                     else
                         convert_w8<ADT>(w, A[2 * h][f], A[2 * h + 1][f]);
                 }
+            if constexpr (ROUNDQ) {
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
+                for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-                for (int a = 0; a < NA; ++a) A[ks][a] = ref_dq_f16<REFQ == 2>(A[ks][a], rq_c, rq_z[a], rq_s[a]);
+                    for (int a = 0; a < NA; ++a) A[ks][a] = ref_dq_f16<REFQ == 2>(A[ks][a], rq_c, rq_z[a], rq_s[a]);
+            }
         };
         auto mfma_slab = [&](const v4u(&A)[4][NA], const char* sa) {
 #pragma unroll
@@ -335,9 +345,11 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) B[ks] = *(const v4u*)(sa + a_rd[ks >> 1][ks & 1] + b * 16 * 256);
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks)
+                for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
                     for (int a = 0; a < NA; ++a) outv[a][b] = MT::mma(A[ks][a], B[ks], outv[a][b]);
+                    if constexpr (!ROUNDQ) asum[b] = MT::mma(ones, B[ks], asum[b]);
+                }
             }
         };
         // the order asked of the scheduler: per activation fragment its four LDS reads, then each of its MFMAs
@@ -349,9 +361,9 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
             for (int b = 0; b < FB; ++b) {
                 __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-                for (int q = 0; q < 4 * NA; ++q) {
+                for (int q = 0; q < 4 * (NA + (ROUNDQ ? 0 : 1)); ++q) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, ROUNDQ ? 2 : 1, 0);
                 }
             }
         };
@@ -437,7 +449,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
 #undef FNN_TILE_ITER
     }
     // ---- per-channel scales: one fold at the end
-    if constexpr (!G128 && REFQ == 0) {
+    if constexpr (!G128 && !ROUNDQ) {
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
             float sc[4], zc[4];
@@ -470,7 +482,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
             if (!MOE && m >= p.M) continue;
             // (rows converted from bf16 were scaled by a power of two: the exact inverse)
             float un = 1.f;
-            if constexpr (REFQ != 0) un = p.act_unscale ? p.act_unscale[m] : 1.f;
+            if constexpr (ROUNDQ) un = p.act_unscale ? p.act_unscale[m] : 1.f;
             if constexpr (MOE) {       // the output row is the routed row; `un` carries the routing weight
                 m = q.sorted_ids[m];
                 if (m >= q.num_valid) continue;
@@ -517,7 +529,10 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
         WoArgs q;
         if (convert_act_to_f16(p, q, st) && launch_tile_t<WBITS, FNN_F16>(q, st)) return true;
     }
-    const int bm = (p.M <= 128 || WBITS == 8) ? 128 : 256;
+    // 256 rows per workgroup for int4 from 129 rows on - unless the 256-row tiles would leave half the CUs
+    // idle: then twice as many workgroups of 128 rows, each with half the work, finish sooner
+    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * (p.N / 128);
+    const int bm = (p.M <= 128 || WBITS == 8 || tiles256 <= 128) ? 128 : 256;
     const int tiles_m = (p.M + bm - 1) / bm;
     const int tiles = tiles_m * (p.N / 128);
     const dim3 grid(((tiles + 7) / 8) * 8);   // (workgroups beyond the last tile return at once)
@@ -546,7 +561,7 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
         if (p.scale_dtype == FNN_F16) FNN_TILE(true, FNN_F16, 0);
         else FNN_TILE(true, FNN_BF16, 0);
     } else {
-        FNN_TILE(false, FNN_F16, 0);
+        FNN_TILE(false, FNN_F16, 3);
     }
 #undef FNN_TILE
     return true;
@@ -561,8 +576,8 @@ static bool launch_tile_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
     const int tiles = tiles_m * (p.N / 128);
     const dim3 grid(((tiles + 7) / 8) * 8);
     note_kernel("gemm_wo_tile_kernel(moe)", 4, bm, 128);
-    if (bm == 256) gemm_wo_tile_kernel<4, ADT, false, FNN_F16, 256, 0, true><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, q);
-    else gemm_wo_tile_kernel<4, ADT, false, FNN_F16, 128, 0, true><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, q);
+    if (bm == 256) gemm_wo_tile_kernel<4, ADT, false, FNN_F16, 256, 3, true><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, q);
+    else gemm_wo_tile_kernel<4, ADT, false, FNN_F16, 128, 3, true><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, q);
     return true;
 }
 
