@@ -601,9 +601,72 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
         for (int i = 0; i < FN; ++i) ac[i] = *(const v4f*)&sc_col[wn * WTN + i * 16 + 4 * csel];
         // a tile that lies wholly inside the matrix stores without bounds checks (a uniform choice)
         const bool inside = m0 + BM <= p.M && n0 + BN <= p.N && (p.ldc & 7) == 0;
-        auto store_rows = [&](auto guarded) {
-            constexpr bool G = decltype(guarded)::value;
+        // the 16 bytes a lane holds of fragments i and i + 1 (8 consecutive columns of row frow) after the scales,
+        // the conversion and the exchange between the two fragments
+        auto pair_val = [&](int i, int j, float ar, float wr) __attribute__((always_inline)) -> v4u {
+            uint32_t lo[2], hi[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = ((float)acc[i + h][j][e] * ar) * ac[i + h][e];
+                    if constexpr (MOE) {
+                        if (moe.mul_w) v[e] = v[e] * wr;
+                    }
+                }
+                if constexpr (MODE == OUT_BF16) {
+                    lo[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2bf));
+                    hi[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2bf));
+                } else {
+                    lo[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2h));
+                    hi[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2h));
+                }
+            }
+            const v2u sl = __builtin_amdgcn_permlane16_swap(lo[0], lo[1], false, false);
+            const v2u sh = __builtin_amdgcn_permlane16_swap(hi[0], hi[1], false, false);
+            return v4u{sl[0], sh[0], sl[1], sh[1]};
+        };
+        // Inside the matrix: whole 128-byte lines per store instruction.  A fragment pair gives every row 64
+        // contiguous bytes; two pairs side by side (fragments i .. i + 3) give 128, held by lanes of the same
+        // row in two registers.  A rotation by 8 within each row of 16 lanes moves the second pair's bytes of
+        // rows 0..7 to the lanes of rows 8..15 and the first pair's bytes of rows 8..15 the other way, so that
+        // one instruction writes rows 0..7 and the next rows 8..15, 128 bytes of each.  (Half lines, written at
+        // different times, reached memory as partial writes: 1.45 times the output's bytes by the counters.)
+        auto store_full = [&]() {
+            const int r8 = frow & 7, hsel = frow >> 3;
             uint16_t* const obase = (uint16_t*)p.out + (int64_t)(wm0 + frow) * p.ldc + wn0 + nsel;
+            uint16_t* const qbase = (uint16_t*)p.out + (int64_t)(wm0 + r8) * p.ldc + wn0 + hsel * 32 + nsel;
+            auto quad = [&](int i, int j, float ar) __attribute__((always_inline)) {
+                const v4u x = pair_val(i, j, ar, 1.f), y = pair_val(i + 2, j, ar, 1.f);
+                v4u v1, v2;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    v1[k] = (uint32_t)__builtin_amdgcn_update_dpp((int)x[k], (int)y[k], 0x128, 0xF, 0xC, false);
+                    v2[k] = (uint32_t)__builtin_amdgcn_update_dpp((int)y[k], (int)x[k], 0x128, 0xF, 0x3, false);
+                }
+                __builtin_nontemporal_store(v1, (v4u*)(qbase + (int64_t)(j * 16) * p.ldc + i * 16));
+                __builtin_nontemporal_store(v2, (v4u*)(qbase + (int64_t)(j * 16 + 8) * p.ldc + i * 16));
+            };
+            auto pair = [&](int i, int j, float ar) __attribute__((always_inline)) {
+                __builtin_nontemporal_store(pair_val(i, j, ar, 1.f), (v4u*)(obase + (int64_t)(j * 16) * p.ldc + i * 16));
+            };
+#pragma unroll
+            for (int j = 0; j < FM; ++j) {
+                const float ar = sc_row[wm * WTM + j * 16 + frow];
+                if constexpr (FN % 4 == 0) {
+#pragma unroll
+                    for (int i = 0; i < FN; i += 4) quad(i, j, ar);
+                } else {
+                    // six fragments (192 bytes a row): the wave's lines are its first two pairs (wn = 0) or its
+                    // last two (wn = 1); the pair in the middle of the tile's row shares its line with the other wave
+                    static_assert(FN % 4 == 0 || FN == 6, "wave tiles of 64, 96 or 128 columns");
+                    if (wn == 0) { quad(0, j, ar); pair(4, j, ar); }
+                    else { pair(0, j, ar); quad(2, j, ar); }
+                }
+            }
+        };
+        auto store_rows = [&]() {
 #pragma unroll
             for (int j = 0; j < FM; ++j) {
                 const float ar = sc_row[wm * WTM + j * 16 + frow];
@@ -617,48 +680,23 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
                 }
 #pragma unroll
                 for (int i = 0; i < FN; i += 2) {
-                    uint32_t lo[2], hi[2];
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        float v[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            v[e] = ((float)acc[i + h][j][e] * ar) * ac[i + h][e];
-                            if constexpr (MOE) {
-                                if (moe.mul_w) v[e] = v[e] * wr;
-                            }
-                        }
-                        if constexpr (MODE == OUT_BF16) {
-                            lo[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2bf));
-                            hi[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2bf));
+                    const v4u val = pair_val(i, j, ar, wr);
+                    const int n = wn0 + i * 16 + nsel;
+                    if ((MOE ? row_ok : m < p.M) && n < p.N) {
+                        uint16_t* o = (uint16_t*)p.out + (int64_t)m * p.ldc + n;
+                        if (n + 7 < p.N && (p.ldc & 7) == 0) {
+                            __builtin_nontemporal_store(val, (v4u*)o);
                         } else {
-                            lo[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[0], v[1]}, v2h));
-                            hi[h] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2f{v[2], v[3]}, v2h));
-                        }
-                    }
-                    const v2u sl = __builtin_amdgcn_permlane16_swap(lo[0], lo[1], false, false);
-                    const v2u sh = __builtin_amdgcn_permlane16_swap(hi[0], hi[1], false, false);
-                    const v4u val = v4u{sl[0], sh[0], sl[1], sh[1]};
-                    if constexpr (!G) {
-                        __builtin_nontemporal_store(val, (v4u*)(obase + (int64_t)(j * 16) * p.ldc + i * 16));
-                    } else {
-                        const int n = wn0 + i * 16 + nsel;
-                        if ((MOE ? row_ok : m < p.M) && n < p.N) {
-                            uint16_t* o = (uint16_t*)p.out + (int64_t)m * p.ldc + n;
-                            if (n + 7 < p.N && (p.ldc & 7) == 0) {
-                                __builtin_nontemporal_store(val, (v4u*)o);
-                            } else {
 #pragma unroll
-                                for (int q = 0; q < 8; ++q)
-                                    if (n + q < p.N) o[q] = (uint16_t)(val[q >> 1] >> (16 * (q & 1)));
-                            }
+                            for (int q = 0; q < 8; ++q)
+                                if (n + q < p.N) o[q] = (uint16_t)(val[q >> 1] >> (16 * (q & 1)));
                         }
                     }
                 }
             }
         };
-        if (inside && !MOE) store_rows(std::false_type{});
-        else store_rows(std::true_type{});
+        if (inside && !MOE) store_full();
+        else store_rows();
     }
 }
 
