@@ -633,36 +633,53 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
         // rows 0..7 to the lanes of rows 8..15 and the first pair's bytes of rows 8..15 the other way, so that
         // one instruction writes rows 0..7 and the next rows 8..15, 128 bytes of each.  (Half lines, written at
         // different times, reached memory as partial writes: 1.45 times the output's bytes by the counters.)
-        auto store_full = [&]() {
+        // RG: rows are checked (the tile's last rows may lie beyond M; MOE: a row goes to its routed row, padding
+        // rows are not stored); the columns all lie inside the matrix.
+        auto store_full = [&](auto row_guard) {
+            constexpr bool RG = decltype(row_guard)::value;
             const int r8 = frow & 7, hsel = frow >> 3;
-            uint16_t* const obase = (uint16_t*)p.out + (int64_t)(wm0 + frow) * p.ldc + wn0 + nsel;
-            uint16_t* const qbase = (uint16_t*)p.out + (int64_t)(wm0 + r8) * p.ldc + wn0 + hsel * 32 + nsel;
-            auto quad = [&](int i, int j, float ar) __attribute__((always_inline)) {
-                const v4u x = pair_val(i, j, ar, 1.f), y = pair_val(i + 2, j, ar, 1.f);
+            // the output row of tile row r, or -1
+            auto out_row = [&](int r) __attribute__((always_inline)) -> int64_t {
+                if constexpr (MOE) {
+                    const int t = sc_tok[r];
+                    return t < moe.num_valid ? t : -1;
+                } else {
+                    return !RG || m0 + r < p.M ? m0 + r : -1;
+                }
+            };
+            uint16_t* const cbase = (uint16_t*)p.out + wn0 + nsel;
+            auto quad = [&](int i, int j, float ar, float wr) __attribute__((always_inline)) {
+                const v4u x = pair_val(i, j, ar, wr), y = pair_val(i + 2, j, ar, wr);
                 v4u v1, v2;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     v1[k] = (uint32_t)__builtin_amdgcn_update_dpp((int)x[k], (int)y[k], 0x128, 0xF, 0xC, false);
                     v2[k] = (uint32_t)__builtin_amdgcn_update_dpp((int)y[k], (int)x[k], 0x128, 0xF, 0x3, false);
                 }
-                __builtin_nontemporal_store(v1, (v4u*)(qbase + (int64_t)(j * 16) * p.ldc + i * 16));
-                __builtin_nontemporal_store(v2, (v4u*)(qbase + (int64_t)(j * 16 + 8) * p.ldc + i * 16));
+                const int64_t ra = out_row(wm * WTM + j * 16 + r8), rb = out_row(wm * WTM + j * 16 + 8 + r8);
+                if (!RG || ra >= 0) __builtin_nontemporal_store(v1, (v4u*)(cbase + ra * p.ldc + hsel * 32 + i * 16));
+                if (!RG || rb >= 0) __builtin_nontemporal_store(v2, (v4u*)(cbase + rb * p.ldc + hsel * 32 + i * 16));
             };
-            auto pair = [&](int i, int j, float ar) __attribute__((always_inline)) {
-                __builtin_nontemporal_store(pair_val(i, j, ar, 1.f), (v4u*)(obase + (int64_t)(j * 16) * p.ldc + i * 16));
+            auto pair = [&](int i, int j, float ar, float wr) __attribute__((always_inline)) {
+                const v4u v = pair_val(i, j, ar, wr);
+                const int64_t r = out_row(wm * WTM + j * 16 + frow);
+                if (!RG || r >= 0) __builtin_nontemporal_store(v, (v4u*)(cbase + r * p.ldc + i * 16));
             };
 #pragma unroll
             for (int j = 0; j < FM; ++j) {
                 const float ar = sc_row[wm * WTM + j * 16 + frow];
+                float wr = 1.f;
+                if constexpr (MOE) wr = sc_wr[wm * WTM + j * 16 + frow];
                 if constexpr (FN % 4 == 0) {
 #pragma unroll
-                    for (int i = 0; i < FN; i += 4) quad(i, j, ar);
+                    for (int i = 0; i < FN; i += 4) quad(i, j, ar, wr);
                 } else {
                     // six fragments (192 bytes a row): the wave's lines are its first two pairs (wn = 0) or its
-                    // last two (wn = 1); the pair in the middle of the tile's row shares its line with the other wave
+                    // last two (wn = 1); the pair in the middle of the tile's row shares its line with the other
+                    // wave (handing the halves over through LDS so that one wave writes it whole gained nothing)
                     static_assert(FN % 4 == 0 || FN == 6, "wave tiles of 64, 96 or 128 columns");
-                    if (wn == 0) { quad(0, j, ar); pair(4, j, ar); }
-                    else { pair(0, j, ar); quad(2, j, ar); }
+                    if (wn == 0) { quad(0, j, ar, wr); pair(4, j, ar, wr); }
+                    else { pair(0, j, ar, wr); quad(2, j, ar, wr); }
                 }
             }
         };
@@ -695,7 +712,9 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
                 }
             }
         };
-        if (inside && !MOE) store_full();
+        const bool cols_inside = n0 + BN <= p.N && (p.ldc & 7) == 0;
+        if (inside && !MOE) store_full(std::false_type{});
+        else if (cols_inside) store_full(std::true_type{});
         else store_rows();
     }
 }
