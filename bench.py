@@ -226,6 +226,43 @@ def main():
         sustained[label] = round(rate.value, 1)
     roofline["mfma_only_sustained"] = dict(sustained, unit="TOP/s")
     roofline["frac_of_sustained_random"] = round(gemm_tops / sustained["random_operand_bytes"], 4)
+    # what the memory side delivers without arithmetic: the tile's copy pattern alone (direct-to-LDS copies of
+    # 448 rows x 128 bytes per slab, one workgroup per CU, over the QKV operands' row length), and a stream of
+    # the decode GEMV's request pattern over the bytes of its weights
+    probe.fnn_probe_copy_rate.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                          ctypes.c_int, ctypes.c_void_p, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+    probe.fnn_probe_stream_rate.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
+                                            ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+    src = torch.randint(-128, 128, (1 << 29,), dtype=torch.int8, device=dev)     # 512 MiB
+    rate = ctypes.c_double(0.0)
+    rc = probe.fnn_probe_copy_rate(_lib.ptr(src), 200 << 20, 4096, 32, 2, 50, _lib.ptr(sink), ctypes.byref(rate),
+                                   _lib.current_stream(torch.device(dev)))
+    if rc != 0:
+        sys.exit(f"bench.py: the copy rate probe failed with hipError {rc}")
+    tile_bytes = (256 + 192) * 4096
+    roofline["copy_only"] = {"GBps_per_cu": round(rate.value, 1), "pattern": "448 rows x 128 B per slab, direct to LDS, one workgroup per CU, rows shared within an XCD as in the kernel",
+                             "kernel_GBps_per_cu": round(2 * tile_bytes / (primary["ms_gemm"] * 1e-3) / 1e9, 1)}
+    a16w4_bytes = 28672 * 8192 // 2 + 4 * 64 * 28672
+    rc = probe.fnn_probe_stream_rate(_lib.ptr(src), a16w4_bytes, 100, _lib.ptr(sink), ctypes.byref(rate),
+                                     _lib.current_stream(torch.device(dev)))
+    if rc != 0:
+        sys.exit(f"bench.py: the stream rate probe failed with hipError {rc}")
+    stream_hot = rate.value
+    # ... and with the range moving through 500 MB, so that nothing is left in the caches from the launch before
+    t_cold = []
+    for rep in range(24):
+        off = (rep % 4) * a16w4_bytes // 4096 * 4096
+        rc = probe.fnn_probe_stream_rate(src.data_ptr() + off, a16w4_bytes, 1, _lib.ptr(sink), ctypes.byref(rate),
+                                         _lib.current_stream(torch.device(dev)))
+        if rc != 0:
+            sys.exit(f"bench.py: the stream rate probe failed with hipError {rc}")
+        t_cold.append(rate.value)
+    t_cold.sort()
+    roofline["stream_only"] = {"bytes": a16w4_bytes, "TBps_rotating": round(t_cold[len(t_cold) // 2], 2),
+                               "TBps_same_range": round(stream_hot, 2),
+                               "pattern": "9 non-temporal 16-byte loads per lane in flight, 8 waves per CU, launch gap included"}
+    del src
+    torch.cuda.empty_cache()
 
     # ------------------------------------------------------- c1: DynamicQuant + A8W8, M = 16, fp16 out
     x1_cpu = workloads.activations(16, 4096, torch.float16, seed=10)
