@@ -138,6 +138,12 @@ def _a8w8_workspace(lib, device, stream, M, N, K):
         need = _A8W8_WS_BYTES[(M, N, K)] = int(lib.fnn_gemm_a8w8_workspace_bytes(M, N, K))
     if need == 0:
         return None
+    return _a8w8_workspace_of(device, stream, need)
+
+
+def _a8w8_workspace_of(device, stream, need):
+    """This device's and stream's workspace, at least `need` bytes (and large enough for every plan of the
+    library's own)."""
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     ws = _A8W8_WORKSPACES.get(key)
     if ws is None or ws.numel() < need:
@@ -151,9 +157,10 @@ def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col, tile=None):
     """Replaces triton_gemm_a8w8_forward (flashnn/triton_kernels/gemm_a8w8.py:182-221).
 
     Unlike the Triton launcher the scale type need not equal the output type: fp16, bf16 and
-    fp32 scales are accepted in any combination.  `tile` = (rows, columns, waves) names a tile of
-    the MFMA kernel and bypasses the tuned-configuration lookup (not part of the reference's
-    signature; the results are the same bits for every tile)."""
+    fp32 scales are accepted in any combination.  `tile` = (rows, columns, waves[, parts of K]) names a
+    tile of the MFMA kernel (and a split of K over that many workgroups per tile) and bypasses the
+    tuned-configuration lookup (not part of the reference's signature; the results are the same bits for
+    every choice)."""
     assert a.dtype == torch.int8 and b.dtype == torch.int8, "Matrix A/B must be int8 type"
     assert a.is_contiguous(), "Matrix A must be contiguous"
     assert out.dtype == torch.float16 or out.dtype == torch.bfloat16, \
@@ -176,10 +183,19 @@ def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col, tile=None):
     # shape-keyed tuned tile, named as the reference names the launch (gemm_a8w8.py:199)
     if tile is None:
         tile = tuned_configs.CACHE.shape_tile("gemm_a8w8", M, N, K)
-    if tile is None and get_autotune_triton_kernels():
-        tile = tuned_configs.tune(f"gemm_a8w8_{M}_{N}_{K}", tuned_configs.A8W8_CANDIDATES,
-                                  lambda t: _lib.check(lib.fnn_gemm_a8w8_tiled(*args, *t, stream)))
-    if tile is None or tile[0] == 0:
+    def run_named(t):
+        bm, bn, waves, parts = tuned_configs.as_config(t)
+        if bm == 0:
+            return run_default()
+        if parts > 1:
+            ws = _a8w8_workspace_of(a.device, stream, _A8W8_WS_ALLOC)
+            rc = lib.fnn_gemm_a8w8_ws_tiled(*args, bm, bn, parts, ws.data_ptr(), ws.numel(), stream)
+            if rc != 0:
+                _A8W8_WORKSPACES.clear()
+            return _lib.check(rc)
+        return _lib.check(lib.fnn_gemm_a8w8_tiled(*args, bm, bn, waves, stream))
+
+    def run_default():
         ws = _a8w8_workspace(lib, a.device, stream, M, N, K) if M > 64 else None
         if ws is None:
             _lib.check(lib.fnn_gemm_a8w8(*args, stream))
@@ -189,8 +205,13 @@ def hip_gemm_a8w8_forward(out, a, b, alpha_row, alpha_col, tile=None):
                 # a split call that failed half way may have left counters behind: never reuse the buffer
                 _A8W8_WORKSPACES.clear()
             _lib.check(rc)
+
+    if tile is None and get_autotune_triton_kernels():
+        tile = tuned_configs.tune(f"gemm_a8w8_{M}_{N}_{K}", tuned_configs.A8W8_CANDIDATES, run_named)
+    if tile is None:
+        run_default()
     else:
-        _lib.check(lib.fnn_gemm_a8w8_tiled(*args, *tile, stream))
+        run_named(tile)
     return out
 
 

@@ -10,7 +10,9 @@ processes, the recorded configuration is used without timing anything.  With tun
 recorded configurations are still honoured; shapes without one take the library's static choice.
 
 File format (the reference's, triton_utils.py:38-57): {method_name: [kwargs, launch_options]} with
-kwargs = {"BLOCK_M": .., "BLOCK_N": ..} ((0, 0) = the library's own choice) and launch_options =
+kwargs = {"BLOCK_M": .., "BLOCK_N": ..} ((0, 0) = the library's own choice, its own split of K included), an
+optional "SPLIT_K": n (K cut into n parts per tile, met through the launcher's workspace; the name the
+reference's weight-only kernels give the notion, gemm_a16w8.py:17-80; absent = 1) and launch_options =
 {"num_warps": 4} (absent = the tile's default; every tile runs four waves), the reference's own option names (gemm_a8w8.py:17-50).
 The file lives at $FLASHNN_AMD_TUNED_CONFIGS or flashnn_amd/configs/hip_autotune_best_configs.json.
 FORECE_RE_TUNE_TRITON_KERNELS (the reference's spelling, triton_utils.py:22-24) lists method-name
@@ -22,9 +24,20 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 JSON_FILENAME = "hip_autotune_best_configs.json"
 
-# candidate (rows, columns, waves) of the A8W8 MFMA kernel; (0, 0, 0) = static choice (which may be a
-# few-row kernel); waves = 0 is the tile's default (four)
-A8W8_CANDIDATES = [(0, 0, 0), (256, 256, 0), (256, 192, 0), (256, 128, 0), (128, 128, 0), (64, 128, 0)]
+# candidate (rows, columns, waves, parts of K) of the A8W8 MFMA kernel; (0, 0, 0, 0) = static choice (which may
+# be a few-row kernel, or a split of its own); waves = 0 is the tile's default (four).  Splits a shape does not
+# admit (parts shorter than four slabs, M or N too small) are refused by the library and skipped by tune().
+A8W8_CANDIDATES = [(0, 0, 0, 0), (256, 256, 0, 1), (256, 192, 0, 1), (256, 128, 0, 1), (128, 128, 0, 1), (64, 128, 0, 1),
+                   (128, 128, 0, 2), (128, 128, 0, 3), (128, 128, 0, 4), (128, 128, 0, 6), (128, 128, 0, 8)]
+
+
+def as_config(tile):
+    """(rows, columns[, waves[, parts]]) -> the full 4-tuple; a named tile without parts is unsplit."""
+    t = tuple(int(v) for v in tile)
+    t = t + (0,) * (3 - len(t)) if len(t) < 3 else t
+    if len(t) == 3:
+        t = t + ((1,) if t[0] else (0,))
+    return t
 
 
 def json_file_path():
@@ -40,13 +53,17 @@ def force_re_tune(method_name):
 
 
 def serialize_best_config(tile):
-    waves = int(tile[2]) if len(tile) > 2 else 0
-    return [{"BLOCK_M": int(tile[0]), "BLOCK_N": int(tile[1])}, {"num_warps": waves} if waves else {}]
+    bm, bn, waves, parts = as_config(tile)
+    kwargs = {"BLOCK_M": bm, "BLOCK_N": bn}
+    if parts > 1:
+        kwargs["SPLIT_K"] = parts
+    return [kwargs, {"num_warps": waves} if waves else {}]
 
 
 def deserialize_best_config(entry):
     kwargs, options = entry[0], entry[1] if len(entry) > 1 else {}
-    return int(kwargs["BLOCK_M"]), int(kwargs["BLOCK_N"]), int(options.get("num_warps", 0))
+    bm = int(kwargs["BLOCK_M"])
+    return bm, int(kwargs["BLOCK_N"]), int(options.get("num_warps", 0)), int(kwargs.get("SPLIT_K", 1 if bm else 0))
 
 
 class TunedConfigs:
@@ -113,11 +130,17 @@ CACHE = TunedConfigs()
 
 def tune(method_name, candidates, run, reps=5):
     """Times run(candidate) for every candidate with GPU events (one warm-up call, then the median of
-    `reps` calls each), records and returns the fastest."""
+    `reps` calls each), records and returns the fastest.  A candidate the library refuses for this shape
+    (run raises) is skipped; the first candidate must be one that every shape admits."""
     import torch
     best, best_ms = candidates[0], float("inf")
-    for cand in candidates:
-        run(cand)
+    for n, cand in enumerate(candidates):
+        try:
+            run(cand)
+        except Exception:
+            if n == 0:
+                raise
+            continue
         torch.cuda.synchronize()
         times = []
         for _ in range(reps):

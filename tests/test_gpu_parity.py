@@ -509,6 +509,54 @@ def test_a8w8_tuned_config_cache(tmp_path, monkeypatch):
     assert np.array_equal(plain.float().numpy(), want)
 
 
+def test_a8w8_tuned_config_with_split_k(tmp_path, monkeypatch):
+    """A long-K shape with few tiles: the candidates include splits of K (met through the launcher's
+    workspace); whatever wins is recorded with its SPLIT_K and used again, and every candidate - the named
+    splits included - gives the bits of the plain call.  Splits the shape does not admit are skipped."""
+    import json
+    from flashnn_amd import tuned_configs as TC
+    path = tmp_path / "best.json"
+    monkeypatch.setenv("FLASHNN_AMD_TUNED_CONFIGS", str(path))
+    TC.CACHE.reset()
+    M, N, K = 200, 1024, 8192
+    a, b = _rand_i8((M, K), 41), _rand_i8((N, K), 42)
+    g = torch.Generator().manual_seed(43)
+    ar, ac = (torch.rand(M, generator=g) * 0.05).half(), (torch.rand(N, generator=g) * 0.05).half()
+    ad, bd, ard, acd = a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV)
+    want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.numpy(), b.numpy()), O.to_np(ar), O.to_np(ac), O.BF16)
+    for cand in TC.A8W8_CANDIDATES:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        launchers.hip_gemm_a8w8_forward(out, ad, bd, ard, acd, tile=cand)
+        if cand[3] > 1:
+            assert _lib.last_kernel() == f"gemm_a8w8_ring_kernel(split K)<128,128,{cand[3]}>"
+        assert np.array_equal(out.float().cpu().numpy(), want), cand
+    with pytest.raises(_lib.FlashnnHipError):      # 64 slabs cannot make 17 parts of four
+        launchers.hip_gemm_a8w8_forward(out, ad, bd, ard, acd, tile=(128, 128, 0, 17))
+    op = flashnn_amd.GemmA8W8(torch.bfloat16)
+    flashnn_amd.set_autotune_triton_kernels(True)
+    try:
+        tuned = op(ad, bd, ard, acd)
+    finally:
+        flashnn_amd.set_autotune_triton_kernels(False)
+    entry = json.load(open(path))[f"gemm_a8w8_{M}_{N}_{K}"]
+    tile = TC.deserialize_best_config(entry)
+    assert tile in TC.A8W8_CANDIDATES and (tile[3] <= 1) == ("SPLIT_K" not in entry[0])
+    again = op(ad, bd, ard, acd)
+    assert np.array_equal(tuned.float().cpu().numpy(), want) and torch.equal(tuned, again)
+    # a short K admits no split at all: the tuner skips those candidates instead of failing
+    a2, b2 = _rand_i8((96, 640), 44), _rand_i8((256, 640), 45)
+    flashnn_amd.set_autotune_triton_kernels(True)
+    try:
+        short = flashnn_amd.GemmA8W8(torch.float16)(a2.to(DEV), b2.to(DEV), ard[:96], acd[:256])
+    finally:
+        flashnn_amd.set_autotune_triton_kernels(False)
+    want2 = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a2.numpy(), b2.numpy()), O.to_np(ar[:96]), O.to_np(ac[:256]), O.F16)
+    assert np.array_equal(short.float().cpu().numpy(), want2)
+    assert TC.deserialize_best_config(json.load(open(path))["gemm_a8w8_96_256_640"])[3] <= 1
+    monkeypatch.undo()
+    TC.CACHE.reset()
+
+
 # ------------------------------------------------------------------ mixture of experts
 @pytest.mark.parametrize("out_ty", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("mul_w", [False, True])

@@ -177,24 +177,30 @@ def test_tuned_config_file_format_and_lookup(tmp_path, monkeypatch):
                     "gemm_a8w8_16_4096_4096": [{"BLOCK_M": 0, "BLOCK_N": 0}, {}]}
     # a fresh view (another process) reads the file back
     other = TC.TunedConfigs()
-    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 192, 4) and other.lookup("gemm_a8w8_1_1_1") is None
+    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 192, 4, 1) and other.lookup("gemm_a8w8_1_1_1") is None
     # forced re-tune by method-name prefix, once per process
     monkeypatch.setenv("FORECE_RE_TUNE_TRITON_KERNELS", "gemm_a8w8_2048;fuse_moe")
     assert TC.force_re_tune("gemm_a8w8_2048_12288_4096") and not TC.force_re_tune("gemm_a8w8_16_4096_4096")
-    assert other.lookup("gemm_a8w8_2048_12288_4096") is None and other.lookup("gemm_a8w8_16_4096_4096") == (0, 0, 0)
+    assert other.lookup("gemm_a8w8_2048_12288_4096") is None and other.lookup("gemm_a8w8_16_4096_4096") == (0, 0, 0, 0)
     other.record("gemm_a8w8_2048_12288_4096", (256, 128, 0))
-    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 128, 0)
+    assert other.lookup("gemm_a8w8_2048_12288_4096") == (256, 128, 0, 1)
     # the per-shape answer a launcher uses: resolved once, dropped by a new record or reset()
-    assert other.shape_tile("gemm_a8w8", 16, 4096, 4096) == (0, 0, 0) and other.shape_tile("gemm_a8w8", 1, 1, 1) is None
+    assert other.shape_tile("gemm_a8w8", 16, 4096, 4096) == (0, 0, 0, 0) and other.shape_tile("gemm_a8w8", 1, 1, 1) is None
     other.record("gemm_a8w8_1_1_1", (64, 128, 0))
-    assert other.shape_tile("gemm_a8w8", 1, 1, 1) == (64, 128, 0)
+    assert other.shape_tile("gemm_a8w8", 1, 1, 1) == (64, 128, 0, 1)
+    # a split of K is part of the record (absent = 1)
+    other.record("gemm_a8w8_256_4096_8192", (128, 128, 0, 4))
+    assert json.load(open(path))["gemm_a8w8_256_4096_8192"] == [{"BLOCK_M": 128, "BLOCK_N": 128, "SPLIT_K": 4}, {}]
+    assert TC.TunedConfigs().lookup("gemm_a8w8_256_4096_8192") == (128, 128, 0, 4)
     os.remove(path)
-    assert other.shape_tile("gemm_a8w8", 1, 1, 1) == (64, 128, 0)       # answered without touching the file
+    assert other.shape_tile("gemm_a8w8", 1, 1, 1) == (64, 128, 0, 1)       # answered without touching the file
     other.reset()
     assert other.shape_tile("gemm_a8w8", 1, 1, 1) is None
     assert TC.serialize_best_config((128, 128)) == [{"BLOCK_M": 128, "BLOCK_N": 128}, {}]
-    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 192}, {}]) == (256, 192, 0)
-    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 256}, {"num_warps": 4}]) == (256, 256, 4)
+    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 192}, {}]) == (256, 192, 0, 1)
+    assert TC.deserialize_best_config([{"BLOCK_M": 256, "BLOCK_N": 256}, {"num_warps": 4}]) == (256, 256, 4, 1)
+    assert TC.deserialize_best_config([{"BLOCK_M": 0, "BLOCK_N": 0}, {}]) == (0, 0, 0, 0)
+    assert TC.as_config((128, 128)) == (128, 128, 0, 1) and TC.as_config((0, 0, 0)) == (0, 0, 0, 0)
 
 
 def test_tiled_entry_rejects_unknown_tiles(hip_lib):
