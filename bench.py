@@ -546,6 +546,17 @@ def main():
             secondary.append(_entry(f"fused_moe_a16w4 per-channel tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block={blk} "
                                     f"({rows_padded} sorted rows)", ms, "mfma16", 2.0 * Mt * top_k * Nm * Km, kern,
                                     f"moe a16w4 {Mt} tokens block {blk}"))
+        # ... and tables per group of 128 in the launcher's [E, N, K/128] layout (128-row tiles, fp32 scaling per slab)
+        sc4 = (torch.rand(E, Nm, Km // 128, device=dev, generator=g) * 9e-3 + 1e-3).to(torch.bfloat16)
+        zp4m = torch.randint(-3, 4, (E, Nm, Km // 128), device=dev, generator=g).to(torch.bfloat16)
+        sid, eid, used = workloads.moe_align_block_size(tid, 128, E)
+        rows_padded = int(used[0])
+        twd, tidd, sid, eid, used = [t.to(dev) for t in (tw.float().contiguous(), tid, sid, eid, used)]
+        f = lambda i: flashnn_amd.fused_moe_a16w4_forward(a4, b4, cm, sc4, zp4m, twd, tidd, sid, eid, used, True, top_k, 128)
+        kern = kernel_of(f)
+        ms, _ = _timed(f, 5, torch)
+        secondary.append(_entry(f"fused_moe_a16w4 group 128 tokens={Mt} E={E} top_k={top_k} K={Km} N={Nm} block=128 "
+                                f"({rows_padded} sorted rows)", ms, "mfma16", 2.0 * Mt * top_k * Nm * Km, kern))
         del b4
         torch.cuda.empty_cache()
 

@@ -57,7 +57,10 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     constexpr bool ROUNDQ = REFQ == 1 || REFQ == 2;
     static_assert(!ROUNDQ || (ADT == FNN_F16 && SDT == FNN_F16), "reference rounding: fp16 activations and tables");
     static_assert(REFQ != 3 || !G128, "the pipeline without rounding: per-channel tables");
-    static_assert(!MOE || (!G128 && (REFQ == 0 || REFQ == 3) && WBITS == 4), "the gathered form: int4, per-channel tables");
+    // The gathered form takes per-channel tables (pipelined, REFQ = 3) or tables per group of 128 in the
+    // layout of the reference's MoE launcher, [expert][channel][group] (fp32 scaling per slab, 128-row tiles):
+    // the tile's slice of both tables is transposed into LDS once, in the format of a table stage per group.
+    static_assert(!MOE || (WBITS == 4 && ((!G128 && REFQ == 3) || (G128 && REFQ == 0 && BM == 128))), "the gathered form");
     typedef MfmaT<ADT> MT;
     static_assert(WBITS == 4 || BM == 128, "three stages of 128 int8 weight rows leave room for 128 activation rows");
     constexpr int NH = WBITS == 4 ? 2 : 1;          // channels per weight row
@@ -81,6 +84,8 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     __shared__ __attribute__((aligned(1024))) char st0[TSTG];
     __shared__ __attribute__((aligned(1024))) char st1[TSTG];
     __shared__ __attribute__((aligned(1024))) char st2[TSTG];
+    constexpr int kMoeGroups = 64;                   // K / 128 at most, where the gathered form has group tables
+    __shared__ __attribute__((aligned(1024))) char mtab[MOE && G128 ? kMoeGroups * TSTG / 2 : 16];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -127,6 +132,16 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
             const int tok = q.sorted_ids[m0 + r];
             a_rows[r] = tok < q.num_valid ? tok / q.top_k : 0;
         }
+        if constexpr (G128) {
+            // group g of the tile: 256 bytes of scales, then 256 of zero points, channel by channel
+            const uint16_t* const sc = (const uint16_t*)p.scale + (int64_t)expert * q.stride_scale_be + (int64_t)n0 * KT;
+            const uint16_t* const zp = p.zp ? (const uint16_t*)p.zp + (int64_t)expert * q.stride_zp_be + (int64_t)n0 * KT : nullptr;
+            for (int e = threadIdx.x; e < BN * KT; e += 512) {
+                const int ch = e / KT, g2 = e - ch * KT;
+                *(uint16_t*)(mtab + g2 * 512 + ch * 2) = sc[e];
+                *(uint16_t*)(mtab + g2 * 512 + 256 + ch * 2) = zp ? zp[e] : (uint16_t)0;
+            }
+        }
         __syncthreads();
     }
     auto copy_a = [&](char* stage, int j) {
@@ -162,7 +177,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     const char* const t_src = (lane & 16) && has_zp ? (const char*)p.zp : (const char*)p.scale;
     const uint32_t gt = (uint32_t)n0 * 2 + (lane & 15) * 16;
     auto copy_t = [&](char* stage, int j) {
-        if constexpr (G128) {
+        if constexpr (G128 && !MOE) {
             const int64_t off = (int64_t)min(j, KT - 1) * p.N * 2;
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(t_src + off + gt), (lds_ptr_t)stage, 16, 0, 0);
         }
@@ -421,7 +436,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
         copy_t(FT, (J) + 1);                                              \
         copy_w(FW, (J) + 2);                                              \
         __builtin_amdgcn_sched_barrier(0);                                \
-        slab(CA, CW, CT);                                                 \
+        slab(CA, CW, MOE && G128 ? mtab + (J) * 512 : CT);                \
         __builtin_amdgcn_sched_barrier(0);                                \
     } while (0)
 
@@ -571,6 +586,17 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
 // form does not apply.
 template <int ADT>
 static bool launch_tile_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
+    if (p.group == 128) {
+        const int tiles_m = p.M / 128;
+        const int tiles = tiles_m * (p.N / 128);
+        const dim3 grid(((tiles + 7) / 8) * 8);
+        note_kernel("gemm_wo_tile_kernel(moe, group tables)", 4, 128, 128);
+        if (p.scale_dtype == FNN_F16)
+            gemm_wo_tile_kernel<4, ADT, true, FNN_F16, 128, 0, true><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, q);
+        else
+            gemm_wo_tile_kernel<4, ADT, true, FNN_BF16, 128, 0, true><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, q);
+        return true;
+    }
     const int bm = q.block_m % 256 == 0 ? 256 : 128;
     const int tiles_m = p.M / bm;
     const int tiles = tiles_m * (p.N / 128);
@@ -583,11 +609,16 @@ static bool launch_tile_moe_t(WoArgs& p, const MoeArgs& q, hipStream_t st) {
 
 bool launch_wo_tile_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t st) {
     const int64_t rows = (q.num_valid + q.top_k - 1) / q.top_k;          // activation rows
-    const bool ok = p.group == 0 && q.block_m % 128 == 0 && q.EM % q.block_m == 0 && p.N % 128 == 0 &&
+    const int G = p.K / 128;
+    // group tables: contiguous [expert][channel][group] of one 16-bit type, at most 64 groups
+    const bool tables_ok = p.group == 0 ? q.stride_scale_n == 1 && (!p.zp || (q.stride_zp_n == 1 && p.zp_dtype != FNN_I8))
+                                        : p.group == 128 && G <= 64 && is16(p.scale_dtype) && q.stride_scale_k == 1 &&
+                                              q.stride_scale_n == G &&
+                                              (!p.zp || (p.zp_dtype == p.scale_dtype && q.stride_zp_k == 1 && q.stride_zp_n == G));
+    const bool ok = tables_ok && q.block_m % 128 == 0 && q.EM % q.block_m == 0 && p.N % 128 == 0 &&
                     p.K % 256 == 0 && p.K >= 512 && p.lda % 8 == 0 && p.ldw % 16 == 0 &&
                     q.stride_be % 16 == 0 && ((uintptr_t)p.qw % 16) == 0 && ((uintptr_t)p.act % 16) == 0 &&
                     rows * p.lda * 2 < (1LL << 32) && (int64_t)64 * p.ldw < (1LL << 31) &&
-                    q.stride_scale_n == 1 && (!p.zp || (q.stride_zp_n == 1 && p.zp_dtype != FNN_I8)) &&
                     (int64_t)(p.M / 128) * (p.N / 128) < (1LL << 31);
     if (!ok) return false;
     return act_dtype == FNN_F16 ? launch_tile_moe_t<FNN_F16>(p, q, st) : launch_tile_moe_t<FNN_BF16>(p, q, st);

@@ -351,9 +351,10 @@ int fnn_fused_moe_a8w8(void* c, const void* a, const void* b, const void* alpha_
  * N % 16 == 0, K >= 1024, block_m % 16 == 0, EM % block_m == 0 and 16-byte aligned rows; anything else
  * takes a slow guarded kernel.  The reference multiplies the dequantised weights of a K block by their scale
  * before the dot product and rounds them to the scale type; here the block's dot product is scaled
- * afterwards, in fp32.  Many routed rows per expert: with group = 0, floating zero points, block_m a multiple
- * of 128, 2N % 128 == 0 and K % 256 == 0 the call runs the tiled MFMA kernel over the sorted rows (128 or 256
- * rows x 128 channels per workgroup).
+ * afterwards, in fp32.  Many routed rows per expert: with block_m a multiple of 128, 2N % 128 == 0, K % 256 == 0
+ * and either group = 0 with floating zero points or group = 128 with contiguous tables of one 16-bit type
+ * (zero points in the scales' type, K <= 8192) the call runs the tiled MFMA kernel over the sorted rows (128 or
+ * 256 rows x 128 channels per workgroup).
  */
 int fnn_fused_moe_a16w4(void* c, const void* a, const void* b, const void* scale_b,
                         const void* zero_points, const void* topk_weights,
