@@ -1308,6 +1308,68 @@ def test_quant_gemm_step_under_graph_capture():
         assert bool(out.abs().sum() > 0)
 
 
+def test_split_k_packed_decode_and_moe_under_graph_capture():
+    """The paths with state beyond inputs and outputs, captured into a HIP graph: an A8W8 GEMM whose K the
+    library splits through the launcher's workspace (counters must be back at zero after every replay), the
+    decode on packed weights, the tiled weight-only GEMM on bf16 rows (its scratch comes from torch's caching
+    allocator inside the capture) and a fused MoE on the tiled kernel.  Every replay, with fresh inputs and
+    eager work in between, equals the eager result."""
+    M, K, N = 256, 8192, 2048
+    w, ws = workloads.int8_weights(N, K, seed=91)
+    wd, wsd = w.to(DEV), ws.to(DEV)
+    a8 = torch.zeros(M, K, dtype=torch.int8, device=DEV)
+    sr = (torch.rand(M, device=DEV) * 1e-2).half()
+    out8 = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    packed, scale, zp, _, _ = workloads.int4_group_weights(1024, K, 128, torch.float16, seed=92)
+    packed, scale, zp = packed.to(DEV), scale.to(DEV), zp.to(DEV)
+    op4 = flashnn_amd.GemmWeightOnly(torch.bfloat16)
+    pk = op4.prepack(packed, scale, zp)
+    xb = torch.zeros(M, K, dtype=torch.bfloat16, device=DEV)
+    outp = torch.empty(1, 1024, dtype=torch.bfloat16, device=DEV)
+    outw = torch.empty(M, 1024, dtype=torch.bfloat16, device=DEV)
+    E, top_k, BM = 4, 2, 128
+    be = torch.randint(-128, 128, (E, 512, 1024), dtype=torch.int8, device=DEV)
+    ace = torch.rand(E, 512, device=DEV) * 1e-2
+    tw, ids = torch.topk(torch.softmax(torch.randn(M, E, generator=torch.Generator().manual_seed(93)), -1), top_k)
+    sid, eid, used = [t.to(DEV) for t in workloads.moe_align_block_size(ids, BM, E)]
+    tw, ids = tw.float().contiguous().to(DEV), ids.to(DEV)
+    outm = torch.empty(M, top_k, 512, dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        launchers.hip_gemm_a8w8_forward(out8, a8, wd, sr, wsd)
+        launchers.hip_gemm_a16w4_prepacked_forward(outp, xb[:1], pk)
+        launchers.hip_gemm_a16w4_forward(outw, xb, packed, scale, zero_points=zp)
+        flashnn_amd.fused_moe_a8w8_forward(a8[:, :1024], be, outm, sr, ace, tw, ids, sid, eid, used, True, top_k, BM)
+
+    kernels = []
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up outside the capture (allocates the workspace)
+    torch.cuda.current_stream().wait_stream(side)
+    launchers.hip_gemm_a8w8_forward(out8, a8, wd, sr, wsd)
+    assert _lib.last_kernel().startswith("gemm_a8w8_ring_kernel(split K)")
+    launchers.hip_gemm_a16w4_forward(outw, xb, packed, scale, zero_points=zp)
+    assert _lib.last_kernel().startswith("gemm_wo_tile_kernel(per-weight rounding)")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    outs = (out8, outp, outw, outm)
+    for rep in range(3):
+        a8.copy_(torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=torch.Generator().manual_seed(100 + rep)).to(DEV))
+        xb.copy_(workloads.activations(M, K, torch.bfloat16, seed=110 + rep).to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        for o in outs:
+            o.zero_()
+        step()                                   # eager, same buffers
+        torch.cuda.synchronize()
+        for g, o in zip(got, outs):
+            assert torch.equal(g, o), f"replay {rep}"
+            assert bool(o.float().abs().sum() > 0)
+
+
 # ------------------------------------------------------------------ strides through the C ABI
 def test_c_abi_row_strides(hip_lib):
     """The launchers keep the reference's contiguity asserts, the C ABI takes row strides: operands and
