@@ -963,6 +963,16 @@ def test_weight_only_bf16_rows_through_the_conversion_pass(hip_lib, bits, group)
     assert hip_lib.fnn_gemm_weight_only_workspace_bytes(64, N, K, group, 1, 0) == 0        # few rows: other kernels
     assert hip_lib.fnn_gemm_weight_only_workspace_bytes(M, N, K, group, 0, 0) == 0         # fp16 rows need no conversion
     assert hip_lib.fnn_gemm_weight_only_workspace_bytes(M, N, K, group, 1, 1) == 0         # bf16 tables: fp32 scaling
+    # scratch that is too small, or not 16-byte aligned, is not used: the call still succeeds, on the fp32-scaling kernel
+    fn_ws = hip_lib.fnn_gemm_a16w4_ws if bits == 4 else hip_lib.fnn_gemm_a16w8_ws
+    ws = torch.empty(need + 16, dtype=torch.uint8, device=DEV)
+    for ptr, size, kernel in ((ws.data_ptr(), need - 1, "gemm_wo_tile_kernel<"), (ws.data_ptr() + 8, need, "gemm_wo_tile_kernel<"),
+                              (ws.data_ptr(), need, "gemm_wo_tile_kernel(per-weight rounding)")):
+        again = torch.zeros_like(out)
+        rc = fn_ws(again.data_ptr(), a_d.data_ptr(), q_d.data_ptr(), s_d.data_ptr(), b_d.data_ptr(), z_d.data_ptr(), M, N, K, K, K, N,
+                   group, 1, 1, 0, 0, _lib.dtype_code(b_d.dtype), ptr, size, _lib.current_stream(a_d.device))
+        assert rc == 0 and _lib.last_kernel().startswith(kernel), (size, _lib.last_kernel())
+        assert torch.equal(again, plain if "rounding" not in kernel else out)
 
 
 def test_weight_only_tiled_one_hot():
@@ -1341,7 +1351,6 @@ def test_split_k_packed_decode_and_moe_under_graph_capture():
         launchers.hip_gemm_a16w4_forward(outw, xb, packed, scale, zero_points=zp)
         flashnn_amd.fused_moe_a8w8_forward(a8[:, :1024], be, outm, sr, ace, tw, ids, sid, eid, used, True, top_k, BM)
 
-    kernels = []
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
