@@ -18,6 +18,7 @@ struct A8W8Args {
     int64_t lda, ldb, ldc;
     int out_dtype, arow_dtype, acol_dtype;
     int tiles_m, tiles_n, tiles_per_xcd;
+    int gn;                 // tile columns per group of the tile numbering
     // K cut into kparts ranges of k_chunk bytes per row (the tiled kernel's split form only)
     int kparts, k_chunk;
     int* ws_count;          // one ticket counter per tile, zero between calls

@@ -135,9 +135,10 @@ __global__ __launch_bounds__(WGM * 128) void gemm_a8w8_ring_kernel(const A8W8Arg
     // (the last part takes what the others leave: a few slabs more, so that it arrives last as a rule)
     const int Kl = SPLIT ? (kpart == p.kparts - 1 ? p.K - kpart * p.k_chunk : p.k_chunk) : p.K;
     // tiles are numbered in groups of GN tile columns, the column fastest within a group: the 32 workgroups
-    // an XCD runs at a time then cover 8 tile rows x 4 tile columns whatever M is, and fetch
-    // 8*BM + 4*BN operand rows per slab into its L2 instead of tiles_m*BM + BN
-    constexpr int GN = 4;
+    // an XCD runs at a time then cover 32 / GN tile rows x GN tile columns whatever M is, and fetch
+    // (32 / GN) * BM + GN * BN operand rows per slab into its L2 instead of tiles_m*BM + BN.  GN = 8 for the tiles
+    // of 192 and 256 columns, 4 for the narrower ones (measured, see the launchers).
+    const int GN = p.gn;
     const int grp = t / (GN * p.tiles_m);
     const int rem = t - grp * (GN * p.tiles_m);
     const int gw = min(GN, p.tiles_n - grp * GN);
@@ -849,12 +850,19 @@ static A8W8Args rows_from(const A8W8Args& p, int64_t m0, int m, int mode) {
     return q;
 }
 
+// Tile columns per group of the tile numbering (the kernel's GN).  Both libraries on one box, bf16 out, us,
+// groups of 4 / 8 / 16 columns: QKV (256x192 tiles) 83.7 / 81.6 / 85.1, gate_up (256x256) 157.2 / 153.2 / 157.5,
+// 8192^3 (256x256) 370.4 / 368.9 / 384.8; with 256x128 tiles: down (K = 11008) 78.6 / 80.9 / 84.6, O 32.3 / 32.0 /
+// 31.9, M = 1024 N = 8192 33.1 / 32.9 / 33.9; 128x128: M = 512 K = N = 8192 40.8 / 40.9 / 42.0.
+static int group_columns(int bn) { return bn >= 192 ? 8 : 4; }
+
 template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2>
 static void launch_mfma(A8W8Args& p, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
+    p.gn = group_columns(BN);
     note_kernel("gemm_a8w8_ring_kernel", BM, BN, WGM * 2);
     gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, WGM><<<dim3(p.tiles_per_xcd * 8), dim3(WGM * 128), 0, st>>>(p, MoeArgs{});
 }
@@ -866,6 +874,7 @@ static void launch_mfma_split(A8W8Args& p, hipStream_t st) {
     p.tiles_n = (p.N + BN - 1) / BN;
     const int units = p.tiles_m * p.tiles_n * p.kparts;
     p.tiles_per_xcd = (units + 7) / 8;
+    p.gn = group_columns(BN);
     note_kernel("gemm_a8w8_ring_kernel(split K)", BM, BN, p.kparts);
     gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, 2, true><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p, MoeArgs{});
 }
@@ -1042,6 +1051,7 @@ static void launch_mfma_moe(A8W8Args& p, const MoeArgs& q, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     p.tiles_per_xcd = (p.tiles_m * p.tiles_n + 7) / 8;
+    p.gn = 4;
     note_kernel("gemm_a8w8_ring_kernel(moe)", BM, BN, 4);
     gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, 2, false, true><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p, q);
 }
