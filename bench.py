@@ -191,10 +191,21 @@ def main():
             torch.cuda.synchronize()
             ms_step, wall_ms = _timed(step, args.steps, torch, preroll_s=0.06)
             preroll_steps = _timed.preroll_calls
-            ms_gemm, _ = _timed(gemm_only, args.steps, torch)
+            # the GEMM kernel's duration inside the step: the same steps once more (straight after the timed
+            # ones, clocks as they were), with an event on either side of every GEMM launch.  The first event
+            # completes when the quantisation kernel has, so the launch gap between the two kernels is inside.
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+            for i in range(args.steps):
+                quant_only(i)
+                evs[i][0].record()
+                gemm_only(i)
+                evs[i][1].record()
+            torch.cuda.synchronize()
+            ms_gemm = sum(a.elapsed_time(b) for a, b in evs) / args.steps
+            ms_gemm_alone, _ = _timed(gemm_only, args.steps, torch)      # ... and launched back to back on its own
             ms_quant, _ = _timed(quant_only, args.steps, torch)
             primary = dict(M=M, K=K, N=N, ops=ops, ms_step=ms_step, wall_ms=wall_ms, ms_gemm=ms_gemm, nset=n,
-                           preroll_steps=preroll_steps,
+                           ms_gemm_alone=ms_gemm_alone, preroll_steps=preroll_steps,
                            k_gemm=k_gemm, k_quant=k_quant)
             if "rows" in legs:
                 secondary.append(_entry(f"dynamic_quant fp16 M={M} K={K}", ms_quant, "hbm", 3.0 * M * K + 2.0 * M,
@@ -209,7 +220,9 @@ def main():
     gemm_tops = primary["ops"] / (primary["ms_gemm"] * 1e-3) / 1e12
     roofline = {"kernel": primary["k_gemm"], "bound": "mfma", "achieved": round(gemm_tops, 2),
                 "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
-                "us_per_launch": round(primary["ms_gemm"] * 1e3, 2), "traffic": _traffic("a8w8 qkv")}
+                "us_per_launch": round(primary["ms_gemm"] * 1e3, 2), "traffic": _traffic("a8w8 qkv"),
+                "timed": "events around every GEMM launch of the step loop (launch gap behind the quantisation included)",
+                "us_per_launch_back_to_back": round(primary["ms_gemm_alone"] * 1e3, 2)}
     # what this device sustains on int8 MFMAs alone (operands in registers, about 0.1 s each): the
     # clock follows the power drawn, so random operand bytes run well below the datasheet rate
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
