@@ -854,7 +854,9 @@ static A8W8Args rows_from(const A8W8Args& p, int64_t m0, int m, int mode) {
 // groups of 4 / 8 / 16 columns: QKV (256x192 tiles) 83.7 / 81.6 / 85.1, gate_up (256x256) 157.2 / 153.2 / 157.5,
 // 8192^3 (256x256) 370.4 / 368.9 / 384.8; with 256x128 tiles: down (K = 11008) 78.6 / 80.9 / 84.6, O 32.3 / 32.0 /
 // 31.9, M = 1024 N = 8192 33.1 / 32.9 / 33.9; 128x128: M = 512 K = N = 8192 40.8 / 40.9 / 42.0.
-static int group_columns(int bn) { return bn >= 192 ? 8 : 4; }
+// Over a long K the wider groups lose again (M = 8192 N = 17792 K = 13312: 1349 / 1442; M = 2048 N = 35584 K = 13312:
+// 732 / 741; K = 7392 .. 8896: within 1 %), so they are taken up to K = 8192.
+static int group_columns(int bn, int k) { return bn >= 192 && k <= 8192 ? 8 : 4; }
 
 template <int BM, int BN, int MODE, bool PAIR = false, int WGM = 2>
 static void launch_mfma(A8W8Args& p, hipStream_t st) {
@@ -862,7 +864,7 @@ static void launch_mfma(A8W8Args& p, hipStream_t st) {
     p.tiles_n = (p.N + BN - 1) / BN;
     const int tiles = p.tiles_m * p.tiles_n;
     p.tiles_per_xcd = (tiles + 7) / 8;
-    p.gn = group_columns(BN);
+    p.gn = group_columns(BN, p.K);
     note_kernel("gemm_a8w8_ring_kernel", BM, BN, WGM * 2);
     gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, WGM><<<dim3(p.tiles_per_xcd * 8), dim3(WGM * 128), 0, st>>>(p, MoeArgs{});
 }
@@ -874,7 +876,7 @@ static void launch_mfma_split(A8W8Args& p, hipStream_t st) {
     p.tiles_n = (p.N + BN - 1) / BN;
     const int units = p.tiles_m * p.tiles_n * p.kparts;
     p.tiles_per_xcd = (units + 7) / 8;
-    p.gn = group_columns(BN);
+    p.gn = group_columns(BN, p.K);
     note_kernel("gemm_a8w8_ring_kernel(split K)", BM, BN, p.kparts);
     gemm_a8w8_ring_kernel<BM, BN, MODE, PAIR, 2, true><<<dim3(p.tiles_per_xcd * 8), dim3(256), 0, st>>>(p, MoeArgs{});
 }
