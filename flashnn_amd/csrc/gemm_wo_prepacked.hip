@@ -239,6 +239,246 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemv_w4_prepacked_kernel(const 
     }
 }
 
+// ---- 2 .. 64 activation rows per pass on the packed form ---------------------------------------------------
+// A workgroup of NW waves (8, or 4 for 64 rows) owns up to T neighbouring tiles and walks K in ranges of
+// 128 NW values; in a range wave w takes the group of 128 values that is the kilobyte at 1024 (w + NW sub) of
+// every tile's unit, so the waves read a unit's nibbles as one contiguous piece, and what a wave needs of the
+// activations for a range - its 128 values of up to 64 rows, already in operand order - serves all tiles of
+// the workgroup.  Those rows arrive by 16-byte direct-to-LDS copies, whole 128-byte lines per instruction, into
+// a wave-private area one range ahead (fragment (mb, i) of lane (c, g): row 16 mb + c, values 32 i + 8 g .. + 7
+// of the group); the weights and table entries of (tile, range + PD) are requested as those of
+// (tile, range) are consumed, and the main loop has no barrier.  The integer weights go into the MFMAs as
+// OFF + u (exponent trick, OFF = 1024 for fp16 and 128 for bf16 activations, u the nibble as an unsigned
+// number); per group
+//   out += s * (dot - (OFF + 8 + zp) * sum_k a_k),
+// in fp32, the activation sums coming from MFMAs against ones once per range and wave.  The partial sums of
+// the waves meet in LDS and are added in ascending wave order, then bias, rounding, store.
+// 64 rows take four waves: 7 x 4 x 4 output registers per lane, the fragments of 64 rows and two ranges of
+// weights in flight need more than the 256 registers a wave of an 8-wave workgroup can have.
+constexpr int kPkRowTiles = 7;       // most tiles per workgroup
+
+typedef __attribute__((address_space(3))) void* pk_lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* pk_gbl_ptr_t;
+
+// A word of eight nibbles -> the eight numbers OFF + u of one MFMA operand: the nibble pair (j, j + 4) of the
+// word, shifted to bits 0..3 and 16..19, set into the exponent pattern.  `k` holds that pattern in a register
+// the compiler cannot see through, so that (w & m) | (k & ~m) is one bit-field insert (an and-or of a
+// register with two constants takes two instructions on this ISA).
+__device__ __forceinline__ v4u pk_operand(const uint32_t w, const uint32_t k) {
+    constexpr uint32_t m = 0x000F000Fu;
+    const uint32_t w1 = w >> 4, w2 = w >> 8, w3 = w >> 12;
+    return v4u{(w & m) | (k & ~m), (w1 & m) | (k & ~m), (w2 & m) | (k & ~m), (w3 & m) | (k & ~m)};
+}
+
+constexpr int pk_rows_lds_bytes(int MB, int NW, int T) { return NW * MB * (T > 4 ? T : 4) * 1024; }
+
+template <int ADT, int MB, int NW, int T, int PD, bool NT>
+__global__ __launch_bounds__(NW * 64) void gemm_w4_prepacked_rows_kernel(const PkArgs p) {
+    typedef MfmaT<ADT> MT;
+    constexpr int SUB = 8 / NW;                 // ranges per unit
+    constexpr int FR = 4 * MB;                  // activation fragments per range and wave
+    constexpr int WAVE_LDS = FR * 1024;
+    constexpr int LPS = 2 * T;                  // register loads per range and wave
+    constexpr float OFF8 = (ADT == FNN_F16 ? 1024.f : 128.f) + 8.f;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int KC = p.K >> 10;
+    const int NR = KC * SUB;                    // ranges
+    const int tile0 = blockIdx.x * p.tpw;
+    const int ntile = min(p.tpw, p.tiles - tile0);
+    const int m0 = blockIdx.y * (MB * 16);
+
+    // ---- activations: rows beyond M repeat the last row (their results are not stored)
+    char* const mine = smem + wave * WAVE_LDS;
+    const char* const abase = (const char*)p.act + (int64_t)m0 * p.lda * 2 + wave * 256;
+    // Copy j of a range brings rows 4 j .. 4 j + 3, each row's 256 bytes of the wave's group as two whole
+    // 128-byte lines: lane 16 q + ch asks for 16-byte chunk ch ^ (row & 15) of row 4 j + q, which lands in slot
+    // ch of that row (the area is [row][slot], 256 bytes a row), so that the 16 lanes which later read the same
+    // chunk of 16 different rows find it in 16 different slots.
+    uint32_t aoff[FR];
+#pragma unroll
+    for (int j = 0; j < FR; ++j) {
+        const int row = 4 * j + (lane >> 4);
+        aoff[j] = (uint32_t)min(row, p.M - 1 - m0) * (uint32_t)(p.lda * 2) + (((lane & 15) ^ (row & 15)) << 4);
+    }
+    auto copy_act = [&](int r) __attribute__((always_inline)) {
+        const char* const src = abase + (int64_t)r * (NW * 256);
+#pragma unroll
+        for (int j = 0; j < FR; ++j)
+            __builtin_amdgcn_global_load_lds((pk_gbl_ptr_t)(src + aoff[j]), (pk_lds_ptr_t)(mine + j * 1024), 16, 0, 0);
+    };
+
+    // ---- weights and tables: tile t of the workgroup, range r.  A tile the workgroup does not have, and a
+    // range behind the last one, are replaced by 16 bytes (4 for the tables) of a unit that exists, the same
+    // for all lanes: every wave then has the same loads in flight at every point of the loop.  One table load
+    // serves both tables: the lanes of even g ask for the scale of channel c, those of odd g for its zero point
+    // (the aligned 32-bit word that holds the 16-bit entry; the half is taken where it is used).
+    const char* const units = p.packed + (int64_t)tile0 * KC * kPkUnitBytes;
+    const uint32_t w_lane = wave * 1024 + lane * 16, t_lane = 8192 + 256 * (g & 1) + 2 * (8 * c + (wave & ~1));
+    const uint32_t t_shift = 16 * (wave & 1);
+    v4u wq[PD][T];
+    uint32_t tq[PD][T];
+    auto unit_of = [&](int t, int r) -> const char* {
+        const int rr = r < NR ? r : NR - 1;
+        return units + ((int64_t)(t < ntile ? t : 0) * KC + rr / SUB) * kPkUnitBytes + (rr % SUB) * (NW * 1024);
+    };
+    auto load_w = [&](auto slot, int t, int r) __attribute__((always_inline)) {
+        const v4u* const wp = (const v4u*)(unit_of(t, r) + (t < ntile && r < NR ? w_lane : 0u));
+        wq[decltype(slot)::value][t] = NT ? __builtin_nontemporal_load(wp) : *wp;
+    };
+    auto load_t = [&](auto slot, int t, int r) __attribute__((always_inline)) {
+        const bool have = t < ntile && r < NR;
+        const int sub = (r < NR ? r : NR - 1) % SUB;
+        // (the tables lie behind the unit's eight kilobytes of nibbles, not behind this range's)
+        tq[decltype(slot)::value][t] =
+            *(const uint32_t*)(unit_of(t, r) - sub * (NW * 1024) + (have ? t_lane + sub * NW * 2 : 8192u));
+    };
+    // Every wait for a load is written out.  (As long as direct-to-LDS copies are in flight the compiler
+    // answers a register whose load it cannot place behind one of these waits with a wait for everything.)
+    // A tile's weights and, one load later, the table entries of the tile before it were asked for PD ranges
+    // ago; behind them came the rest of that range's loads, PD - 1 whole ranges, PD sets of copies and this
+    // range's loads so far: 2 PD T - 2 + PD FR loads in all, whatever the tile.
+    constexpr int NTILE_WAIT = (PD * T - 1) * 2 + PD * FR;
+    static_assert(NTILE_WAIT < 64 && LPS < 64, "vmcnt range");
+    auto wait_tile = [&]() __attribute__((always_inline)) {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (NTILE_WAIT & 15) | ((NTILE_WAIT >> 4) << 14));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);       // nothing that reads the loaded registers moves above the wait
+    };
+
+    v4f out[T][MB];
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) out[t][mb] = v4f{0.f, 0.f, 0.f, 0.f};
+    const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+    uint32_t kexp = ADT == FNN_F16 ? 0x64006400u : 0x43004300u;       // OFF in both halves
+    asm volatile("" : "+v"(kexp));
+
+    // issue order: the older ranges' weights, the first range's activations, the newest range's weights
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<PD - 1>([&](auto d) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) { load_w(d, t, decltype(d)::value); load_t(d, t, decltype(d)::value); }
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    copy_act(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        load_w(std::integral_constant<int, PD - 1>{}, t, PD - 1);
+        load_t(std::integral_constant<int, PD - 1>{}, t, PD - 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    auto range = [&](int r, auto slot, auto tail) __attribute__((always_inline)) {
+        constexpr int S = decltype(slot)::value;
+        constexpr bool TAIL = decltype(tail)::value;
+        // the copies of this range were issued before the LPS loads that followed them: they have landed
+        // once at most LPS loads are outstanding.  The ranges behind the loop ask for nothing further (the
+        // compiler would drop loads nobody uses, and the count with them) and wait for everything instead.
+        constexpr int TOP_WAIT = TAIL ? 0 : LPS;
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (TOP_WAIT & 15) | ((TOP_WAIT >> 4) << 14));
+        asm volatile("" ::: "memory");
+        v4u a[MB][4];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[mb][i] = *(const v4u*)(mine + (16 * mb + c) * 256 + (((4 * i + g) ^ c) << 4));
+        // the reads are back before the next range's copies may overwrite the area
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        copy_act(r + 1 < NR ? r + 1 : r);          // (behind the last range: once more the same, unused)
+        __builtin_amdgcn_sched_barrier(0);
+
+        v4f asum[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) asum[mb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) asum[mb] = MT::mma(a[mb][i], ones, asum[mb]);
+
+        // A tile in two halves, the second one tile behind the first, in one stretch of code, so that the
+        // compiler can place the vector instructions of a fold between the MFMAs of the next tile (a wave
+        // issues in order: what shall run under an MFMA has to stand behind it): (A) convert the tile's nibbles
+        // and issue its MFMAs into one of two accumulator sets; (B) scale and zero point of the tile before,
+        // fold.  Then the loads, in a fixed order: this tile's weights and the previous tile's table entries
+        // PD ranges on.  One wait at the top covers the weights and, one load younger, the table entries.
+        // (A tile the workgroup does not have is worked on all the same, on the bytes its loads fetched:
+        // straight code, and nothing of it is stored.)
+        v4f d[2][MB];
+        static_for<T + 1>([&](auto tt) __attribute__((always_inline)) {
+            constexpr int t = decltype(tt)::value;
+            constexpr int tp = t > 0 ? t - 1 : 0;     // the tile whose fold runs here
+            wait_tile();
+            if constexpr (t < T) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) d[t & 1][mb] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const v4u x = pk_operand(wq[S][t < T ? t : 0][i], kexp);
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) d[t & 1][mb] = MT::mma(a[mb][i], x, d[t & 1][mb]);
+                }
+            }
+            if constexpr (t > 0) {
+                const v2u sz = __builtin_amdgcn_permlane16_swap(tq[S][tp], tq[S][tp], false, false);
+                const float s32 = f16_bits_to_f32(sz[0] >> t_shift);
+                const float cz = OFF8 + f16_bits_to_f32(sz[1] >> t_shift);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        out[tp][mb][q] = __builtin_fmaf(s32, __builtin_fmaf(-cz, asum[mb][q], d[tp & 1][mb][q]), out[tp][mb][q]);
+            }
+            // (arithmetic may move across these; loads stay in their order)
+            __builtin_amdgcn_sched_barrier(0xF);
+            if constexpr (!TAIL && t < T) load_w(slot, t < T ? t : 0, r + PD);
+            __builtin_amdgcn_sched_barrier(0xF);
+            if constexpr (!TAIL && t > 0) load_t(slot, tp, r + PD);
+            __builtin_amdgcn_sched_barrier(0xF);
+        });
+    };
+    // whole rounds of PD ranges, then the ranges left over (the same code with the slots named at compile time)
+    int r = 0;
+    for (; r + PD <= NR; r += PD)
+        static_for<PD>([&](auto d) __attribute__((always_inline)) { range(r + decltype(d)::value, d, std::false_type{}); });
+    static_for<PD - 1>([&](auto d) __attribute__((always_inline)) {
+        if (r + decltype(d)::value < NR) range(r + decltype(d)::value, d, std::true_type{});
+    });
+
+    // ---- the waves' parts, [wave][tile][mb][lane] as float4, added in wave order
+    __syncthreads();
+    v4f* const parts = (v4f*)smem;
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) parts[((wave * T + t) * MB + mb) * 64 + lane] = out[t][mb];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < ntile * MB * 64; idx += NW * 64) {
+        const int t = idx / (MB * 64), rem = idx - t * (MB * 64);
+        const int mb = rem >> 6, ln = rem & 63;
+        v4f v = parts[(t * MB + mb) * 64 + ln];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) v += parts[((w * T + t) * MB + mb) * 64 + ln];
+        const int n = (tile0 + t) * 16 + (ln & 15);
+        const float bias = p.bias ? load_as_f32(p.bias, n, p.bias_dtype) : 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int m = m0 + 16 * mb + 4 * (ln >> 4) + q;
+            if (m < p.M) store_from_f32(p.out, (int64_t)m * p.ldc + n, v[q] + bias, p.out_dtype);
+        }
+    }
+}
+
 // ---- the repacking: one thread per 32-bit word of the packed form
 __global__ __launch_bounds__(256) void prepack_w4_kernel(uint32_t* dst, const uint8_t* qw, const uint16_t* scale,
                                                          const uint16_t* zp, int N, int K, int64_t ldw, int64_t words) {
@@ -291,6 +531,38 @@ static void launch_pk(PkArgs& p, hipStream_t st) {
     kfn<<<dim3((p.tiles + p.tpw - 1) / p.tpw), dim3(kPkWaves * 64), lds, st>>>(p);
 }
 
+template <int ADT, int MB, int NW, int T, int PD, bool NT>
+static void launch_pk_rows_t(const PkArgs& p, int passes, hipStream_t st) {
+    auto kfn = gemm_w4_prepacked_rows_kernel<ADT, MB, NW, T, PD, NT>;
+    static std::atomic<uint64_t> raised{0};
+    allow_large_lds((const void*)kfn, raised);
+    note_kernel("gemm_w4_prepacked_rows_kernel", MB, T, passes);
+    kfn<<<dim3((p.tiles + p.tpw - 1) / p.tpw, passes), dim3(NW * 64), (size_t)pk_rows_lds_bytes(MB, NW, T), st>>>(p);
+}
+
+// 2 or more rows: passes of 16, 32 or 64 rows; a single pass reads the weights with non-temporal loads.
+// As many tiles per workgroup as give every CU one workgroup, at most kPkRowTiles; the kernel is built for 1, 2, 4
+// or 7 and keeps the more ranges in flight the fewer tiles a range has.  Up to 32 rows: 8 waves; more: 4 waves
+// (about 300 registers per lane).
+template <int ADT>
+static void launch_pk_rows(PkArgs& p, hipStream_t st) {
+    const int tpw = (p.tiles + 255) / 256;
+    p.tpw = tpw > kPkRowTiles ? kPkRowTiles : tpw;
+    const int passes = (p.M + 63) / 64;
+#define FNN_PK_ROWS(T, PD1, PD2, PD4)                                                \
+    do {                                                                            \
+        if (p.M <= 16) launch_pk_rows_t<ADT, 1, 8, T, PD1, true>(p, 1, st);          \
+        else if (p.M <= 32) launch_pk_rows_t<ADT, 2, 8, T, PD2, true>(p, 1, st);     \
+        else if (passes == 1) launch_pk_rows_t<ADT, 4, 4, T, PD4, true>(p, 1, st);   \
+        else launch_pk_rows_t<ADT, 4, 4, T, PD4, false>(p, passes, st);              \
+    } while (0)
+    if (p.tpw == 1) FNN_PK_ROWS(1, 8, 4, 3);
+    else if (p.tpw == 2) FNN_PK_ROWS(2, 6, 3, 3);
+    else if (p.tpw <= 4) FNN_PK_ROWS(4, 4, 2, 2);
+    else FNN_PK_ROWS(7, 2, 2, 2);
+#undef FNN_PK_ROWS
+}
+
 }  // namespace fnn
 
 using namespace fnn;
@@ -341,8 +613,8 @@ extern "C" int fnn_gemm_a16w4_prepacked(void* out, const void* act, const void* 
         set_error("%s: no packed form for N=%lld K=%lld group=%lld", fn, (long long)N, (long long)K, (long long)group);
         return FNN_ERR_UNSUPPORTED;
     }
-    if (M > 1) {
-        set_error("%s: the packed form serves the decode of one token (M=%lld); use fnn_gemm_a16w4", fn, (long long)M);
+    if (M > 1 && (64 * lda * 2 >= (1LL << 32) || (M + 63) / 64 > 65535)) {
+        set_error("%s: M=%lld rows of stride %lld are beyond what the kernel addresses", fn, (long long)M, (long long)lda);
         return FNN_ERR_UNSUPPORTED;
     }
     if (!is16(act_dtype) || !is16(out_dtype) || (bias && !isflt(bias_dtype))) {
@@ -364,7 +636,13 @@ extern "C" int fnn_gemm_a16w4_prepacked(void* out, const void* act, const void* 
     p.tpw = tpw;
     const Call call(fn);
     const hipStream_t st = (hipStream_t)stream;
-    if (act_dtype == FNN_F16) launch_pk<FNN_F16>(p, st);
-    else launch_pk<FNN_BF16>(p, st);
+    if (M > 1) {
+        if (act_dtype == FNN_F16) launch_pk_rows<FNN_F16>(p, st);
+        else launch_pk_rows<FNN_BF16>(p, st);
+    } else if (act_dtype == FNN_F16) {
+        launch_pk<FNN_F16>(p, st);
+    } else {
+        launch_pk<FNN_BF16>(p, st);
+    }
     return call.done();
 }

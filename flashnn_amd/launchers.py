@@ -313,8 +313,8 @@ class PrepackedInt4:
 
 def hip_a16w4_prepack(quant_w, scale_w, zero_points=None):
     """Repack int4 weights in the reference layout (quant_w [N/2, K] int8 as GemmWeightOnly takes them,
-    flashnn/quant_gemm.py:174-204; scale_w and zero_points [K/128, N] fp16) into one stream for the decode
-    of one token.  Returns a PrepackedInt4; the originals are not modified and can be freed.  No
+    flashnn/quant_gemm.py:174-204; scale_w and zero_points [K/128, N] fp16) into one stream, made for the
+    decode of one or a few tokens.  Returns a PrepackedInt4; the originals are not modified and can be freed.  No
     counterpart in the reference, whose launcher reads the layout above as it is (gemm_a16w4.py:336-406)."""
     assert quant_w.dtype == torch.int8 and quant_w.dim() == 2 and quant_w.stride(1) == 1, "Weight must be int8 type"
     assert scale_w.dim() == 2 and scale_w.dtype == torch.float16 and scale_w.is_contiguous(), \
@@ -338,8 +338,9 @@ def hip_a16w4_prepack(quant_w, scale_w, zero_points=None):
 
 
 def hip_gemm_a16w4_prepacked_forward(out, act, packed, bias=None):
-    """triton_gemm_a16w4_forward (flashnn/triton_kernels/gemm_a16w4.py:336-406) for one activation row on
-    weights packed by hip_a16w4_prepack."""
+    """triton_gemm_a16w4_forward (flashnn/triton_kernels/gemm_a16w4.py:336-406) on weights packed by
+    hip_a16w4_prepack: any number of activation rows (one row and up to 64 rows are what the packed form
+    is fast for)."""
     assert isinstance(packed, PrepackedInt4)
     assert act.is_contiguous(), "Activation must be contiguous"
     assert act.dim() == 2 and act.shape[1] == packed.k, "Matrix B must be transposed"

@@ -168,7 +168,7 @@ int fnn_gemm_a16w4_ws(void* out, const void* act, const void* qw, const void* sc
                       void* workspace, size_t ws_bytes, void* stream);
 
 /*
- * fnn_gemm_a16w4 for the decode of one token (M = 1) on weights repacked once by the caller.  The
+ * fnn_gemm_a16w4 on weights repacked once by the caller (made for the decode of one or a few tokens).  The
  * reference keeps int4 weights as [N/2, K] bytes with [K/group, N] tables beside them
  * (flashnn/quant_gemm.py:174-204; its Triton launcher, flashnn/triton_kernels/gemm_a16w4.py:336-406, reads
  * that layout as it is); a decode kernel then fetches rows K bytes apart plus two side tables.  The packed
@@ -184,9 +184,14 @@ int fnn_gemm_a16w4_ws(void* out, const void* act, const void* qw, const void* sc
  *   fnn_a16w4_prepack(packed, qw, scale, zp, ...)   packed <- the reference layout (qw [N/2, K] with row stride
  *                                           ldw, scale and zp [K/128, N] fp16, zp may be NULL = zeros);
  *                                           a device-side copy, asynchronous on `stream`
- *   fnn_gemm_a16w4_prepacked(out, act, packed, bias, ...)   out[0, n] as fnn_gemm_a16w4 computes it, within
+ *   fnn_gemm_a16w4_prepacked(out, act, packed, bias, ...)   out[m, n] as fnn_gemm_a16w4 computes it, within
  *                                           rtol = atol = 1e-2 of the reference (group scales are applied in
- *                                           fp32 to group sums); M > 1 is FNN_ERR_UNSUPPORTED
+ *                                           fp32 to group sums).  M = 1: a kernel that streams the packed
+ *                                           form at the rate of a bare load stream; M > 1: a kernel for 16,
+ *                                           32 or 64 rows per pass over the weights (more rows: more passes;
+ *                                           from about 100 rows on the reference layout's tiled kernel is
+ *                                           faster on large matrices).  act rows lda elements apart (lda % 8
+ *                                           == 0 for M > 1, 64 rows within 4 GB), out rows ldc apart.
  * Nothing repacks implicitly: fnn_gemm_a16w4 always reads the reference layout.
  */
 size_t fnn_a16w4_prepacked_bytes(int64_t N, int64_t K, int64_t group);

@@ -1103,11 +1103,69 @@ def test_a16w4_prepacked_argument_errors(hip_lib):
     qw = torch.zeros(8, 1024, dtype=torch.int8, device=DEV)
     scale = torch.ones(8, 16, dtype=torch.float16, device=DEV)
     pk = flashnn_amd.GemmWeightOnly.prepack(qw, scale)
-    act = torch.zeros(2, 1024, dtype=torch.float16, device=DEV)
-    with pytest.raises(_lib.FlashnnHipError, match="one token"):
-        flashnn_amd.GemmWeightOnly(torch.float16).forward_prepacked(act, pk)
     with pytest.raises(AssertionError):
         flashnn_amd.GemmWeightOnly.prepack(qw, scale.bfloat16())
+    # rows whose stride is not a multiple of 16 bytes are refused before anything is launched
+    act = torch.zeros(2, 1028, dtype=torch.float16, device=DEV)
+    out = torch.full((2, 16), 3.0, dtype=torch.float16, device=DEV)
+    rc = hip_lib.fnn_gemm_a16w4_prepacked(_lib.ptr(out), _lib.ptr(act), _lib.ptr(pk.buffer), None, 2, 16, 1024, 1028, 16, 128,
+                                          _lib.FNN_F16, _lib.FNN_F16, 0, _lib.current_stream(out.device))
+    torch.cuda.synchronize()
+    assert rc != 0 and b"16-byte aligned" in hip_lib.fnn_last_error() and bool((out == 3.0).all())
+
+
+@pytest.mark.parametrize("M,N,K,act_ty,with_zp,with_bias", [
+    (2, 28672, 8192, torch.bfloat16, True, False),      # 7 tiles per workgroup, 16-row pass with 2 rows in use
+    (16, 28672, 8192, torch.float16, True, True),
+    (17, 14336, 8192, torch.bfloat16, True, False),     # 4 tiles per workgroup, 32-row pass
+    (32, 28672, 8192, torch.bfloat16, False, False),
+    (33, 4096, 4096, torch.float16, True, True),        # one tile per workgroup, 64-row pass, 4 waves
+    (64, 28672, 8192, torch.bfloat16, True, False),
+    (100, 8192, 2048, torch.bfloat16, True, True),      # two passes of 64 rows, 2 tiles per workgroup
+    (5, 8208, 16384, torch.float16, True, False),       # tiles that leave the last workgroup short, 16 ranges
+    (48, 1040, 9216, torch.bfloat16, True, True),       # an odd number of ranges (one left over behind the loop)
+    (3, 16, 1024, torch.float16, False, True),          # one tile, one range
+    (20, 48, 2048, torch.bfloat16, True, False),
+    (130, 27696, 11264, torch.float16, True, False),    # three passes; 1731 tiles: the last workgroup has 2 of 7
+])
+def test_a16w4_prepacked_rows(hip_lib, M, N, K, act_ty, with_zp, with_bias):
+    """More than one row on the packed weights: every tile count and row block the kernel is built for,
+    ranges left over behind its unrolled loop, short last workgroups, rows of very different magnitudes
+    (one of them all zero) - against the oracle on a band of channels and against the reference-layout
+    kernels everywhere."""
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    w = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(K // 128, N).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(-8, 8, (K // 128, N), generator=g).half() if with_zp else None
+    bias = torch.randn(N, generator=g).to(act_ty) if with_bias else None
+    act = torch.randn(M, K, generator=g)
+    act[:, ::7] *= 30.0
+    act[0] *= 100.0
+    act[M - 1] *= 1e-3
+    if M > 2:
+        act[1] = 0.0
+    act = act.to(act_ty)
+    qw = torch.from_numpy(O.pack_int4(w.numpy()))
+    op = flashnn_amd.GemmWeightOnly(act_ty)
+    pk = op.prepack(qw.to(DEV), scale.to(DEV), None if zp is None else zp.to(DEV))
+    out = op.forward_prepacked(act.to(DEV), pk, None if bias is None else bias.to(DEV))
+    assert _lib.last_kernel().startswith("gemm_w4_prepacked_rows_kernel") and out.shape == (M, N)
+    ncol = min(N, max(16, (1 << 24) // (M * K) // 16 * 16))
+    cols = slice(N - ncol, N)
+    want = O.weight_only_gemm(O.to_np(act), w[cols].numpy(), O.to_np(scale[:, cols]), None if zp is None else O.to_np(zp[:, cols]),
+                              None if bias is None else O.to_np(bias[cols]), O.F16, O.tag_of(act), 128, True)
+    got = out[:, cols].float().cpu().numpy()
+    # per row: the tolerance is relative to the row's own scale (rows differ by five orders of magnitude)
+    row_scale = np.maximum(1.0, np.abs(want).max(axis=1, keepdims=True) / 50)
+    assert np.all(np.abs(got - want) <= RTOL * np.abs(want) + ATOL * row_scale), float(np.abs(got - want).max())
+    full = op(act.to(DEV), qw.to(DEV), scale.to(DEV), None if bias is None else bias.to(DEV), None if zp is None else zp.to(DEV))
+    f = full.float().cpu().numpy()
+    o = out.float().cpu().numpy()
+    row_scale = np.maximum(1.0, np.abs(f).max(axis=1, keepdims=True) / 50)
+    assert np.all(np.abs(o - f) <= RTOL * np.abs(f) + ATOL * row_scale), float(np.abs(o - f).max())
+    if M > 2:
+        zero_row = out[1].float().cpu().numpy()
+        assert np.array_equal(zero_row, np.zeros(N, np.float32) if bias is None else bias.float().numpy())
 
 
 @pytest.mark.parametrize("bits,M,N,K", [(4, 1, 24576, 8192), (4, 2, 24576, 8192), (4, 3, 20480, 8192), (4, 4, 28672, 8192),

@@ -62,7 +62,7 @@ def test_argument_errors_are_reported_without_a_gpu(hip_lib):
     assert rc == -2 and b"row stride too large" in hip_lib.fnn_last_error()
     rc = hip_lib.fnn_gemm_a16w4(one, one, one, one, null, null, 4, 64, 1024, 1024, 1 << 31, 64, 0, 0, 0, 0, 0, 0, null)
     assert rc == -2 and b"row stride too large" in hip_lib.fnn_last_error()
-    # the packed int4 form: shapes without one, more than one row, and bad table types are refused
+    # the packed int4 form: shapes without one, rows the kernel cannot address, and bad table types are refused
     assert hip_lib.fnn_a16w4_prepacked_bytes(28672, 8192, 128) == 28672 * 8192 // 2 + 4 * 64 * 28672
     assert hip_lib.fnn_a16w4_prepacked_bytes(28672, 8192, 64) == 0 and hip_lib.fnn_a16w4_prepacked_bytes(24, 8192, 128) == 0
     assert hip_lib.fnn_a16w4_prepacked_bytes(4096, 3072, 128) == 0 and hip_lib.fnn_a16w4_prepacked_bytes(4096, 4000, 128) == 0
@@ -70,8 +70,10 @@ def test_argument_errors_are_reported_without_a_gpu(hip_lib):
     assert rc == -2 and b"fp16 scales" in hip_lib.fnn_last_error()
     rc = hip_lib.fnn_a16w4_prepack(one, one, one, null, 64, 1000, 1000, 128, 0, 0, null)
     assert rc == -2 and b"packed form needs" in hip_lib.fnn_last_error()
-    rc = hip_lib.fnn_gemm_a16w4_prepacked(one, one, one, null, 2, 64, 1024, 1024, 64, 128, 0, 0, 0, null)
-    assert rc == -2 and b"one token" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a16w4_prepacked(one, one, one, null, 2, 64, 1024, 1 << 31, 64, 128, 0, 0, 0, null)
+    assert rc == -2 and b"beyond what the kernel addresses" in hip_lib.fnn_last_error()
+    rc = hip_lib.fnn_gemm_a16w4_prepacked(one, one, one, null, 2, 64, 1024, 1028, 64, 128, 0, 0, 0, null)
+    assert rc == -1 and b"16-byte aligned" in hip_lib.fnn_last_error()
     assert hip_lib.fnn_gemm_a16w4_prepacked(null, null, null, null, 0, 64, 1024, 1024, 64, 128, 0, 0, 0, null) == 0
     # empty problems are a no-op
     assert hip_lib.fnn_gemm_a8w8_i32(one, one, one, 0, 4, 128, 128, 128, 4, null) == 0
