@@ -382,6 +382,16 @@ def main():
                packed_bytes=int(packs[0].buffer.numel()))
     secondary.append(e)
     decode["prepacked"] = e
+    if "c4" in legs:      # a few rows on the packed form (its kernel for 16, 32 or 64 rows per pass)
+        for m4 in (4, 16, 64):
+            act = workloads.activations(m4, K4, torch.bfloat16, seed=3).to(dev)
+            o4 = torch.empty(m4, N4, dtype=torch.bfloat16, device=dev)
+            f = lambda i: launchers.hip_gemm_a16w4_prepacked_forward(o4, act, packs[i % n])
+            kern = kernel_of(f)
+            ms, _ = _timed(f, iters, torch)
+            secondary.append(_entry(f"c4 a16w4 g128 M={m4} K={K4} N={N4} bf16, weights prepacked", ms, "hbm",
+                                    wbytes + 2.0 * m4 * K4 + 2.0 * m4 * N4, kern, f"a16w4 g128 M={m4} prepacked",
+                                    weight_GBps=round(wbytes / (ms * 1e-3) / 1e9, 1)))
     del pk, sc, zp, packs
     torch.cuda.empty_cache()
 

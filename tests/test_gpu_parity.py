@@ -1168,6 +1168,33 @@ def test_a16w4_prepacked_rows(hip_lib, M, N, K, act_ty, with_zp, with_bias):
         assert np.array_equal(zero_row, np.zeros(N, np.float32) if bias is None else bias.float().numpy())
 
 
+@pytest.mark.parametrize("act_ty", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M", [9, 24, 50, 70])
+@pytest.mark.parametrize("tiles_per_wg,K", [(1, 2048), (2, 1024), (4, 2048), (7, 4096)])
+def test_a16w4_prepacked_rows_every_build(hip_lib, tiles_per_wg, K, M, act_ty):
+    """Every build of the rows kernel on packed weights (1, 2, 4 or 7 tiles per workgroup x 16, 32 or 64 rows
+    per pass, one pass or two x fp16 or bf16 rows): the output against the oracle on the last 64 channels and
+    against the reference-layout kernels on all of them."""
+    N = 16 * 256 * tiles_per_wg
+    g = torch.Generator().manual_seed(N + K + M)
+    w = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(K // 128, N).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(-8, 8, (K // 128, N), generator=g).half()
+    act = torch.randn(M, K, generator=g).to(act_ty)
+    qw = torch.from_numpy(O.pack_int4(w.numpy()))
+    op = flashnn_amd.GemmWeightOnly(act_ty)
+    pk = op.prepack(qw.to(DEV), scale.to(DEV), zp.to(DEV))
+    out = op.forward_prepacked(act.to(DEV), pk)
+    kernel = _lib.last_kernel()
+    assert kernel == f"gemm_w4_prepacked_rows_kernel<{1 if M <= 16 else 2 if M <= 32 else 4},{tiles_per_wg},{(M + 63) // 64}>", kernel
+    cols = slice(N - 64, N)
+    want = O.weight_only_gemm(O.to_np(act), w[cols].numpy(), O.to_np(scale[:, cols]), O.to_np(zp[:, cols]), None,
+                              O.F16, O.tag_of(act), 128, True)
+    np.testing.assert_allclose(out[:, cols].float().cpu().numpy(), want, rtol=RTOL, atol=ATOL)
+    full = op(act.to(DEV), qw.to(DEV), scale.to(DEV), None, zp.to(DEV))
+    np.testing.assert_allclose(out.float().cpu().numpy(), full.float().cpu().numpy(), rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("bits,M,N,K", [(4, 1, 24576, 8192), (4, 2, 24576, 8192), (4, 3, 20480, 8192), (4, 4, 28672, 8192),
                                         (8, 1, 12288, 8192), (4, 2, 28672, 4096), (4, 1, 16384, 8192)])
 def test_weight_only_gemv_equal_chunks(bits, M, N, K):
