@@ -196,7 +196,7 @@ __global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoA
         const int wr = row0 + 4 * (l >> 4) + r;
         const int n = WBITS == 4 ? 2 * wr + h : wr;
         if (m < p.M && n < p.N) {
-            if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+            if (p.bias) v = add_bias<WBITS>(v, load_as_f32(p.bias, n, p.bias_dtype), p.out_dtype);
             store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
         }
     }
@@ -429,7 +429,7 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_kernel(const Wo
             v += red[((w * NH + h) * 4 + r) * 64 + lane1] + red[((w * NH + h) * 4 + r) * 64 + lane2];
         const int n = n0 + c;
         if (n < p.N) {
-            if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+            if (p.bias) v = add_bias<WBITS>(v, load_as_f32(p.bias, n, p.bias_dtype), p.out_dtype);
             store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
         }
     }
@@ -730,7 +730,7 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
             }
         const int n = n0 + c;
         if (n < p.N) {
-            if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+            if (p.bias) v = add_bias<WBITS>(v, load_as_f32(p.bias, n, p.bias_dtype), p.out_dtype);
             store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
         }
     }
@@ -985,7 +985,7 @@ __global__ __launch_bounds__(kGemvMaxWaves * 64) void gemm_wo_gemv_kernel(const 
         }
         const int n = n0 + c;
         if (tile_ok && n < p.N) {
-            if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+            if (p.bias) v = add_bias<WBITS>(v, load_as_f32(p.bias, n, p.bias_dtype), p.out_dtype);
             store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
         }
     }
@@ -1267,7 +1267,7 @@ __global__ __launch_bounds__(512) void gemm_wo_gemv_flat_kernel(const WoArgs p, 
             v += part[(h * 4 + r) * 64 + lane1] + part[(h * 4 + r) * 64 + lane2];
         }
         const int n = n0 + c;
-        if (p.bias) v += load_as_f32(p.bias, n, p.bias_dtype);
+        if (p.bias) v = add_bias<WBITS>(v, load_as_f32(p.bias, n, p.bias_dtype), p.out_dtype);
         store_from_f32(p.out, (int64_t)m * p.ldc + n, v, p.out_dtype);
     }
 }
@@ -1295,7 +1295,7 @@ __global__ __launch_bounds__(256) void gemm_wo_any_kernel(const WoArgs p) {
         }
         total += sc * part;
     }
-    if (p.bias) total += load_as_f32(p.bias, n, p.bias_dtype);
+    if (p.bias) total = add_bias<WBITS>(total, load_as_f32(p.bias, n, p.bias_dtype), p.out_dtype);
     store_from_f32(p.out, (int64_t)m * p.ldc + n, total, p.out_dtype);
 }
 
@@ -1542,8 +1542,18 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
     // whose waves share the activations through LDS; the other decode kernels for a single row and
     // for the shapes the panel kernel does not take.
     if (p.M <= 4 && (WBITS == 4 || p.M == 1) && launch_decode<WBITS, ADT>(p, st, true)) return;
-    // more than 64 rows: every weight dequantised once per 128 or 256 rows (the panel kernel takes 64 a pass)
-    if (p.M > 64 && launch_wo_tile(p, WBITS, ADT, st)) return;
+    // More than 64 rows: the tiled kernel dequantises every weight once per 128 or 256 rows (the panel kernel
+    // takes 64 a pass), but a tile is one workgroup walking all of K: with 128 tiles or fewer half the CUs
+    // or more stand idle while the others each need about 1.3 us per 128 values of K, and 64-row passes of the
+    // panel kernel finish sooner (fp16 rows, int4 g128, tiled / passes: M=128 N=4096 K=11008 102 / 31 us, M=256
+    // N=K=8192 83 / 58 us, M=512 N=K=4096 46 / 33 us; from 172 tiles on the tiled kernel wins: M=256 N=11008
+    // K=4096 45 / 57 us, M=128 N=28672 K=8192 90 / 109 us; int8 weights alike).
+    if (p.M > 64) {
+        const bool fills = wo_tile_count(p, WBITS) > 128;
+        if (fills && launch_wo_tile(p, WBITS, ADT, st)) return;
+        if (launch_wo_panel(p, WBITS, ADT, st)) return;
+        if (!fills && launch_wo_tile(p, WBITS, ADT, st)) return;
+    }
     if (p.M >= 2 && launch_wo_panel(p, WBITS, ADT, st)) return;
     if (launch_decode<WBITS, ADT>(p, st, false)) return;
     // up to 64 activation rows per pass over the weights

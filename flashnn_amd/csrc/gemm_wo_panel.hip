@@ -501,8 +501,14 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         uint32_t pk[NCL / 2];
 #pragma unroll
         for (int c = 0; c < NCL; c += 2) {
-            const float v0 = ((NH == 2 ? outv[mb][0][c >> 1] : outv[mb][0][c]) + bias[c]) * wroute;
-            const float v1 = ((NH == 2 ? outv[mb][1][c >> 1] : outv[mb][0][c + 1]) + bias[c + 1]) * wroute;
+            float v0 = NH == 2 ? outv[mb][0][c >> 1] : outv[mb][0][c];
+            float v1 = NH == 2 ? outv[mb][1][c >> 1] : outv[mb][0][c + 1];
+            if (p.bias) {
+                v0 = add_bias<WBITS>(v0, bias[c], p.out_dtype);
+                v1 = add_bias<WBITS>(v1, bias[c + 1], p.out_dtype);
+            }
+            v0 *= wroute;
+            v1 *= wroute;
             const uint32_t b0 = out_f16 ? f32_to_f16_bits(v0) : f32_to_bf16_bits(v0);
             const uint32_t b1 = out_f16 ? f32_to_f16_bits(v1) : f32_to_bf16_bits(v1);
             pk[c >> 1] = (b0 & 0xFFFFu) | (b1 << 16);

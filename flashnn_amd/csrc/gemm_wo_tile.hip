@@ -507,8 +507,12 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
 #pragma unroll
             for (int c = 0; c < 4 * NH; c += 2) {
                 // channel c of the lane: int4: register c >> 1 of operand 2 f + (c & 1); int8: register c of operand f
-                const float v0 = (NH == 2 ? outv[2 * f][b][c >> 1] : outv[f][b][c]) * un + bias[c];
-                const float v1 = (NH == 2 ? outv[2 * f + 1][b][c >> 1] : outv[f][b][c + 1]) * un + bias[c + 1];
+                float v0 = (NH == 2 ? outv[2 * f][b][c >> 1] : outv[f][b][c]) * un;
+                float v1 = (NH == 2 ? outv[2 * f + 1][b][c >> 1] : outv[f][b][c + 1]) * un;
+                if (p.bias) {
+                    v0 = add_bias<WBITS>(v0, bias[c], p.out_dtype);
+                    v1 = add_bias<WBITS>(v1, bias[c + 1], p.out_dtype);
+                }
                 const uint32_t b0 = out_f16 ? f32_to_f16_bits(v0) : f32_to_bf16_bits(v0);
                 const uint32_t b1 = out_f16 ? f32_to_f16_bits(v1) : f32_to_bf16_bits(v1);
                 pk[c >> 1] = (b0 & 0xFFFFu) | (b1 << 16);
@@ -523,6 +527,18 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
             }
         }
     }
+}
+
+// Rows per tile: 256 for int4 from 129 rows on - unless the 256-row tiles would leave half the CUs idle: then
+// twice as many workgroups of 128 rows, each with half the work, finish sooner.
+static int tile_rows(const WoArgs& p, int wbits) {
+    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * (p.N / 128);
+    return (p.M <= 128 || wbits == 8 || tiles256 <= 128) ? 128 : 256;
+}
+
+int wo_tile_count(const WoArgs& p, int wbits) {
+    const int bm = tile_rows(p, wbits);
+    return (int)((p.M + bm - 1) / bm) * (p.N / 128);
 }
 
 // Launches the tiled kernel if the shape suits it; returns false otherwise.
@@ -544,10 +560,7 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
         WoArgs q;
         if (convert_act_to_f16(p, q, st) && launch_tile_t<WBITS, FNN_F16>(q, st)) return true;
     }
-    // 256 rows per workgroup for int4 from 129 rows on - unless the 256-row tiles would leave half the CUs
-    // idle: then twice as many workgroups of 128 rows, each with half the work, finish sooner
-    const int64_t tiles256 = (int64_t)((p.M + 255) / 256) * (p.N / 128);
-    const int bm = (p.M <= 128 || WBITS == 8 || tiles256 <= 128) ? 128 : 256;
+    const int bm = tile_rows(p, WBITS);
     const int tiles_m = (p.M + bm - 1) / bm;
     const int tiles = tiles_m * (p.N / 128);
     const dim3 grid(((tiles + 7) / 8) * 8);   // (workgroups beyond the last tile return at once)

@@ -117,6 +117,19 @@ __device__ __forceinline__ v4u ref_dq_f16(v4u x, const v2h coff, const v2h zp, c
 }
 constexpr int FNN_I8 = 3;   // type code of int8 zero points (mixture-of-experts entry point only)
 
+// The bias as the reference adds it: its int8 branch casts the product to the output type and then adds the
+// bias in that type (flashnn/quant_gemm.py:168-173) - two roundings, which show where product and bias nearly
+// cancel; its int4 branch adds in fp32 and rounds once (:201-204).  The caller rounds the returned sum to
+// the output type.
+template <int WBITS>
+__device__ __forceinline__ float add_bias(float v, float bias, int out_dtype) {
+    if constexpr (WBITS == 8) {
+        if (out_dtype == FNN_F16) v = f16_bits_to_f32(f32_to_f16_bits(v));
+        else if (out_dtype == FNN_BF16) v = bf16_bits_to_f32(f32_to_bf16_bits(v));
+    }
+    return v + bias;
+}
+
 __device__ __forceinline__ float load_zp_f32(const void* p, int64_t i, int dtype) {
     return dtype == FNN_I8 ? (float)((const int8_t*)p)[i] : load_as_f32(p, i, dtype);
 }
@@ -164,6 +177,8 @@ size_t act_f16_ws_bytes(int64_t M, int64_t K);
 bool launch_wo_panel(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
 // gemm_wo_tile.hip: more than 64 activation rows, tiled MFMA kernel; false if the shape does not suit it
 bool launch_wo_tile(WoArgs& p, int wbits, int act_dtype, hipStream_t st);
+// ... and the number of tiles (workgroups) it would launch for this problem
+int wo_tile_count(const WoArgs& p, int wbits);
 // ... its mixture-of-experts form (int4, per-channel tables, blocks of 128 rows or more); false otherwise
 bool launch_wo_tile_moe(WoArgs& p, const MoeArgs& q, int act_dtype, hipStream_t st);
 // the int4 per-channel kernel over gathered rows of a mixture of experts; false if the shape does not suit it
