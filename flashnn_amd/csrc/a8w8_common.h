@@ -25,8 +25,9 @@ struct A8W8Args {
     int32_t* ws_part;       // kparts slots of tile-rows x tile-columns accumulators per tile
 };
 
-// gemm_a8w8_skinny.hip: up to 64 activation rows, the weights streamed once; false if the shape
-// does not suit it
+// gemm_a8w8_skinny.hip: up to 64 activation rows, the weights streamed once (its panel form also takes up to
+// kA8PanelRowsNarrow rows, in passes of 64); false if the shape does not suit it
+constexpr int kA8PanelRowsNarrow = 256;
 bool launch_a8w8_skinny(A8W8Args& p, int mode, hipStream_t st);
 // the same kernel over gathered rows (p.M is ignored); false if the shape does not suit it
 bool launch_a8w8_moe(A8W8Args& p, const MoeArgs& q, int mode, hipStream_t st);

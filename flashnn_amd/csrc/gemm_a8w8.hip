@@ -971,7 +971,13 @@ static void dispatch_band(A8W8Args& p, hipStream_t st, bool aligned, int force_b
     // the MFMA kernel walks K in slabs of 128 bytes
     const bool fast = aligned && p.K % 32 == 0 && p.K >= 512;
     // few activation rows: stream the weights once (unless the caller names a tile of the tiled kernel)
-    if (force_bm == 0 && p.M <= 64 && launch_a8w8_skinny(p, MODE, st)) return;
+    // ... and up to 256 rows over a narrow weight matrix with long rows, where the tiled kernel has a handful
+    // of tiles and splits K to fill the machine: 64-row passes of the few-row kernel stream the weights through
+    // all CUs instead (bf16 out, tiled / passes: M=128 N=2048 K=8192 19.8 / 11.6 us, M=256 23.3 / 17.5; M=128
+    // N=1920 K=13312 25.3 / 17.4; M=128 N=1024 K=4096 10.1 / 8.7; from N = 3584 on the tiled kernel wins:
+    // M=128 N=3584 K=18944 30.5 / 34.5, N=K=8192 23.3 / 24.7).  The same bits either way.
+    const bool narrow = p.M <= kA8PanelRowsNarrow && p.N <= 2048 && p.K >= 4096;
+    if (force_bm == 0 && (p.M <= 64 || narrow) && launch_a8w8_skinny(p, MODE, st)) return;
     if (fast && ws.ptr) {
         if (ws.force_kparts > 1) {          // (the entry point has checked tile, parts and workspace size)
             const int chunk = split_chunk_slabs((p.K + 127) / 128, ws.force_kparts) * 128;
@@ -1189,6 +1195,8 @@ extern "C" int fnn_gemm_a8w8_tiled(void* out, const void* a, const void* b, cons
 
 extern "C" size_t fnn_gemm_a8w8_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 64 || N <= 0 || K < 512 || K % 32 != 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return 0;
+    // (a narrow weight matrix under up to 256 rows goes to the few-row kernel in passes: see dispatch_band)
+    if (M <= kA8PanelRowsNarrow && N <= 2048 && K >= 4096 && N % 16 == 0) return 0;
     const SplitPlan s = plan_split(M, N, K, 0);
     return s.kparts > 1 ? split_ws_bytes(s, M, N) : 0;
 }

@@ -388,7 +388,7 @@ __global__ __launch_bounds__(512) void gemm_a8w8_panel_kernel(const A8W8Args p, 
 
 template <int MODE>
 static bool launch_a8_panel_t(A8W8Args& p, hipStream_t st) {
-    if (p.M > 64 || p.N % 16 != 0 || p.K % 32 != 0 || p.K < 8 * 128 || p.lda % 16 != 0 || p.ldb % 16 != 0 ||
+    if (p.M > kA8PanelRowsNarrow || p.N % 16 != 0 || p.K % 32 != 0 || p.K < 8 * 128 || p.lda % 16 != 0 || p.ldb % 16 != 0 ||
         ((uintptr_t)p.a % 16) != 0 || ((uintptr_t)p.b % 16) != 0)
         return false;
     // Rows per workgroup (16 rt) and 16-row activation blocks per pass (RT = 4 takes 2 or 4, RT = 2 takes 1 or

@@ -1632,6 +1632,10 @@ extern "C" size_t fnn_gemm_weight_only_workspace_bytes(int64_t M, int64_t N, int
     // once, so that every weight can be rounded as the reference rounds it
     if (M <= 64 || N <= 0 || K <= 0 || K % 8 != 0 || M > (1 << 30) || K > (1 << 30)) return 0;
     if (act_dtype != FNN_BF16 || scale_dtype != FNN_F16 || (group != 0 && group != 128)) return 0;
+    // ... where the tiled kernel takes the call (dispatch_wo): a shape it accepts, and more than 128 tiles or
+    // rows too short for the panel kernel (the count of 128-row tiles decides for 256-row tiles as well)
+    if (N % 128 != 0 || K % 256 != 0 || K < 512) return 0;
+    if (((M + 127) / 128) * (N / 128) <= 128 && K >= 1024) return 0;
     return act_f16_ws_bytes(M, K);
 }
 

@@ -307,6 +307,8 @@ class PrepackedInt4:
     """int4 weights with groups of 128 in the library's packed form (see hip_a16w4_prepack): the buffer and
     the shape it stands for."""
 
+    version = 1     # of the packed layout (written out in csrc/gemm_wo_prepacked.hip)
+
     def __init__(self, buffer, n, k, group):
         self.buffer, self.n, self.k, self.group = buffer, n, k, group
 

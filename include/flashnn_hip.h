@@ -146,7 +146,9 @@ int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const void* scale
  * rounds every dequantised weight to fp16 before the dot product, (q - zp) * s with both operations rounded
  * (flashnn/quant_gemm.py:14-36); the tiled kernel for more than 64 rows does the same where activations and
  * tables are fp16 (so do the few-row kernels with per-channel tables), and the result then differs from the
- * reference's only by the order of the fp32 additions.  bf16 activations (more than 64 rows, fp16 tables
+ * reference's only by the order of the fp32 additions.  (The tiled kernel takes the calls for which it has
+ * more than 128 tiles of 128 rows x 128 channels; narrower problems run as 64-row passes of the few-row
+ * kernel, faster there, and need no workspace.)  bf16 activations (more than 64 rows, fp16 tables
  * per channel or per group of 128) reach that form through
  * one conversion pass: every row becomes an fp16 row in the workspace, scaled by a power of two that makes
  * every value representable (undone exactly on the output).  Without a workspace, or with less than

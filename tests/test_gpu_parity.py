@@ -349,7 +349,7 @@ def test_a8w8_split_k_bit_exact(hip_lib, plan, mnk):
     assert torch.equal(plain, out)
 
 
-@pytest.mark.parametrize("mnk", [(256, 4096, 8192), (128, 2048, 16384), (384, 1920, 13312), (100, 1000, 9248), (2048, 4096, 4096),
+@pytest.mark.parametrize("mnk", [(256, 4096, 8192), (128, 2304, 16384), (384, 1920, 13312), (100, 1000, 9248), (2048, 4096, 4096),
                                  (1024, 1920, 13312), (640, 3584, 18944), (256, 4096, 6144)])
 def test_a8w8_workspace_entry_matches_plain(hip_lib, mnk):
     """fnn_gemm_a8w8_ws: shapes the library splits (and one it does not) against fnn_gemm_a8w8, bit for bit,
@@ -1445,7 +1445,7 @@ def test_split_k_packed_decode_and_moe_under_graph_capture():
     decode on packed weights, the tiled weight-only GEMM on bf16 rows (its scratch comes from torch's caching
     allocator inside the capture) and a fused MoE on the tiled kernel.  Every replay, with fresh inputs and
     eager work in between, equals the eager result."""
-    M, K, N = 256, 8192, 2048
+    M, K, N = 256, 8192, 2304
     w, ws = workloads.int8_weights(N, K, seed=91)
     wd, wsd = w.to(DEV), ws.to(DEV)
     a8 = torch.zeros(M, K, dtype=torch.int8, device=DEV)
@@ -1501,6 +1501,30 @@ def test_split_k_packed_decode_and_moe_under_graph_capture():
         for g, o in zip(got, outs):
             assert torch.equal(g, o), f"replay {rep}"
             assert bool(o.float().abs().sum() > 0)
+
+
+@pytest.mark.parametrize("M,N,K,out_ty", [(65, 2048, 8192, torch.bfloat16), (128, 1024, 4096, torch.float16), (200, 1920, 13312, torch.bfloat16),
+                                          (256, 2048, 4096, torch.float16), (257, 2048, 4096, torch.bfloat16), (130, 2064, 4096, torch.float16)])
+def test_a8w8_narrow_weights_run_as_passes_of_the_few_row_kernel(hip_lib, M, N, K, out_ty):
+    """65 to 256 rows over a weight matrix of at most 2048 channels with rows of 4096 bytes and more: 64-row
+    passes of the few-row kernel instead of a handful of tiles with K split; the same bits as the tiled
+    kernel named through the C ABI, and as the oracle's epilogue on the exact accumulators."""
+    a, b = _rand_i8((M, K), 5 + M).to(DEV), _rand_i8((N, K), 6 + N).to(DEV)
+    g = torch.Generator().manual_seed(M + N)
+    ar = (torch.rand(M, generator=g) * 0.05).half().to(DEV)
+    ac = (torch.rand(N, generator=g) * 0.05).half().to(DEV)
+    out = torch.empty(M, N, dtype=out_ty, device=DEV)
+    launchers.hip_gemm_a8w8_forward(out, a, b, ar, ac)
+    narrow = M <= 256 and N <= 2048
+    assert _lib.last_kernel().startswith("gemm_a8w8_panel_kernel" if narrow else "gemm_a8w8_ring_kernel"), _lib.last_kernel()
+    tiled = torch.empty_like(out)
+    rc = hip_lib.fnn_gemm_a8w8_tiled(_lib.ptr(tiled), _lib.ptr(a), _lib.ptr(b), _lib.ptr(ar), _lib.ptr(ac), M, N, K, K, K, N,
+                                     _lib.dtype_code(out_ty), _lib.FNN_F16, _lib.FNN_F16, 128, 128, 0, _lib.current_stream(out.device))
+    assert rc == 0 and _lib.last_kernel().startswith("gemm_a8w8_ring_kernel")
+    assert torch.equal(out, tiled)
+    acc = O.gemm_a8w8_acc(a.cpu().numpy(), b.cpu().numpy())
+    want = O.gemm_a8w8_epilogue_fp32(acc, O.to_np(ar.cpu()), O.to_np(ac.cpu()), O.tag_of(out))
+    assert np.array_equal(out.float().cpu().numpy(), want.astype(np.float32))
 
 
 # ------------------------------------------------------------------ strides through the C ABI

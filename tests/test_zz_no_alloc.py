@@ -35,7 +35,7 @@ def test_static_workspace_entry_matches_the_workspace_entry(hip_lib):
     ws = torch.zeros(16 << 20, dtype=torch.uint8, device=DEV)
     # (shape, named plan): the library's own choice on a large and then a smaller input, then named splits -
     # the last one smaller again and with more parts than the call before it
-    cases = [((384, 1920, 13312), (0, 0, 0)), ((128, 1024, 8192), (0, 0, 0)), ((300, 520, 8192), (256, 192, 3)),
+    cases = [((384, 1920, 13312), (0, 0, 0)), ((320, 1024, 8192), (0, 0, 0)), ((300, 520, 8192), (256, 192, 3)),
              ((96, 200, 4128), (128, 128, 5)), ((2048, 4096, 4096), (0, 0, 0))]
     for (M, N, K), plan in cases:
         print(f"[gpu-case] static workspace M={M} N={N} K={K} plan={plan}", file=sys.__stderr__, flush=True)
