@@ -1507,7 +1507,7 @@ size_t act_f16_ws_bytes(int64_t M, int64_t K) { return (size_t)((M * K * 2 + 255
 
 bool convert_act_to_f16(const WoArgs& p, WoArgs& q, hipStream_t st) {
     if (!p.cvt_ws || p.cvt_ws_bytes < act_f16_ws_bytes(p.M, p.K) || ((uintptr_t)p.cvt_ws % 16) != 0) return false;
-    if (p.scale_dtype != FNN_F16 || (p.zp && p.zp_dtype != FNN_F16) || (p.group != 0 && p.group != 128)) return false;
+    if (p.scale_dtype != FNN_F16 || (p.zp && p.zp_dtype != FNN_F16) || (p.group != 0 && group_shift(p.group) < 0)) return false;
     if (p.K % 8 != 0 || p.lda % 8 != 0 || ((uintptr_t)p.act % 16) != 0 || p.m_base != 0) return false;
     q = p;
     q.act = p.cvt_ws;
@@ -1521,6 +1521,30 @@ bool convert_act_to_f16(const WoArgs& p, WoArgs& q, hipStream_t st) {
     return true;
 }
 
+// Any number of rows through the decode kernels, as many rows a pass as they take (8, 4, 2 or 1: their
+// activations and group tables have to fit the LDS); false, with nothing launched, if they do not take the
+// shape at all.  Every pass reads the weights again: for the shapes that would otherwise fall to the
+// one-thread-per-output kernel (groups of 32 with more than 8 rows: 0.5 - 130 ms there, 20 to 100 times less
+// here).
+template <int WBITS, int ADT>
+static bool decode_in_passes(const WoArgs& p, hipStream_t st) {
+    const int esz = p.out_dtype == FNN_F32 ? 4 : 2;
+    for (int rows = 8; rows >= 1; rows >>= 1) {
+        for (int m0 = 0; m0 < p.M; m0 += rows) {
+            WoArgs q = p;
+            q.act = (const char*)p.act + (int64_t)m0 * p.lda * 2;
+            q.out = (char*)p.out + (int64_t)m0 * p.ldc * esz;
+            q.M = p.M - m0 < rows ? p.M - m0 : rows;
+            if (!launch_decode<WBITS, ADT>(q, st, false)) {
+                if (m0 != 0) return true;      // (cannot happen: a pass of fewer rows needs less than the first)
+                break;
+            }
+            if (m0 + rows >= p.M) return true;
+        }
+    }
+    return false;
+}
+
 template <int WBITS, int ADT>
 static void dispatch_wo(WoArgs& p, hipStream_t st) {
     const bool aligned = p.K % 64 == 0 && p.ldw % 16 == 0 && p.lda % 8 == 0 && ((uintptr_t)p.qw % 16) == 0 &&
@@ -1530,7 +1554,7 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
     if (p.group == 0 && p.K % 128 != 0 && launch_wo_panel(p, WBITS, ADT, st)) return;
     // groups of 32: only the decode kernel that dequantises every weight takes them (the kernels below walk
     // groups of 64 and more)
-    if (aligned && p.group == 32 && launch_decode<WBITS, ADT>(p, st, false)) return;
+    if (aligned && p.group == 32 && decode_in_passes<WBITS, ADT>(p, st)) return;
     if (!fast) {
         const int64_t total = (int64_t)p.M * p.N;
         note_kernel("gemm_wo_any_kernel", WBITS);
@@ -1554,6 +1578,11 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
         if (launch_wo_panel(p, WBITS, ADT, st)) return;
         if (!fills && launch_wo_tile(p, WBITS, ADT, st)) return;
     }
+    // groups of 64, up to 8 rows, fp16 throughout: the decode kernel rounds every dequantised weight to fp16 as the
+    // reference does (flashnn/quant_gemm.py:14-36), the panel kernel scales group sums in fp32
+    if (p.group == 64 && p.M <= 8 && ADT == FNN_F16 && p.scale_dtype == FNN_F16 && (!p.zp || p.zp_dtype == FNN_F16) &&
+        launch_decode<WBITS, ADT>(p, st, false))
+        return;
     if (p.M >= 2 && launch_wo_panel(p, WBITS, ADT, st)) return;
     if (launch_decode<WBITS, ADT>(p, st, false)) return;
     // up to 64 activation rows per pass over the weights
@@ -1631,7 +1660,7 @@ extern "C" size_t fnn_gemm_weight_only_workspace_bytes(int64_t M, int64_t N, int
     // bf16 activations with fp16 tables, more than 64 rows (the tiled kernel): the rows are converted to fp16
     // once, so that every weight can be rounded as the reference rounds it
     if (M <= 64 || N <= 0 || K <= 0 || K % 8 != 0 || M > (1 << 30) || K > (1 << 30)) return 0;
-    if (act_dtype != FNN_BF16 || scale_dtype != FNN_F16 || (group != 0 && group != 128)) return 0;
+    if (act_dtype != FNN_BF16 || scale_dtype != FNN_F16 || (group != 0 && (group_shift((int)group) < 0 || K % group != 0))) return 0;
     // ... where the tiled kernel takes the call (dispatch_wo): a shape it accepts, and more than 128 tiles or
     // rows too short for the panel kernel (the count of 128-row tiles decides for 256-row tiles as well)
     if (N % 128 != 0 || K % 256 != 0 || K < 512) return 0;

@@ -50,9 +50,12 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // Three more instructions per pair of weights where the fold costs two per output and slab: at these row
 // counts the kernel streams weights, and the vector unit has no room for it.  Not kept; the tiled kernel for
 // more than 64 rows has it.)
-template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL, bool MOE = false, int REFQ = 0>
+// GSUB = 2: tables per group of 64 values - two groups per slab, each half of the slab's MFMAs folded with its own
+// table row (G128 is set as well: the table path is the same, with twice the rows).
+template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL, bool MOE = false, int REFQ = 0, int GSUB = 1>
 __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, const int passes, const MoeArgs q) {
     static_assert(!REFQ || (ADT == FNN_F16 && !G128 && !MOE), "reference rounding: fp16, per-channel");
+    static_assert(GSUB == 1 || (GSUB == 2 && G128 && !MOE), "groups of 64: plain calls with group tables");
     // Gathered form with group tables: the reference's mixture-of-experts launcher lays them out
     // [expert][channel][group] (flashnn/triton_kernels/fused_moe_a16w4.py:336-344), the transpose of the
     // [group][channel] tables above, so 16-byte loads of 8 neighbouring channels do not exist.  The
@@ -186,14 +189,16 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     // ---- group tables: NCL consecutive channels per lane
     typedef typename std::conditional<NH == 2, v4u, v2u>::type tab_t;
     const int n0 = NH * (row0 + 4 * lg);
-    const uint16_t* sptr = (const uint16_t*)p.scale + (int64_t)sl0 * p.N + NH * row0;             // scalar
-    const uint16_t* zptr = (p.zp ? (const uint16_t*)p.zp : (const uint16_t*)p.scale) + (int64_t)sl0 * p.N + NH * row0;
+    const uint16_t* sptr = (const uint16_t*)p.scale + NH * row0;             // scalar
+    const uint16_t* zptr = (p.zp ? (const uint16_t*)p.zp : (const uint16_t*)p.scale) + NH * row0;
     const uint32_t tab_off = NH * 4 * lg * 2;                                                        // bytes
     const bool has_zp = p.zp != nullptr;
     // without zero points the second table load reads the scales again and is multiplied away
     const float zmul = has_zp ? 1.f : 0.f;
-    auto load_tab = [&](const uint16_t* base, int jj) -> tab_t {
-        const int j = min(jj, nsl - 1);
+    // (groups of 128 << gshift values: the slab's table row is its number >> gshift; groups of 64: rows 2 j and 2 j + 1)
+    auto load_tab = [&](const uint16_t* base, int jj, int sub) -> tab_t {
+        const int slab = sl0 + min(jj, nsl - 1);
+        const int j = GSUB == 2 ? 2 * slab + sub : slab >> p.gshift;
         return *(const tab_t*)((const char*)(base + (int64_t)j * p.N) + tab_off);
     };
 
@@ -219,7 +224,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
 
     // loads issued per iteration, in this order: NCP copies, 2 weight loads, 2 table loads
-    constexpr int C = NCP + 2 + (TABG ? 2 : 0);
+    constexpr int C = NCP + 2 + (TABG ? 2 * GSUB : 0);
     // the newest load slab j depends on is its last copy, issued three iterations earlier; after
     // it came the rest of that iteration and two whole ones
     constexpr int X = (C - NCP) + 2 * C;
@@ -233,7 +238,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     };
 
     v4u wq[D][2];
-    tab_t sq[4], zq[4];
+    tab_t sq[4][GSUB], zq[4][GSUB];
     constexpr int CHW = RT * 16 * NH;           // channels of the workgroup
     constexpr int TABG_MAX = 64;                // groups the LDS tables hold (K <= 8192)
     __shared__ __attribute__((aligned(16))) uint16_t tabs[TABLDS ? 2 * TABG_MAX * CHW : 8];
@@ -268,7 +273,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
 
     // All activation fragments of the slab are requested first, the weights are converted while
     // those reads are in flight, and the MFMAs then run back to back behind a single wait.
-    auto compute = [&](const char* stage, const v4u w0, const v4u w1, const bool last) {
+    auto compute = [&](const char* stage, const v4u w0, const v4u w1, const bool last, const tab_t s_first, const tab_t z_first) {
         v4u bf[2][MB][2];
 #pragma unroll
         for (int s = 0; s < 2; ++s)
@@ -302,7 +307,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
                     }
             }
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
+            for (int s = 0; s < 2; ++s) {
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
                     accg[mb][0] = MT::mma(e[s][0], bf[s][mb][0], accg[mb][0]);
@@ -312,6 +317,8 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
                     accg[mb][1] = MT::mma(o[s][1], bf[s][mb][1], accg[mb][1]);
                     if constexpr (!REFQ) asum[mb] = MT::mma(ones, bf[s][mb][1], asum[mb]);
                 }
+                if constexpr (GSUB == 2) { if (s == 0) fold(s_first, z_first); }     // values 0 .. 63 of the slab: a group of their own
+            }
         } else {
             v4u c[2][2];
             convert_w8<ADT>(w0, c[0][0], c[0][1]);
@@ -323,7 +330,7 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
                     for (int h = 0; h < 2; ++h) c[s][h] = ref_dq_f16<REFQ == 2>(c[s][h], rq_c, rq_z[0], rq_s[0]);
             }
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
+            for (int s = 0; s < 2; ++s) {
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
                     accg[mb][0] = MT::mma(c[s][0], bf[s][mb][0], accg[mb][0]);
@@ -331,6 +338,8 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
                     accg[mb][0] = MT::mma(c[s][1], bf[s][mb][1], accg[mb][0]);
                     if constexpr (!REFQ) asum[mb] = MT::mma(ones, bf[s][mb][1], asum[mb]);
                 }
+                if constexpr (GSUB == 2) { if (s == 0) fold(s_first, z_first); }
+            }
         }
     };
 
@@ -348,13 +357,15 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         __builtin_amdgcn_sched_barrier(0);                                 \
         if (mine_) {                                                       \
             compute(CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1]), \
-                    !G128 && part_tail && (JJ) == nsl - 1);                \
+                    !G128 && part_tail && (JJ) == nsl - 1, sq[Q][0], zq[Q][0]); \
             if constexpr (TABLDS) fold(lds_tab(0, (JJ)), lds_tab(1, (JJ))); \
-            else if constexpr (G128) fold(sq[Q], zq[Q]);                   \
+            else if constexpr (G128) fold(sq[Q][GSUB - 1], zq[Q][GSUB - 1]); \
         }                                                                  \
         if constexpr (TABG) {                                              \
-            sq[Q] = load_tab(sptr, (JJ) + 4);                              \
-            zq[Q] = load_tab(zptr, (JJ) + 4);                              \
+            _Pragma("unroll") for (int sub_ = 0; sub_ < GSUB; ++sub_) {    \
+                sq[Q][sub_] = load_tab(sptr, (JJ) + 4, sub_);              \
+                zq[Q][sub_] = load_tab(zptr, (JJ) + 4, sub_);              \
+            }                                                              \
         }                                                                  \
         __builtin_amdgcn_sched_barrier(0);                                 \
     } while (0)
@@ -366,22 +377,22 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         wq[d][0] = load_w(d, 0);
         wq[d][1] = load_w(d, 1);
     }
-    if constexpr (TABG) { sq[0] = load_tab(sptr, 0); zq[0] = load_tab(zptr, 0); }
+    if constexpr (TABG) { for (int sub = 0; sub < GSUB; ++sub) { sq[0][sub] = load_tab(sptr, 0, sub); zq[0][sub] = load_tab(zptr, 0, sub); } }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st0, 0);
     wq[D - 3][0] = load_w(D - 3, 0);
     wq[D - 3][1] = load_w(D - 3, 1);
-    if constexpr (TABG) { sq[1] = load_tab(sptr, 1); zq[1] = load_tab(zptr, 1); }
+    if constexpr (TABG) { for (int sub = 0; sub < GSUB; ++sub) { sq[1][sub] = load_tab(sptr, 1, sub); zq[1][sub] = load_tab(zptr, 1, sub); } }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st1, 1);
     wq[D - 2][0] = load_w(D - 2, 0);
     wq[D - 2][1] = load_w(D - 2, 1);
-    if constexpr (TABG) { sq[2] = load_tab(sptr, 2); zq[2] = load_tab(zptr, 2); }
+    if constexpr (TABG) { for (int sub = 0; sub < GSUB; ++sub) { sq[2][sub] = load_tab(sptr, 2, sub); zq[2][sub] = load_tab(zptr, 2, sub); } }
     __builtin_amdgcn_sched_barrier(0);
     copy_act(st2, 2);
     wq[D - 1][0] = load_w(D - 1, 0);
     wq[D - 1][1] = load_w(D - 1, 1);
-    if constexpr (TABG) { sq[3] = load_tab(sptr, 3); zq[3] = load_tab(zptr, 3); }
+    if constexpr (TABG) { for (int sub = 0; sub < GSUB; ++sub) { sq[3][sub] = load_tab(sptr, 3, sub); zq[3][sub] = load_tab(zptr, 3, sub); } }
     __builtin_amdgcn_sched_barrier(0);
 
     if constexpr (TABLDS) {
@@ -558,10 +569,14 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     constexpr int NH = WBITS == 4 ? 2 : 1;
     const int wrows = WBITS == 4 ? p.N / 2 : p.N;
     if (wrows % 16 != 0 || p.K % 32 != 0 || p.K < 8 * 128) return false;
-    if (p.group != 0 && p.group != 128) return false;
-    if (p.group == 128 && p.K % 128 != 0) return false;
+    // tables per channel, or per group of 128, 256, 512 .. values
+    // (or per group of 64: two groups per slab, K a multiple of 128)
+    const bool g64 = p.group == 64 && p.K % 128 == 0;
+    const int gs = p.group == 0 || g64 ? 0 : group_shift(p.group);
+    if (gs < 0 || (p.group != 0 && p.K % p.group != 0)) return false;
+    p.gshift = gs;
     if (p.lda % 8 != 0 || p.ldw % 16 != 0 || ((uintptr_t)p.qw % 16) != 0 || ((uintptr_t)p.act % 16) != 0) return false;
-    if (p.group == 128) {
+    if (p.group != 0) {
         const bool tables16 = is16(p.scale_dtype) && (!p.zp || p.zp_dtype == p.scale_dtype) &&
                               p.N % (4 * NH) == 0 && ((uintptr_t)p.scale % (8 * NH)) == 0 &&
                               (!p.zp || ((uintptr_t)p.zp % (8 * NH)) == 0);
@@ -586,6 +601,12 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
                 break;                                                                                   \
             }                                                                                            \
         }                                                                                                \
+        if constexpr (G) {                                                                               \
+            if (g64) {                                                                                   \
+                gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, NTLV, false, 0, 2><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{}); \
+                break;                                                                                   \
+            }                                                                                            \
+        }                                                                                                \
         gemm_wo_panel_kernel<WBITS, ADT, G, SDTV, MBV, RTV, 4, NTLV><<<grid, dim3(512), 0, st>>>(p, passes, MoeArgs{}); \
     } while (0)
 #define FNN_PANEL2(G, SDTV, MBV, RTV)                                                                    \
@@ -606,7 +627,7 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
             FNN_PANEL2(G, SDTV, 1, 1);                       \
         }                                                    \
     } while (0)
-    if (p.group == 128) {
+    if (p.group != 0) {
         if (p.scale_dtype == FNN_F16) FNN_PANEL(true, FNN_F16);
         else FNN_PANEL(true, FNN_BF16);
     } else {

@@ -178,7 +178,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     const uint32_t gt = (uint32_t)n0 * 2 + (lane & 15) * 16;
     auto copy_t = [&](char* stage, int j) {
         if constexpr (G128 && !MOE) {
-            const int64_t off = (int64_t)min(j, KT - 1) * p.N * 2;
+            const int64_t off = (int64_t)(min(j, KT - 1) >> p.gshift) * p.N * 2;      // groups of 128 << gshift values
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(t_src + off + gt), (lds_ptr_t)stage, 16, 0, 0);
         }
     };
@@ -546,11 +546,14 @@ template <int WBITS, int ADT>
 static bool launch_tile_t(WoArgs& p, hipStream_t st) {
     constexpr int NH = WBITS == 4 ? 2 : 1;
     if (p.M <= 64 || p.N % 128 != 0 || p.K % 256 != 0 || p.K < 512) return false;
-    if (p.group != 0 && p.group != 128) return false;
+    // tables per channel, or per group of 128, 256, 512 .. values
+    const int gs = p.group == 0 ? 0 : group_shift(p.group);
+    if (gs < 0 || (p.group != 0 && p.K % p.group != 0)) return false;
+    p.gshift = gs;
     if (p.lda % 8 != 0 || p.ldw % 16 != 0 || ((uintptr_t)p.qw % 16) != 0 || ((uintptr_t)p.act % 16) != 0) return false;
     // the copies address rows with 32-bit offsets from the tile's first row
     if ((int64_t)256 * p.lda * 2 >= (1LL << 31) || (int64_t)(128 / NH) * p.ldw >= (1LL << 31)) return false;
-    if (p.group == 128) {
+    if (p.group != 0) {
         const bool tables16 = is16(p.scale_dtype) && (!p.zp || p.zp_dtype == p.scale_dtype) &&
                               ((uintptr_t)p.scale % 16) == 0 && (!p.zp || ((uintptr_t)p.zp % 16) == 0);
         if (!tables16) return false;
@@ -566,7 +569,7 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
     const dim3 grid(((tiles + 7) / 8) * 8);   // (workgroups beyond the last tile return at once)
     // fp16 activations with fp16 tables: every weight rounded as the reference rounds it
     const bool refq = ADT == FNN_F16 && p.scale_dtype == FNN_F16 && (!p.zp || p.zp_dtype == FNN_F16) &&
-                      (p.group == 128 || ((uintptr_t)p.scale % 2) == 0);
+                      (p.group != 0 || ((uintptr_t)p.scale % 2) == 0);
     note_kernel(refq ? "gemm_wo_tile_kernel(per-weight rounding)" : "gemm_wo_tile_kernel", WBITS, bm, 128);
 #define FNN_TILE(G, SDTV, RQ)                                                                            \
     do {                                                                                                 \
@@ -580,12 +583,12 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
     } while (0)
     if constexpr (ADT == FNN_F16) {
         if (refq) {
-            if (p.group == 128) { if (p.zp) FNN_TILE(true, FNN_F16, 2); else FNN_TILE(true, FNN_F16, 1); }
+            if (p.group != 0) { if (p.zp) FNN_TILE(true, FNN_F16, 2); else FNN_TILE(true, FNN_F16, 1); }
             else { if (p.zp) FNN_TILE(false, FNN_F16, 2); else FNN_TILE(false, FNN_F16, 1); }
             return true;
         }
     }
-    if (p.group == 128) {
+    if (p.group != 0) {
         if (p.scale_dtype == FNN_F16) FNN_TILE(true, FNN_F16, 0);
         else FNN_TILE(true, FNN_BF16, 0);
     } else {

@@ -17,6 +17,7 @@ struct WoArgs {
     int M, N, K;          // N = output channels
     int64_t lda, ldw, ldc;
     int group;            // 0 = per channel
+    int gshift;           // groups of 128 << gshift values (the panel and tiled kernels: table row of slab j is j >> gshift)
     int out_dtype, scale_dtype, zp_dtype, bias_dtype;
     int m_base;           // first activation row handled by this launch
     void* cvt_ws;         // scratch for bf16 activations converted to fp16 (NULL: none), cvt_ws_bytes of it
@@ -24,6 +25,14 @@ struct WoArgs {
     const float* act_unscale;   // per activation row: what the output is multiplied by (NULL: nothing); set where
                                 // the rows were scaled by a power of two on their way from bf16 to fp16
 };
+
+// s if group == 128 << s (the group sizes whose tables the 128-value slabs of the panel and tiled kernels can
+// walk: a slab lies within one group), else -1
+inline int group_shift(int group) {
+    for (int s = 0; s < 16; ++s)
+        if (group == (128 << s)) return s;
+    return -1;
+}
 
 constexpr int kWoWaves = 8;
 constexpr int kPF = 8;    // weight loads in flight per lane

@@ -149,7 +149,7 @@ int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const void* scale
  * reference's only by the order of the fp32 additions.  (The tiled kernel takes the calls for which it has
  * more than 128 tiles of 128 rows x 128 channels; narrower problems run as 64-row passes of the few-row
  * kernel, faster there, and need no workspace.)  bf16 activations (more than 64 rows, fp16 tables
- * per channel or per group of 128) reach that form through
+ * per channel or per group of 128, 256, 512 .. values) reach that form through
  * one conversion pass: every row becomes an fp16 row in the workspace, scaled by a power of two that makes
  * every value representable (undone exactly on the output).  Without a workspace, or with less than
  *   fnn_gemm_weight_only_workspace_bytes(M, N, K, group, act_dtype, scale_dtype)   (0: the call would not use one)

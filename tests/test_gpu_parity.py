@@ -957,6 +957,56 @@ def test_weight_only_large_m_on_narrow_matrices(bits, group, M, N, K):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("group", [64, 256, 512])
+@pytest.mark.parametrize("M,N,K", [(5, 1024, 1024), (16, 4096, 2048), (40, 1056, 2560), (64, 8192, 1024), (100, 2048, 1536),
+                                   (200, 8320, 2560), (300, 512, 4096)])
+def test_weight_only_groups_of_64_256_512(bits, group, M, N, K):
+    """Tables per group of 64 (two groups per 128-value slab, each half folded with its own table row) and of 256
+    or 512 values (a table row serves 2 or 4 slabs) on the MFMA kernels: the panel kernel up to 64 rows and in
+    64-row passes, the tiled kernel on wide matrices with groups of 256 and 512."""
+    if K % group:
+        K = (K // group) * group
+    act_ty = torch.float16 if M % 16 else torch.bfloat16
+    scale_ty = torch.bfloat16 if M == 40 else torch.float16
+    case = _wo_inputs(M, N, K, group, bits, act_ty, scale_ty, with_zp=M != 16, with_bias=M in (5, 200), seed=900 + M + group)
+    _wo_check(*case, group, bits, act_ty, cols=None if N <= 1056 else np.r_[0:64, N // 2 - 32:N // 2 + 32, N - 64:N])
+    tiled = M > 64 and group != 64 and N == 8320
+    # (groups of 64 with up to 8 rows, fp16 throughout, stay on the kernel that rounds per weight as the reference does)
+    want_kernel = "gemm_wo_tile_kernel" if tiled else "gemm_wo_decode_lds_kernel" if (group, M) == (64, 5) else "gemm_wo_panel_kernel"
+    assert _lib.last_kernel().startswith(want_kernel), _lib.last_kernel()
+
+
+@pytest.mark.parametrize("group,M,N", [(64, 48, 4096), (256, 48, 4096), (512, 24, 2048), (64, 150, 1024), (256, 200, 16640), (512, 130, 16640)])
+def test_weight_only_group_rows_one_hot(group, M, N):
+    """One-hot activation rows pick single weight columns, each scaled by the table row of its own group: a table
+    row taken from a neighbouring group shows as a wrong scale or zero point (tables differ from group to group)."""
+    K = 2048
+    g = torch.Generator().manual_seed(group + M)
+    w = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(K // group, N).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(-4, 4, (K // group, N), generator=g).half()
+    ks = torch.randperm(K, generator=g)[:M]
+    ks[:4] = torch.tensor([0, group - 1, group, K - 1])
+    act = torch.zeros(M, K, dtype=torch.float16)
+    act[torch.arange(M), ks] = 2.0
+    qw = torch.from_numpy(O.pack_int4(w.numpy()))
+    out = flashnn_amd.GemmWeightOnly(torch.float16)(act.to(DEV), qw.to(DEV), scale.to(DEV), None, zp.to(DEV))
+    assert _lib.last_kernel().startswith("gemm_wo_tile_kernel" if N == 16640 else "gemm_wo_panel_kernel"), _lib.last_kernel()
+    want = 2.0 * (w[:, ks].float() - zp[ks // group].float().t()) * scale[ks // group].float().t()   # [N, M]
+    np.testing.assert_allclose(out.float().cpu().numpy(), want.t().half().float().numpy(), rtol=2.0 ** -10, atol=1e-6)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("M,N,K", [(9, 1024, 4096), (20, 520, 1152), (70, 256, 2944)])
+def test_weight_only_groups_of_32_many_rows(bits, M, N, K):
+    """Tables per group of 32 with more than 8 rows: passes of the few-row kernel over blocks of up to 8 rows, with
+    the reference's per-weight rounding (fp16 activations and tables), so the stated tolerance holds throughout."""
+    case = _wo_inputs(M, N, K, 32, bits, torch.float16, torch.float16, True, M == 20, seed=M + K)
+    _wo_check(*case, 32, bits, torch.float16, strict=True)
+    assert _lib.last_kernel().startswith("gemm_wo_decode_lds_kernel"), _lib.last_kernel()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("group", [0, 128])
 def test_weight_only_bf16_rows_through_the_conversion_pass(hip_lib, bits, group):
     """bf16 activations, fp16 tables, more than 64 rows: with scratch memory the rows become fp16 rows (scaled
