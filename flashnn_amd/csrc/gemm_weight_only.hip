@@ -31,8 +31,13 @@
 namespace fnn {
 
 
-template <int WBITS, int ADT, int MB, bool GROUPED>
+// G32: tables per group of 32 values.  A 64-value step is then two groups, and the two MFMAs of a step must each
+// cover one of them: a lane takes values 8 lg .. 8 lg + 7 of either half of the step (two 8-byte weight loads
+// and two activation pieces 32 values apart) instead of 16 consecutive ones, and the sums are folded after
+// each half.
+template <int WBITS, int ADT, int MB, bool GROUPED, bool G32 = false>
 __global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoArgs p) {
+    static_assert(!G32 || GROUPED, "groups of 32 are group tables");
     typedef MfmaT<ADT> MT;
     constexpr int NH = WBITS == 4 ? 2 : 1;      // channel halves per weight row (int4: even/odd)
     constexpr float c_off = WBITS == 4 ? (ADT == FNN_F16 ? 1024.f + 8.f : 128.f + 8.f)
@@ -58,23 +63,28 @@ __global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoA
     const int s_end = (int)((int64_t)steps * (wave + 1) / kWoWaves);
 
     const int wrow = min(row0 + li, wrows - 1);
-    const char* wptr = (const char*)p.qw + (int64_t)wrow * p.ldw + lg * 16;
+    const char* wptr = (const char*)p.qw + (int64_t)wrow * p.ldw + lg * (G32 ? 8 : 16);
     const uint16_t* aptr[MB];
     bool avalid[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const int m = p.m_base + mb * 16 + li;
         avalid[mb] = m < p.M;
-        aptr[mb] = (const uint16_t*)p.act + (int64_t)min(m, p.M - 1) * p.lda + lg * 16;
+        aptr[mb] = (const uint16_t*)p.act + (int64_t)min(m, p.M - 1) * p.lda + lg * (G32 ? 8 : 16);
     }
 
     auto load_w = [&](int step) -> v4u {
         const int s = min(step, s_end - 1);
-        return *(const v4u*)(wptr + (int64_t)s * 64);
+        if constexpr (G32) {
+            const v2u lo = *(const v2u*)(wptr + (int64_t)s * 64), hi = *(const v2u*)(wptr + (int64_t)s * 64 + 32);
+            return v4u{lo[0], lo[1], hi[0], hi[1]};
+        } else {
+            return *(const v4u*)(wptr + (int64_t)s * 64);
+        }
     };
     auto load_a = [&](int mb, int step, int half) -> v4u {
         const int s = min(step, s_end - 1);
-        return avalid[mb] ? *(const v4u*)(aptr[mb] + (int64_t)s * 64 + half * 8) : v4u{0, 0, 0, 0};
+        return avalid[mb] ? *(const v4u*)(aptr[mb] + (int64_t)s * 64 + half * (G32 ? 32 : 8)) : v4u{0, 0, 0, 0};
     };
 
     v4f outv[MB][NH], accg[MB][NH], asum[MB];
@@ -141,7 +151,22 @@ __global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoA
                         aq[i % kPFA][mb][0] = load_a(mb, step + kPFA, 0);
                         aq[i % kPFA][mb][1] = load_a(mb, step + kPFA, 1);
                     }
-                    if constexpr (WBITS == 4) {
+                    if constexpr (G32) {
+                        v4u e[2], o[2];
+                        if constexpr (WBITS == 4) convert_w4<ADT>(w, e[0], e[1], o[0], o[1]);
+                        else convert_w8<ADT>(w, e[0], e[1]);
+#pragma unroll
+                        for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+                            for (int mb = 0; mb < MB; ++mb) {
+                                const v4u b = WBITS == 4 ? perm_act_w4(a[mb][hf]) : a[mb][hf];
+                                accg[mb][0] = MT::mma(e[hf], b, accg[mb][0]);
+                                if constexpr (WBITS == 4) accg[mb][1] = MT::mma(o[hf], b, accg[mb][1]);
+                                asum[mb] = MT::mma(ones, b, asum[mb]);
+                            }
+                            fold(2 * step + hf);
+                        }
+                    } else if constexpr (WBITS == 4) {
                         v4u e0, e1, o0, o1;
                         convert_w4<ADT>(w, e0, e1, o0, o1);
 #pragma unroll
@@ -166,7 +191,7 @@ __global__ __launch_bounds__(kWoWaves * 64) void gemm_wo_stream_kernel(const WoA
                             asum[mb] = MT::mma(ones, a[mb][1], asum[mb]);
                         }
                     }
-                    if constexpr (GROUPED) {
+                    if constexpr (GROUPED && !G32) {
                         if ((step + 1) % gsteps == 0 || step + 1 == s_end) fold(step / gsteps);
                     }
                 }
@@ -1306,7 +1331,8 @@ static void launch_stream(WoArgs& p, hipStream_t st) {
     const int tiles = (wrows + 15) / 16;
     const dim3 grid(((tiles + 7) / 8) * 8), block(kWoWaves * 64);
     note_kernel("gemm_wo_stream_kernel", WBITS, MB, p.group);
-    if (p.group > 0) gemm_wo_stream_kernel<WBITS, ADT, MB, true><<<grid, block, 0, st>>>(p);
+    if (p.group == 32) gemm_wo_stream_kernel<WBITS, ADT, MB, true, true><<<grid, block, 0, st>>>(p);
+    else if (p.group > 0) gemm_wo_stream_kernel<WBITS, ADT, MB, true><<<grid, block, 0, st>>>(p);
     else gemm_wo_stream_kernel<WBITS, ADT, MB, false><<<grid, block, 0, st>>>(p);
 }
 
@@ -1549,12 +1575,13 @@ template <int WBITS, int ADT>
 static void dispatch_wo(WoArgs& p, hipStream_t st) {
     const bool aligned = p.K % 64 == 0 && p.ldw % 16 == 0 && p.lda % 8 == 0 && ((uintptr_t)p.qw % 16) == 0 &&
                          ((uintptr_t)p.act % 16) == 0;
-    const bool fast = aligned && (p.group == 0 || p.group % 64 == 0);
+    const bool fast = aligned && (p.group == 0 || p.group % 64 == 0 || p.group == 32);
     // per-channel scales with K a multiple of 32 only: the panel kernel handles the partial last slab
     if (p.group == 0 && p.K % 128 != 0 && launch_wo_panel(p, WBITS, ADT, st)) return;
-    // groups of 32: only the decode kernel that dequantises every weight takes them (the kernels below walk
-    // groups of 64 and more)
-    if (aligned && p.group == 32 && decode_in_passes<WBITS, ADT>(p, st)) return;
+    // groups of 32, up to 8 rows, fp16 throughout: the decode kernel that rounds every dequantised weight to fp16
+    // as the reference does, fewer rows at a time where its tables do not fit for all; everything else with
+    // groups of 32 goes to the stream kernel at the end
+    if (aligned && p.group == 32 && p.M <= 8 && decode_in_passes<WBITS, ADT>(p, st)) return;
     if (!fast) {
         const int64_t total = (int64_t)p.M * p.N;
         note_kernel("gemm_wo_any_kernel", WBITS);

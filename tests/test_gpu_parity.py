@@ -997,13 +997,34 @@ def test_weight_only_group_rows_one_hot(group, M, N):
 
 
 @pytest.mark.parametrize("bits", [8, 4])
-@pytest.mark.parametrize("M,N,K", [(9, 1024, 4096), (20, 520, 1152), (70, 256, 2944)])
-def test_weight_only_groups_of_32_many_rows(bits, M, N, K):
-    """Tables per group of 32 with more than 8 rows: passes of the few-row kernel over blocks of up to 8 rows, with
-    the reference's per-weight rounding (fp16 activations and tables), so the stated tolerance holds throughout."""
-    case = _wo_inputs(M, N, K, 32, bits, torch.float16, torch.float16, True, M == 20, seed=M + K)
-    _wo_check(*case, 32, bits, torch.float16, strict=True)
-    assert _lib.last_kernel().startswith("gemm_wo_decode_lds_kernel"), _lib.last_kernel()
+@pytest.mark.parametrize("act_ty,scale_ty", [(torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16),
+                                             (torch.bfloat16, torch.float16)])
+@pytest.mark.parametrize("M,N,K", [(3, 1024, 1024), (9, 1024, 4096), (20, 520, 1152), (70, 256, 2944), (200, 96, 512)])
+def test_weight_only_groups_of_32_many_rows(bits, M, N, K, act_ty, scale_ty):
+    """Tables per group of 32 beyond the decode kernel's reach (more than 8 rows, or bf16 somewhere): the stream
+    kernel's form whose two MFMAs of a 64-value step cover one group each, in 64-row passes."""
+    case = _wo_inputs(M, N, K, 32, bits, act_ty, scale_ty, True, M == 20, seed=M + K)
+    _wo_check(*case, 32, bits, act_ty)
+    small_fp16 = M <= 8 and act_ty == torch.float16
+    assert _lib.last_kernel().startswith("gemm_wo_decode_lds_kernel" if small_fp16 else "gemm_wo_stream_kernel"), _lib.last_kernel()
+
+
+def test_weight_only_groups_of_32_one_hot():
+    """One-hot rows pick single weight columns, each with the table row of its own group of 32."""
+    M, N, K, group = 40, 256, 1024, 32
+    g = torch.Generator().manual_seed(32)
+    w = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(K // group, N).uniform_(1e-3, 1e-2, generator=g).half()
+    zp = torch.randint(-4, 4, (K // group, N), generator=g).half()
+    ks = torch.randperm(K, generator=g)[:M]
+    ks[:6] = torch.tensor([0, 31, 32, 63, 64, K - 1])
+    act = torch.zeros(M, K, dtype=torch.float16)
+    act[torch.arange(M), ks] = 2.0
+    qw = torch.from_numpy(O.pack_int4(w.numpy()))
+    out = flashnn_amd.GemmWeightOnly(torch.float16)(act.to(DEV), qw.to(DEV), scale.to(DEV), None, zp.to(DEV))
+    assert _lib.last_kernel().startswith("gemm_wo_stream_kernel"), _lib.last_kernel()
+    want = 2.0 * (w[:, ks].float() - zp[ks // group].float().t()) * scale[ks // group].float().t()   # [N, M]
+    np.testing.assert_allclose(out.float().cpu().numpy(), want.t().half().float().numpy(), rtol=2.0 ** -10, atol=1e-6)
 
 
 @pytest.mark.parametrize("bits", [4, 8])
