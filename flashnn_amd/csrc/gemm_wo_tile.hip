@@ -218,6 +218,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
 
     // REFQ with per-channel tables: the scale and zero point of the channels this lane's operand rows hold
     const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
+    const v2h rq_c_odd = pair_of_f16_bits(0x5480u);                      // 72: .. to the odd channel of an int4 row
     v2h rq_s[NA], rq_z[NA];
     if constexpr (ROUNDQ && !G128) {
 #pragma unroll
@@ -341,7 +342,9 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
 #pragma unroll
                 for (int f = 0; f < NF; ++f) {
                     const v4u w = *(const v4u*)(sw + w_rd[h] + f * 16 * 128);
-                    if constexpr (WBITS == 4)
+                    if constexpr (WBITS == 4 && ROUNDQ)
+                        convert_w4_nat_f16_2off(w, A[2 * h][2 * f], A[2 * h + 1][2 * f], A[2 * h][2 * f + 1], A[2 * h + 1][2 * f + 1]);
+                    else if constexpr (WBITS == 4)
                         convert_w4_nat<ADT>(w, A[2 * h][2 * f], A[2 * h + 1][2 * f], A[2 * h][2 * f + 1], A[2 * h + 1][2 * f + 1]);
                     else
                         convert_w8<ADT>(w, A[2 * h][f], A[2 * h + 1][f]);
@@ -350,7 +353,8 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-                    for (int a = 0; a < NA; ++a) A[ks][a] = ref_dq_f16<REFQ == 2>(A[ks][a], rq_c, rq_z[a], rq_s[a]);
+                    for (int a = 0; a < NA; ++a)
+                        A[ks][a] = ref_dq_f16<REFQ == 2>(A[ks][a], WBITS == 4 && (a % NH) == 1 ? rq_c_odd : rq_c, rq_z[a], rq_s[a]);
             }
         };
         auto mfma_slab = [&](const v4u(&A)[4][NA], const char* sa) {

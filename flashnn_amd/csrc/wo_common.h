@@ -176,6 +176,27 @@ __device__ __forceinline__ void convert_w4_nat(const v4u w, v4u& e0, v4u& e1, v4
 }
 
 
+// The same for fp16 operands with no shift for the odd channel: its nibble stays at bits 4..7 of each half, where
+// under the exponent of 64 a mantissa step is 1/16, so the operand is 64 + (v + 8) (the even channel's: 1024 + (v + 8)).
+__device__ __forceinline__ void convert_w4_nat_f16_2off(const v4u w, v4u& e0, v4u& e1, v4u& o0, v4u& o1) {
+    constexpr uint32_t m0 = 0x000F000Fu, c0 = 0x64006400u ^ 0x00080008u;
+    constexpr uint32_t m1 = 0x00F000F0u, c1 = 0x54005400u ^ 0x00800080u;
+    uint32_t e[8], o[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t y = __builtin_amdgcn_perm(w[q], w[q], 0x03010200u);   // bytes k0 k2 k1 k3
+        const uint32_t y2 = y >> 8;
+        e[2 * q] = (y & m0) ^ c0;
+        o[2 * q] = (y & m1) ^ c1;
+        e[2 * q + 1] = (y2 & m0) ^ c0;
+        o[2 * q + 1] = (y2 & m1) ^ c1;
+    }
+    e0 = v4u{e[0], e[1], e[2], e[3]};
+    e1 = v4u{e[4], e[5], e[6], e[7]};
+    o0 = v4u{o[0], o[1], o[2], o[3]};
+    o1 = v4u{o[4], o[5], o[6], o[7]};
+}
+
 // gemm_weight_only.hip: where the caller gave scratch and the tables are fp16 (per channel or per group of
 // 128), converts the bf16 activation rows of p to fp16 rows in the scratch, each row scaled by a power of two
 // so that every value is representable, and fills q with the same problem on those rows (q.act_unscale
