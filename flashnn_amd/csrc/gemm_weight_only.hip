@@ -1336,6 +1336,9 @@ static void launch_stream(WoArgs& p, hipStream_t st) {
     else gemm_wo_stream_kernel<WBITS, ADT, MB, false><<<grid, block, 0, st>>>(p);
 }
 
+// the decode kernels keep a copy of the activation rows in LDS up to this size
+constexpr size_t kDecodeActLdsBytes = 33 * 1024;
+
 // gemv_only: take the one-wave-per-tile kernel or nothing
 template <int WBITS, int ADT>
 static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
@@ -1349,7 +1352,7 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
     const size_t fixed = (size_t)ngroups * 8 * NH * 8 + (size_t)kDecWaves * NH * 4 * 64 * 4;
     if (fixed > 40 * 1024) return false;
     const size_t act_bytes = (size_t)p.M * (p.K + 32) * 2;
-    const bool act_lds = act_bytes <= 33 * 1024;
+    const bool act_lds = act_bytes <= kDecodeActLdsBytes;
     const int wrows = WBITS == 4 ? p.N / 2 : p.N;
     const int tiles = (wrows + 7) / 8;
     const dim3 grid(((tiles + 7) / 8) * 8), block(kDecWaves * 64);
@@ -1610,7 +1613,15 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
     if (p.group == 64 && p.M <= 8 && ADT == FNN_F16 && p.scale_dtype == FNN_F16 && (!p.zp || p.zp_dtype == FNN_F16) &&
         launch_decode<WBITS, ADT>(p, st, false))
         return;
-    if (p.M >= 2 && launch_wo_panel(p, WBITS, ADT, st)) return;
+    // One row: the decode kernels, except where they are the slower choice (measured under a captured graph,
+    // rotating weights, decode / panel kernel): rows too long for the decode kernel's LDS copy of the activations
+    // (K > 16864: int4 g128 N=8192 K=28672 54.9 / 30.7 us, N=3584 K=18944 34.8 / 21.4 us; int8 per channel 54.2 /
+    // 37.8 and 31.1 / 18.4 us), and int8 weights with per-channel tables over many channels when K / 128 is not a
+    // multiple of 32, where the decode kernel runs its guarded form (N=15360 K=5120 21.0 / 16.2 us, N=27648
+    // 33.4 / 28.3 us, N=37888 K=3584 40.3 / 30.4 us; with 4096 to 5120 channels the two are equal).
+    const bool one_row_on_panel = p.M == 1 && ((size_t)(p.K + 32) * 2 > kDecodeActLdsBytes ||
+                                               (WBITS == 8 && p.group == 0 && (p.K / 128) % 32 != 0 && p.N >= 12288));
+    if ((p.M >= 2 || one_row_on_panel) && launch_wo_panel(p, WBITS, ADT, st)) return;
     if (launch_decode<WBITS, ADT>(p, st, false)) return;
     // up to 64 activation rows per pass over the weights
     for (int m0 = 0; m0 < p.M; m0 += 64) {

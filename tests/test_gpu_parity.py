@@ -1349,6 +1349,18 @@ def test_weight_only_long_rows_within_the_lds_limit(bits, M, N, K, group):
 
 
 # ------------------------------------------------------- rmsnorm+quant -> A8W8 chain
+@pytest.mark.parametrize("bits,N,K,group,act_ty", [(4, 2048, 28672, 128, torch.bfloat16), (8, 1024, 18944, 0, torch.float16),
+                                                  (8, 1024, 18944, 128, torch.bfloat16), (4, 1024, 17408, 0, torch.float16),
+                                                  (8, 12288, 1280, 0, torch.float16), (8, 15360, 3584, 0, torch.bfloat16)])
+def test_weight_only_one_row_on_the_panel_kernel(bits, N, K, group, act_ty):
+    """One activation row where the decode kernels are the slower choice: rows longer than their LDS copy of the
+    activations holds (K > 16864), and int8 weights with per-channel tables over 12288 and more channels with
+    K / 128 not a multiple of 32."""
+    case = _wo_inputs(1, N, K, group, bits, act_ty, torch.float16, with_zp=True, with_bias=bits == 8, seed=N + K)
+    _wo_check(*case, group, bits, act_ty, cols=None if N <= 2048 else np.r_[0:64, N // 2 - 32:N // 2 + 32, N - 64:N])
+    assert _lib.last_kernel().startswith("gemm_wo_panel_kernel"), _lib.last_kernel()
+
+
 @pytest.mark.parametrize("M", [1, 32, 512, 8192])
 def test_rmsnorm_quant_gemm_chain(M):
     K = N = 8192
