@@ -1028,7 +1028,7 @@ def test_weight_only_groups_of_32_one_hot():
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("group", [0, 128])
+@pytest.mark.parametrize("group", [0, 128, 256, 1024])
 def test_weight_only_bf16_rows_through_the_conversion_pass(hip_lib, bits, group):
     """bf16 activations, fp16 tables, more than 64 rows: with scratch memory the rows become fp16 rows (scaled
     by a power of two per row) and the tiled kernel rounds every weight as the reference does - no output
