@@ -239,6 +239,20 @@ def main():
         sustained[label] = round(rate.value, 1)
     roofline["mfma_only_sustained"] = dict(sustained, unit="TOP/s")
     roofline["frac_of_sustained_random"] = round(gemm_tops / sustained["random_operand_bytes"], 4)
+    # for scale: the int8 GEMM of the image's BLAS on the same shape (torch._int_mm: int32 output, no scale
+    # epilogue), rotating operand sets like the step above
+    try:
+        Mq, Kq, Nq = primary["M"], primary["K"], primary["N"]
+        gq = torch.Generator(device=dev).manual_seed(5)
+        a_sets = [torch.randint(-128, 128, (Mq, Kq), dtype=torch.int8, device=dev, generator=gq) for _ in range(6)]
+        b_sets = [torch.randint(-128, 128, (Nq, Kq), dtype=torch.int8, device=dev, generator=gq) for _ in range(6)]
+        ms_blas, _ = _timed(lambda i: torch._int_mm(a_sets[i % 6], b_sets[i % 6].t()), args.steps, torch)
+        roofline["blas_int8_gemm"] = {"fn": "torch._int_mm(a, b.t()), int32 out, no epilogue", "us": round(ms_blas * 1e3, 2),
+                                      "TOPs": round(primary["ops"] / (ms_blas * 1e-3) / 1e12, 1)}
+        del a_sets, b_sets
+    except Exception as exc:          # (a torch build without the int8 GEMM: the figure is context, not part of the metric)
+        roofline["blas_int8_gemm"] = {"fn": "torch._int_mm", "error": str(exc)[:80]}
+    torch.cuda.empty_cache()
     # what the memory side delivers without arithmetic: the tile's copy pattern alone (direct-to-LDS copies of
     # 448 rows x 128 bytes per slab, one workgroup per CU, over the QKV operands' row length), and a stream of
     # the decode GEMV's request pattern over the bytes of its weights
