@@ -977,7 +977,15 @@ static void dispatch_band(A8W8Args& p, hipStream_t st, bool aligned, int force_b
     // N=1920 K=13312 25.3 / 17.4; M=128 N=1024 K=4096 10.1 / 8.7; from N = 3584 on the tiled kernel wins:
     // M=128 N=3584 K=18944 30.5 / 34.5, N=K=8192 23.3 / 24.7).  The same bits either way.
     const bool narrow = p.M <= kA8PanelRowsNarrow && p.N <= 2048 && p.K >= 4096;
-    if (force_bm == 0 && (p.M <= 64 || narrow) && launch_a8w8_skinny(p, MODE, st)) return;
+    // 17 .. 64 rows over more than 16384 and fewer than 32768 channels: the few-row kernel's workgroups own 64
+    // channels, so there are between 257 and 511 of them - one round of the 256 CUs and a part of a second -
+    // where the tiled kernel has one round of 64x128 tiles (under a captured graph, rotating weights, bf16 out,
+    // M=64, few-row / tiled: N=16384 K=4096 17.8 / 20.7 us, N=16640 26.6 / 21.1, N=20480 27.7 / 22.6, N=24576
+    // 28.8 / 24.6, N=28672 30.0 / 29.8 on one box and 30.4 / 25.4 on another; N=24576 K=8192 55.3 / 45.1;
+    // N=17792 K=13312 86.0 / 60.0; M=33 alike; M=24: N=24576 K=4096 30.4 / 25.3, N=17792 K=13312 60.9 / 55.9,
+    // elsewhere within a few percent, the tiled kernel never behind)
+    const bool between_rounds = fast && p.M > 16 && p.M <= 64 && p.N > 16384 && p.N < 32768;
+    if (force_bm == 0 && !between_rounds && (p.M <= 64 || narrow) && launch_a8w8_skinny(p, MODE, st)) return;
     if (fast && ws.ptr) {
         if (ws.force_kparts > 1) {          // (the entry point has checked tile, parts and workspace size)
             const int chunk = split_chunk_slabs((p.K + 127) / 128, ws.force_kparts) * 128;

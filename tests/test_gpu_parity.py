@@ -206,6 +206,18 @@ def test_a8w8_few_rows_bit_exact(M, nk):
                           O.gemm_a8w8_epilogue_fp32(want, O.to_np(ar), O.to_np(ac), _tag(out_ty)))
 
 
+@pytest.mark.parametrize("M,N,K,kernel", [(33, 16640, 1024, "ring"), (64, 17792, 512, "ring"), (48, 24576, 1056, "ring"),
+                                          (17, 28672, 1024, "ring"), (64, 16384, 1024, "panel"), (16, 17792, 1024, "panel"),
+                                          (64, 32768, 1024, "panel")])
+def test_a8w8_between_one_and_two_rounds_of_few_row_workgroups(M, N, K, kernel):
+    """17 .. 64 rows over 16385 .. 32767 channels run on the tiled kernel (one round of 64x128 tiles) instead of
+    257 .. 511 workgroups of the few-row kernel; the neighbouring shapes stay where they were.  Same bits."""
+    a, b = _rand_i8((M, K), 61), _rand_i8((N, K), 62)
+    acc = flashnn_amd.launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+    assert _lib.last_kernel().startswith(f"gemm_a8w8_{kernel}_kernel"), _lib.last_kernel()
+    assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
+
+
 def test_a8w8_saturation_and_identity():
     a = torch.full((256, 4096), -128, dtype=torch.int8)
     acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), a.to(DEV))
