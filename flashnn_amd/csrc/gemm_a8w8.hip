@@ -810,6 +810,13 @@ static TileChoice choose_tile(int64_t M, int64_t N) {
     // 0.74 at M=K=N=8192; 128x128 0.71 to 0.76; 64x128 0.64 to 0.67 (a 64x128 tile takes 0.55 to 0.6 of
     // the time of a 128x128 one, so it pays where it doubles the workgroups without adding a round).
     // The 128x128 figure is that of one workgroup per CU; the pairs are priced below.
+    // Up to 128 rows over 32769 .. 38912 channels: 257 .. 304 tiles of 128 columns, of which the pricing below
+    // makes pairs - fewer than a fifth of the CUs then run two workgroups and set the time while the others
+    // stream their weights at the rate of one.  One round of 256x192 tiles (the rows beyond M copy the last
+    // row again: L1 hits) is faster: M=128 N=35584 K=13312 116 against 144 us, M=65 110 / 128; N=36864 K=8192
+    // 78 / 90 and 75 / 81; N=37888 K=3584 38 / 43 and 39 / 37; N=33792 K=4096 44 / 49 and 44 / 45.  From 320
+    // tiles on the pairs are level again or ahead (N=40960 K=4096 M=128 49 / 51, N=49152 53 / 52).
+    if (M <= 128 && N > 32768 && N <= 38912) return TileChoice{256, 192};
     double best = 1e300;
     TileChoice c{128, 128};
     for (const auto& t : cand) {
@@ -941,7 +948,17 @@ static SplitPlan plan_split(int64_t M, int64_t N, int64_t K, size_t ws_bytes) {
     for (int q = 2; q <= 8; ++q) {
         const int64_t units = t128 * q;
         const int slabs = split_chunk_slabs(KT, q);
-        if ((units <= 256 && slabs >= 8) || (units <= 512 && slabs >= 40)) parts = q;
+        // More than one round of units (two per CU on some or all CUs) pays with two to four tile rows: their
+        // tiles stream the weights with little reuse, and a second workgroup on the CU keeps that stream going.
+        // With five and more rows the unsplit tiles share their weights through the L2 and are level or ahead,
+        // and with a single row most CUs would run one unit and the rest two, no shorter than before (under a
+        // captured graph, rotating weights, two parts / unsplit: M=256 N=8960 K=13312 52 / 64 us, M=384 N=8192
+        // K=14784 67 / 88, M=512 N=8192 K=28672 125 / 134; but M=640 N=3584 K=18944 66 / 61, M=764 N=4096
+        // K=11008 42.6 / 37.7, M=896 N=3584 K=18944 70 / 59, M=1024 N=4096 K=11008 48 / 43, M=1280 N=1920
+        // K=13312 48.5 / 42.3, M=128 N=17792 K=13312 81 / 72).
+        const int64_t mrows = (M + 127) / 128;
+        const bool pairs_pay = mrows >= 2 && mrows <= 4;
+        if ((units <= 256 && slabs >= 8) || (units <= 512 && slabs >= 40 && pairs_pay)) parts = q;
     }
     // (a workspace too small for the best count takes the largest one it holds)
     for (; parts >= 2; --parts) {

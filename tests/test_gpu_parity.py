@@ -362,7 +362,7 @@ def test_a8w8_split_k_bit_exact(hip_lib, plan, mnk):
 
 
 @pytest.mark.parametrize("mnk", [(256, 4096, 8192), (128, 2304, 16384), (384, 1920, 13312), (100, 1000, 9248), (2048, 4096, 4096),
-                                 (1024, 1920, 13312), (640, 3584, 18944), (256, 4096, 6144)])
+                                 (1024, 1920, 13312), (512, 3584, 18944), (256, 8960, 13312), (256, 4096, 6144)])
 def test_a8w8_workspace_entry_matches_plain(hip_lib, mnk):
     """fnn_gemm_a8w8_ws: shapes the library splits (and one it does not) against fnn_gemm_a8w8, bit for bit,
     through the operator too (its launcher keeps a workspace per stream); a workspace smaller than the

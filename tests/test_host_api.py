@@ -247,7 +247,8 @@ def test_workspace_entries_reject_bad_arguments(hip_lib):
     assert f(256, 4096, 4096) == 0 and f(1024, 4096, 4096) == 0
     assert f(256, 4096, 8192) == 4096 + 64 * 4 * 65536
     assert f(1024, 1920, 13312) == 4096 + 120 * 2 * 65536        # one unit per CU
-    assert f(764, 3584, 18944) == 4096 + 168 * 3 * 65536         # a long K: two per CU
+    assert f(384, 8192, 14784) == 4096 + 192 * 2 * 65536         # a long K and few tile rows: two units per CU
+    assert f(764, 3584, 18944) == 0                              # six tile rows share the weights: unsplit
     assert all(f(M, N, K) <= (32 << 20) + 4096 for M in (65, 100, 128, 500, 1000, 3000) for N in (128, 1000, 4096, 20000)
                for K in (6144, 8192, 16384, 32768))
 
