@@ -218,6 +218,18 @@ def test_a8w8_between_one_and_two_rounds_of_few_row_workgroups(M, N, K, kernel):
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
 
 
+@pytest.mark.parametrize("M,N,tile", [(100, 33024, "256,192"), (128, 38912, "256,192"), (65, 32768, "128,128"), (129, 33024, None)])
+def test_a8w8_few_rows_over_a_little_more_than_one_round_of_tiles(M, N, tile):
+    """Up to 128 rows over 32769 .. 38912 channels take one round of 256x192 tiles (rows beyond M are padding)
+    instead of 257 .. 304 tiles of 128 columns in pairs; the shapes next to that range keep their tiles."""
+    K = 512
+    a, b = _rand_i8((M, K), 71), _rand_i8((N, K), 72)
+    acc = flashnn_amd.launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+    if tile:
+        assert _lib.last_kernel() == f"gemm_a8w8_ring_kernel<{tile},4>", _lib.last_kernel()
+    assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
+
+
 def test_a8w8_saturation_and_identity():
     a = torch.full((256, 4096), -128, dtype=torch.int8)
     acc = launchers.hip_gemm_a8w8_int32(a.to(DEV), a.to(DEV))
