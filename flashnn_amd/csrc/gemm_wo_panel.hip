@@ -545,8 +545,20 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
 // share the weights through its L2).
 // Measured on A16W8, N=4096: M=64 takes 12.6 us with 32 rows per workgroup and two passes, 27.5 us with 16
 // rows and four passes, 22.1 us with 64 rows and one pass of 64 workgroups.
-static int choose_rows(int wrows, int64_t M, int KT, int* mb_out) {
+// What the model does not see: int8 weights, more than 16 activation rows, and a little more than one or two rounds
+// of 64-row workgroups (257 .. 384 or 513 .. 640 of them).  Passes of 32 activation rows with 64-row workgroups, whose
+// LDS lets two share a CU, are then faster than one pass of 64 rows with one workgroup per CU, and than 32-row
+// workgroups (under a captured graph, rotating weights, bf16 rows, model's choice / 64-row workgroups with 32
+// activation rows a pass: N=17792 K=4096 M=64 45.3 / 35.1 us, M=32 36.0 / 27.7; N=22016 K=4096 46.0 / 37.3 and
+// 37.2 / 28.2; N=20480 K=8192 80.8 / 70.0 and 58.0 / 51.6; N=37888 K=3584 M=64 65.5 / 58.6; at 432 and 448
+// workgroups, N=27648 and 28672, the single pass is ahead by 4 to 8 %, and so it is everywhere with int4 weights, whose
+// conversion a second pass repeats).
+static int choose_rows(int wrows, int64_t M, int KT, int* mb_out, int wbits) {
     const int need = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    if (wbits == 8 && M > 16 && wrows % 64 == 0) {
+        const int wg4 = wrows / 64;
+        if ((wg4 > 256 && wg4 <= 384) || (wg4 > 512 && wg4 <= 640)) { *mb_out = 2; return 4; }
+    }
     static const double per_iter[5] = {0, 1.0, 1.2, 0, 1.8};
     int rt = 0;
     double best = 0.0;
@@ -583,7 +595,7 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
         if (!tables16) return false;
     }
     int mb = 1;
-    const int rt = choose_rows(wrows, p.M, (int)((p.K + 127) / 128), &mb);
+    const int rt = choose_rows(wrows, p.M, (int)((p.K + 127) / 128), &mb, WBITS);
     const int tiles = wrows / (16 * rt);
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);

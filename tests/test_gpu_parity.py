@@ -980,6 +980,16 @@ def test_weight_only_large_m_on_narrow_matrices(bits, group, M, N, K):
     assert _lib.last_kernel().startswith("gemm_wo_panel_kernel" if K >= 1024 else "gemm_wo_tile_kernel"), _lib.last_kernel()
 
 
+@pytest.mark.parametrize("M,N,want", [(64, 17792, "<8,2,4>"), (24, 22016, "<8,2,4>"), (48, 37888, "<8,2,4>"), (64, 16384, "<8,4,4>"),
+                                      (64, 27648, "<8,4,4>"), (16, 17792, "<8,1,4>")])
+def test_a16w8_a_little_more_than_one_round_of_64_row_workgroups(M, N, want):
+    """int8 weights, more than 16 rows, 257 .. 384 or 513 .. 640 workgroups of 64 weight rows: passes of 32 activation
+    rows (two workgroups share a CU) instead of one pass of 64; the neighbouring shapes keep the model's choice."""
+    case = _wo_inputs(M, N, 1024, 128, 8, torch.bfloat16, torch.float16, with_zp=True, with_bias=False, seed=M + N)
+    _wo_check(*case, 128, 8, torch.bfloat16, cols=np.r_[0:64, N // 2 - 32:N // 2 + 32, N - 64:N])
+    assert _lib.last_kernel() == "gemm_wo_panel_kernel" + want, _lib.last_kernel()
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("group", [64, 256, 512])
 @pytest.mark.parametrize("M,N,K", [(5, 1024, 1024), (16, 4096, 2048), (40, 1056, 2560), (64, 8192, 1024), (100, 2048, 1536),
