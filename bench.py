@@ -17,6 +17,7 @@ Also measured in the same run and reported in the same JSON line:
                   c4     A16W4 group-128 at K=8192 N=28672, M in {1, 4, 16, 64, 256} (M=1 always runs)
                   c5     RMSNormDquant -> A8W8 at K=N=8192, M in {1, 32, 512, 8192}
                   g64    A16W4 group-64 at the reference test's shape M=3 N=1024 K=4096
+                  other  four shapes off the configured list whose kernel choice was settled by timing alternatives
                   splitk A8W8 shapes whose K the library splits, against the unsplit kernel
                   rows   the row kernels on their own;  moe  the fused mixture-of-experts GEMMs
   cpu_baseline  the reference's torch CPU path (oracle/torch_path.py) on the host cores
@@ -40,7 +41,7 @@ if ROOT not in sys.path:
 PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA, published (5.0 POP/s)
 PEAK_F16_TFLOPS = 2500.0    # dense bf16 / fp16 MFMA, published (2.5 PFLOP/s)
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published (8 TB/s)
-ALL_LEGS = ("c1", "c2", "c3", "c4", "c5", "g64", "splitk", "rows", "moe")
+ALL_LEGS = ("c1", "c2", "c3", "c4", "c5", "g64", "other", "splitk", "rows", "moe")
 
 
 def _timed(fn, iters, torch, preroll_s=0.04):
@@ -452,6 +453,50 @@ def main():
             secondary.append(_entry(f"g64 a16w{bits} group 64 M={Mg} K={Kg} N={Ng} fp16 (the reference test's shape)", ms,
                                     "hbm", Ng * Kg * bits / 8 + 4.0 * (Kg // 64) * Ng + 2.0 * Mg * Kg + 2.0 * Mg * Ng, kern))
             del qgs, sgs, zgs
+        torch.cuda.empty_cache()
+
+    # ----------- other: shapes off the configured list whose kernel choice was settled by timing it against forced alternatives
+    if "other" in legs:
+        # A8W8, 64 rows over 24576 channels (between one and two rounds of the few-row kernel's workgroups)
+        Mo, No, Ko = 64, 24576, 8192
+        xq = workloads.activations(Mo, Ko, torch.float16, seed=80, outlier_frac=0.01).to(dev)
+        qo = torch.empty(Mo, Ko, dtype=torch.int8, device=dev)
+        so = torch.empty(Mo, dtype=torch.float16, device=dev)
+        launchers.hip_dynamic_quantize(qo, xq, so)
+        wo_cpu, wos_cpu = workloads.int8_weights(No, Ko, seed=81)
+        wo = rotating(wo_cpu.to(dev), total_bytes=600e6, at_least=3)
+        n = len(wo)
+        wos = wos_cpu.to(dev)
+        oo = torch.empty(Mo, No, dtype=torch.bfloat16, device=dev)
+        f = lambda i: launchers.hip_gemm_a8w8_forward(oo, qo, wo[i % n], so, wos)
+        kern = kernel_of(f)
+        ms, _ = _timed(f, iters, torch)
+        secondary.append(_entry(f"other a8w8 M={Mo} K={Ko} N={No} bf16", ms, "hbm", float(No) * Ko + Mo * Ko + 2.0 * Mo * No, kern))
+        # A16W8 per channel, 64 rows over 22016 channels (a little more than one round of 64-row workgroups)
+        s8 = wos_cpu[:22016].half().to(dev)
+        act = workloads.activations(64, 4096, torch.float16, seed=82).to(dev)
+        o8 = torch.empty(64, 22016, dtype=torch.float16, device=dev)
+        w8v = [w[:22016, :4096].contiguous() for w in wo]
+        f = lambda i: launchers.hip_gemm_a16w8_forward(o8, act, w8v[i % n], s8)
+        kern = kernel_of(f)
+        ms, _ = _timed(f, iters, torch)
+        secondary.append(_entry("other a16w8 M=64 K=4096 N=22016 fp16", ms, "hbm", 22016.0 * 4096 + 2.0 * 64 * (4096 + 22016), kern))
+        del wo, w8v
+        torch.cuda.empty_cache()
+        # A16W4 g128, one row of 28672 values (beyond the decode kernels' LDS copy); groups of 64 at 64 rows
+        for (Mv, Nv, Kv, gv) in ((1, 8192, 28672, 128), (64, 11008, 4096, 64)):
+            qv, sv, zv, _, _ = workloads.int4_group_weights(Nv, Kv, gv, seed=83)
+            qvs = rotating(qv.to(dev), total_bytes=600e6, at_least=3)
+            n = len(qvs)
+            svd, zvd = sv.to(dev), zv.to(dev)
+            act = workloads.activations(Mv, Kv, torch.bfloat16, seed=84).to(dev)
+            ov = torch.empty(Mv, Nv, dtype=torch.bfloat16, device=dev)
+            f = lambda i: launchers.hip_gemm_a16w4_forward(ov, act, qvs[i % n], svd, None, zvd)
+            kern = kernel_of(f)
+            ms, _ = _timed(f, iters, torch)
+            secondary.append(_entry(f"other a16w4 g{gv} M={Mv} K={Kv} N={Nv} bf16", ms, "hbm",
+                                    Nv * Kv / 2.0 + 4.0 * (Kv // gv) * Nv + 2.0 * Mv * (Kv + Nv), kern))
+            del qvs
         torch.cuda.empty_cache()
 
     # --------------------- splitk: A8W8 shapes whose K the library splits over workgroups, and the unsplit kernel
