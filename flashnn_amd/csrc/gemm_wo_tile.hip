@@ -327,6 +327,35 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
         // both waves of the SIMD cross the same barrier every slab.  The weight stage of slab j is free
         // from barrier j on (its operands were formed during slab j - 1), so the weights are copied three
         // slabs ahead into three stages, the tables two ahead.
+        // Zero points that are whole numbers (the usual case) let the offset of the conversion and the zero point
+        // go in one subtraction, x - (offset + zp): both forms are exact then, so the bits are the same and a
+        // third of the rounding step's instructions is saved.  Whether all zero points of the tile's channels are
+        // whole (and small enough for offset + zp to be exact in fp16) is found once per workgroup, before the
+        // first copy is issued; if not, the two-step form runs.
+        bool whole_zp = false;
+        if constexpr (REFQ == 2) {
+            int bad = 0;
+            auto check = [&](uint32_t pair) {
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float z = f16_bits_to_f32((pair >> (16 * e)) & 0xFFFFu);
+                    bad |= !(z == rintf(z) && fabsf(z) <= 512.f);
+                }
+            };
+            if constexpr (G128) {
+                const int pieces = (KT >> p.gshift) * 16;        // 16-byte pieces of the tile's 128 channels, row by row
+                for (int e = threadIdx.x; e < pieces; e += 512) {
+                    const v4u v = *(const v4u*)((const char*)p.zp + ((int64_t)(e >> 4) * p.N + n0) * 2 + (e & 15) * 16);
+                    check(v[0]); check(v[1]); check(v[2]); check(v[3]);
+                }
+            } else {
+                const uint16_t* const z16 = (const uint16_t*)p.zp + n0;
+                if (threadIdx.x < BN / 2) check((uint32_t)z16[2 * threadIdx.x] | ((uint32_t)z16[2 * threadIdx.x + 1] << 16));
+            }
+            whole_zp = !__syncthreads_or(bad);
+        }
+        auto run = [&](auto merged_tag) {
+        constexpr bool MERGED = decltype(merged_tag)::value;
         v4u A0[4][NA], A1[4][NA];
         auto dequant_slab = [&](v4u(&A)[4][NA], const char* sw, const char* stg) {
             if constexpr (G128) {
@@ -350,11 +379,17 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
                         convert_w8<ADT>(w, A[2 * h][f], A[2 * h + 1][f]);
                 }
             if constexpr (ROUNDQ) {
+                v2h sub[NA];
+#pragma unroll
+                for (int a = 0; a < NA; ++a) {
+                    sub[a] = WBITS == 4 && (a % NH) == 1 ? rq_c_odd : rq_c;
+                    if constexpr (MERGED) sub[a] = sub[a] + rq_z[a];
+                }
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
                     for (int a = 0; a < NA; ++a)
-                        A[ks][a] = ref_dq_f16<REFQ == 2>(A[ks][a], WBITS == 4 && (a % NH) == 1 ? rq_c_odd : rq_c, rq_z[a], rq_s[a]);
+                        A[ks][a] = ref_dq_f16<REFQ == 2 && !MERGED>(A[ks][a], sub[a], rq_z[a], rq_s[a]);
             }
         };
         auto mfma_slab = [&](const v4u(&A)[4][NA], const char* sa) {
@@ -432,6 +467,13 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
             FNN_RQ_ITER(A1, A0, sa1, sw1, st1, sa0, sw0, st2, j + 3);
         }
 #undef FNN_RQ_ITER
+        };
+        if constexpr (REFQ == 2) {
+            if (whole_zp) run(std::true_type{});
+            else run(std::false_type{});
+        } else {
+            run(std::false_type{});
+        }
     } else {
 #define FNN_TILE_ITER(CA, CW, CT, FA, FW, FT, J)                          \
     do {                                                                  \

@@ -1116,6 +1116,37 @@ def test_weight_only_bf16_rows_through_the_conversion_pass(hip_lib, bits, group)
         assert torch.equal(again, plain if "rounding" not in kernel else out)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("group", [0, 128])
+@pytest.mark.parametrize("kind", ["whole", "quarter", "one_fraction", "large"])
+def test_weight_only_tiled_zero_points_whole_or_not(bits, group, kind):
+    """The tiled kernel's per-weight rounding takes offset and zero point in one subtraction where every zero point of
+    the tile is a whole number of moderate size, and in two otherwise; both must be the reference's rounding: whole
+    zero points, quarters, a single fractional one in one tile, and whole ones too large for the short form."""
+    M, N, K = 200, 8320, 1024
+    act, w, qw, scale, zp, bias = _wo_inputs(M, N, K, group, bits, torch.float16, torch.float16, True, False, seed=321)
+    if kind == "quarter":
+        zp = (zp.float() + 0.25).half()
+    elif kind == "one_fraction":
+        zp = zp.clone()
+        zp[..., 4200] = 1.5
+    elif kind == "large":
+        zp = zp.clone()
+        zp[..., 100] = 600.0
+    cols = np.r_[0:256, 4096:4352, N - 64:N]
+    if kind != "large":
+        _wo_check(act, w, qw, scale, zp, bias, group, bits, torch.float16, strict=True, cols=cols)
+    else:
+        # (a zero point of 600 makes outputs of the size of 600 * scale * sum(a): the oracle's own rounding is then
+        # further from the mathematical value than _wo_check's closeness bound allows, so only the tolerance is held)
+        d = lambda t: t.to(DEV)
+        got = flashnn_amd.GemmWeightOnly(torch.float16)(d(act), d(qw), d(scale), None, d(zp)).float().cpu().numpy()[:, cols]
+        want = O.weight_only_gemm(O.to_np(act), w[cols].numpy(), O.to_np(scale[..., cols]), O.to_np(zp[..., cols]), None,
+                                  O.F16, O.F16, group, bits == 4)
+        assert (np.abs(got - want) <= ATOL + RTOL * np.abs(want)).all()
+    assert _lib.last_kernel().startswith("gemm_wo_tile_kernel(per-weight rounding)"), _lib.last_kernel()
+
+
 def test_weight_only_tiled_one_hot():
     """One-hot activation rows pick single weight columns exactly: the k order inside a slab, the row and
     channel mapping of the tiled kernel (int4, group 128; 130 tiles)."""
