@@ -36,12 +36,13 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
 // REFQ (1, or 2 with zero points; fp16 activations, fp16 scales and zero points, per channel or per group of
-// 128): every weight is dequantised and rounded to fp16 as the reference's torch path does before the dot
+// 128 .. values): every weight is dequantised and rounded to fp16 as the reference's torch path does before the dot
 // product, (q - zp) * s with both operations rounded (ref_dq_f16 in wo_common.h; flashnn/quant_gemm.py:14-36).
 // The accumulators then run over all of K: no MFMAs against ones, no fold per slab, no second accumulator
 // set, and the result differs from the reference's only by the order of the fp32 additions.  bf16
 // activations reach this form through the conversion pass of gemm_weight_only.hip (rows scaled by a power
-// of two, p.act_unscale undoes it).
+// of two, p.act_unscale undoes it).  bf16 activations with bf16 tables: the same with both roundings to bf16,
+// worked in fp32 (ref_dq_bf16 in wo_common.h), the operands meeting in the bf16 MFMA.
 // MOE (per-channel tables, no REFQ): the mixture-of-experts form for many routed rows per expert
 // (flashnn/triton_kernels/fused_moe_a16w4.py:50-206).  The M dimension is the list of sorted routed rows,
 // padded per expert to blocks of q.block_m rows, a multiple of BM: tile row r multiplies activation row
@@ -55,7 +56,11 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     // tables of any type: the operands are the converted integers, the activation sums come from MFMAs
     // against ones and scale and zero point are applied once at the end.
     constexpr bool ROUNDQ = REFQ == 1 || REFQ == 2;
-    static_assert(!ROUNDQ || (ADT == FNN_F16 && SDT == FNN_F16), "reference rounding: fp16 activations and tables");
+    static_assert(!ROUNDQ || (ADT == SDT && (ADT == FNN_F16 || ADT == FNN_BF16)), "reference rounding: activations and tables of one 16-bit type");
+    // bf16 activations with bf16 tables: the weights are rounded to bf16 as the reference's torch path rounds them
+    // (in fp32 arithmetic, ref_dq_bf16 in wo_common.h) and meet the activations in the bf16 MFMA
+    constexpr bool RQBF = ROUNDQ && ADT == FNN_BF16;
+    constexpr float kWholeZpMax = RQBF ? 128.f : 512.f;    // whole zero points up to here take the one-step form
     static_assert(REFQ != 3 || !G128, "the pipeline without rounding: per-channel tables");
     // The gathered form takes per-channel tables (pipelined, REFQ = 3) or tables per group of 128 in the
     // layout of the reference's MoE launcher, [expert][channel][group] (fp32 scaling per slab, 128-row tiles):
@@ -220,12 +225,19 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
     const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
     const v2h rq_c_odd = pair_of_f16_bits(0x5480u);                      // 72: .. to the odd channel of an int4 row
     v2h rq_s[NA], rq_z[NA];
+    float bq_s[NA], bq_z[NA];                                            // the same as fp32 numbers (bf16 tables)
     if constexpr (ROUNDQ && !G128) {
 #pragma unroll
         for (int a = 0; a < NA; ++a) {
             const int n = n0 + wn * WTN + (a / NH) * 16 * NH + NH * row16 + (a % NH);
-            rq_s[a] = pair_of_f16_bits(((const uint16_t*)p.scale)[n]);
-            rq_z[a] = pair_of_f16_bits(p.zp ? ((const uint16_t*)p.zp)[n] : 0u);
+            const uint32_t sb = ((const uint16_t*)p.scale)[n], zb = p.zp ? ((const uint16_t*)p.zp)[n] : 0u;
+            if constexpr (RQBF) {
+                bq_s[a] = bf16_bits_to_f32(sb);
+                bq_z[a] = bf16_bits_to_f32(zb);
+            } else {
+                rq_s[a] = pair_of_f16_bits(sb);
+                rq_z[a] = pair_of_f16_bits(zb);
+            }
         }
     }
 
@@ -338,8 +350,8 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
             auto check = [&](uint32_t pair) {
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    const float z = f16_bits_to_f32((pair >> (16 * e)) & 0xFFFFu);
-                    bad |= !(z == rintf(z) && fabsf(z) <= 512.f);
+                    const float z = bits_to_f32<SDT>((pair >> (16 * e)) & 0xFFFFu);
+                    bad |= !(z == rintf(z) && fabsf(z) <= kWholeZpMax);
                 }
             };
             if constexpr (G128) {
@@ -358,6 +370,53 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
         constexpr bool MERGED = decltype(merged_tag)::value;
         v4u A0[4][NA], A1[4][NA];
         auto dequant_slab = [&](v4u(&A)[4][NA], const char* sw, const char* stg) {
+            if constexpr (RQBF) {
+                constexpr float off = WBITS == 4 ? 8.f : 128.f;
+                constexpr bool ONE_STEP = REFQ == 1 || MERGED;          // (no zero points: zeros)
+                float s_[NA], z_[NA], c_[NA];
+#pragma unroll
+                for (int a = 0; a < NA; ++a) {
+                    if constexpr (G128) {
+                        const int ch = wn * WTN + (a / NH) * 16 * NH + NH * row16 + (a % NH);
+                        s_[a] = bf16_bits_to_f32(*(const uint16_t*)(stg + ch * 2));
+                        z_[a] = REFQ == 2 ? bf16_bits_to_f32(*(const uint16_t*)(stg + 256 + ch * 2)) : 0.f;
+                    } else {
+                        s_[a] = bq_s[a];
+                        z_[a] = bq_z[a];
+                    }
+                    c_[a] = -(off + z_[a]) * s_[a];
+                }
+                auto dq = [&](float u0, float u1, int a) {
+                    if constexpr (ONE_STEP) return ref_dq_bf16_merged(u0, u1, s_[a], c_[a]);
+                    else return ref_dq_bf16(u0, u1, off, z_[a], s_[a]);
+                };
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int f = 0; f < NF; ++f) {
+                        const v4u w = *(const v4u*)(sw + w_rd[h] + f * 16 * 128);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {      // 4 k of the row: operand 2 h + (q >> 1), registers 2 (q & 1), + 1
+                            if constexpr (WBITS == 4) {
+                                const uint32_t x = w[q] ^ 0x88888888u;      // two's complement -> offset by 8
+                                float fe[4], fo[4];
+                                bytes_to_f32(x & 0x0F0F0F0Fu, fe);
+                                bytes_to_f32((x >> 4) & 0x0F0F0F0Fu, fo);
+#pragma unroll
+                                for (int i = 0; i < 2; ++i) {
+                                    A[2 * h + (q >> 1)][2 * f][2 * (q & 1) + i] = dq(fe[2 * i], fe[2 * i + 1], 2 * f);
+                                    A[2 * h + (q >> 1)][2 * f + 1][2 * (q & 1) + i] = dq(fo[2 * i], fo[2 * i + 1], 2 * f + 1);
+                                }
+                            } else {
+                                float fb[4];
+                                bytes_to_f32(w[q] ^ 0x80808080u, fb);
+#pragma unroll
+                                for (int i = 0; i < 2; ++i) A[2 * h + (q >> 1)][f][2 * (q & 1) + i] = dq(fb[2 * i], fb[2 * i + 1], f);
+                            }
+                        }
+                    }
+                return;
+            }
             if constexpr (G128) {
 #pragma unroll
                 for (int a = 0; a < NA; ++a) {
@@ -417,7 +476,7 @@ __global__ __launch_bounds__(512) void gemm_wo_tile_kernel(const WoArgs p, const
 #pragma unroll
                 for (int q = 0; q < 4 * (NA + (ROUNDQ ? 0 : 1)); ++q) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, ROUNDQ ? 2 : 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, RQBF ? (BM == 256 ? 3 : 6) : ROUNDQ ? 2 : 1, 0);
                 }
             }
         };
@@ -614,8 +673,9 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
     const int tiles = tiles_m * (p.N / 128);
     const dim3 grid(((tiles + 7) / 8) * 8);   // (workgroups beyond the last tile return at once)
     // fp16 activations with fp16 tables: every weight rounded as the reference rounds it
-    const bool refq = ADT == FNN_F16 && p.scale_dtype == FNN_F16 && (!p.zp || p.zp_dtype == FNN_F16) &&
-                      (p.group != 0 || ((uintptr_t)p.scale % 2) == 0);
+    // .. and bf16 activations with bf16 tables
+    const bool refq = p.scale_dtype == ADT && (!p.zp || p.zp_dtype == ADT) &&
+                      (p.group != 0 || (((uintptr_t)p.scale % 2) == 0 && (!p.zp || ((uintptr_t)p.zp % 2) == 0)));
     note_kernel(refq ? "gemm_wo_tile_kernel(per-weight rounding)" : "gemm_wo_tile_kernel", WBITS, bm, 128);
 #define FNN_TILE(G, SDTV, RQ)                                                                            \
     do {                                                                                                 \
@@ -627,12 +687,10 @@ static bool launch_tile_t(WoArgs& p, hipStream_t st) {
         }                                                                                                \
         gemm_wo_tile_kernel<WBITS, ADT, G, SDTV, 128, RQ><<<grid, dim3(512), 0, st>>>(p, tiles_m, tiles, MoeArgs{}); \
     } while (0)
-    if constexpr (ADT == FNN_F16) {
-        if (refq) {
-            if (p.group != 0) { if (p.zp) FNN_TILE(true, FNN_F16, 2); else FNN_TILE(true, FNN_F16, 1); }
-            else { if (p.zp) FNN_TILE(false, FNN_F16, 2); else FNN_TILE(false, FNN_F16, 1); }
-            return true;
-        }
+    if (refq) {
+        if (p.group != 0) { if (p.zp) FNN_TILE(true, ADT, 2); else FNN_TILE(true, ADT, 1); }
+        else { if (p.zp) FNN_TILE(false, ADT, 2); else FNN_TILE(false, ADT, 1); }
+        return true;
     }
     if (p.group != 0) {
         if (p.scale_dtype == FNN_F16) FNN_TILE(true, FNN_F16, 0);

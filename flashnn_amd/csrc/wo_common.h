@@ -124,6 +124,35 @@ __device__ __forceinline__ v4u ref_dq_f16(v4u x, const v2h coff, const v2h zp, c
     return v4u{ref_dq_f16<ZP>(x[0], coff, zp, s), ref_dq_f16<ZP>(x[1], coff, zp, s), ref_dq_f16<ZP>(x[2], coff, zp, s),
                ref_dq_f16<ZP>(x[3], coff, zp, s)};
 }
+// The same for bf16 scales (the reference's torch path with bf16 tables): there is no packed bf16 arithmetic,
+// so the two operations run in fp32 on the weight as a small whole number u = off + q (off: 8 for int4, 128 for
+// int8) and v_cvt_pk_bf16_f32 rounds a pair to nearest even.
+// Merged form, for whole zero points of at most 128: u * s - (off + zp) * s in one fma.  u * s (8 x 8 bits) and
+// (off + zp) * s (9 x 8 bits) are exact in fp32, so the fma returns (q - zp) * s exactly (17 bits), and q - zp is
+// a bf16 number: the one rounding of the pack is the reference's second rounding and its first changes nothing.
+__device__ __forceinline__ uint32_t ref_dq_bf16_merged(float u0, float u1, float s, float neg_off_zp_s) {
+    const v2f r = {__builtin_fmaf(u0, s, neg_off_zp_s), __builtin_fmaf(u1, s, neg_off_zp_s)};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(r, v2bf));
+}
+// Two-step form, any zero point: (u - off) - zp is the fp32 rounding of q - zp (exact unless zp is below 2^-16 q,
+// where the value is nowhere near a bf16 rounding boundary), rounded to bf16; times s (8 x 8 bits: exact), rounded.
+__device__ __forceinline__ uint32_t ref_dq_bf16(float u0, float u1, float off, float zp, float s) {
+#pragma clang fp contract(off)
+    const v2f d = {(u0 - off) - zp, (u1 - off) - zp};
+    const uint32_t db = __builtin_bit_cast(uint32_t, __builtin_convertvector(d, v2bf));
+    const v2f r = {__uint_as_float(db << 16) * s, __uint_as_float(db & 0xFFFF0000u) * s};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(r, v2bf));
+}
+// The four bytes of x as fp32 (v_cvt_f32_ubyte0..3; x passes through an empty asm so that masks applied before
+// are not folded into one bit-field extract per byte)
+__device__ __forceinline__ void bytes_to_f32(uint32_t x, float (&f)[4]) {
+    asm("" : "+v"(x));
+    f[0] = (float)(x & 0xFFu);
+    f[1] = (float)((x >> 8) & 0xFFu);
+    f[2] = (float)((x >> 16) & 0xFFu);
+    f[3] = (float)(x >> 24);
+}
+
 constexpr int FNN_I8 = 3;   // type code of int8 zero points (mixture-of-experts entry point only)
 
 // The bias as the reference adds it: its int8 branch casts the product to the output type and then adds the
