@@ -26,6 +26,8 @@
 // flashnn/triton_kernels/gemm_a16w4.py:163-182 (nibble order), :296-297 (scale rows).
 #include "fnn_common.h"
 
+#include <type_traits>
+
 #include "wo_common.h"
 
 namespace fnn {
@@ -480,9 +482,12 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_kernel(const Wo
 // pairs, [K / group][channels of the tile], one 4-byte read per channel and step.
 template <int WBITS, int ADT, bool G128, int MP, int CH, bool FULL, int REFQ = 0>
 __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(const WoArgs p) {
-    static_assert(!REFQ || (ADT == FNN_F16 && !G128), "reference rounding: fp16, tables per channel or per small group");
+    static_assert(!REFQ || !G128, "reference rounding: tables per channel or per small group");
+    static_assert(REFQ < 3 || ADT == FNN_F16, "reference rounding with small groups: fp16");
     constexpr bool RQG = REFQ >= 3;              // tables per group of 32 or 64
     constexpr bool RQZ = REFQ == 2 || REFQ == 4;
+    // bf16 activations with per-channel bf16 tables: both roundings to bf16, worked in fp32 (ref_dq_bf16)
+    constexpr bool RQBF = REFQ != 0 && ADT == FNN_BF16;
     typedef MfmaT<ADT> MT;
     constexpr int NH = WBITS == 4 ? 2 : 1;
     constexpr int NC = 8 * NH;
@@ -550,9 +555,22 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     }
     v2h rq_s[NH], rq_z[NH];
     const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
+    float bq_s[2], bq_z[2], bq_c[2];
+    bool whole_zp = true;    // wave-uniform: every zero point of the wave's rows is whole and at most 128 (one-step form)
     if constexpr (REFQ == 1 || REFQ == 2) {
 #pragma unroll
-        for (int h = 0; h < NH; ++h) { rq_s[h] = pair_of_f16_bits(rq_sb[h]); rq_z[h] = pair_of_f16_bits(rq_zb[h]); }
+        for (int h = 0; h < NH; ++h) {
+            if constexpr (RQBF) {
+                bq_s[h] = bf16_bits_to_f32(rq_sb[h]);
+                bq_z[h] = bf16_bits_to_f32(rq_zb[h]);
+                bq_c[h] = -((WBITS == 4 ? 8.f : 128.f) + bq_z[h]) * bq_s[h];
+                whole_zp = whole_zp && bf16_zp_is_whole(bq_z[h]);
+            } else {
+                rq_s[h] = pair_of_f16_bits(rq_sb[h]);
+                rq_z[h] = pair_of_f16_bits(rq_zb[h]);
+            }
+        }
+        if constexpr (RQBF && REFQ == 2) whole_zp = __builtin_amdgcn_ballot_w64(!whole_zp) == 0;
     }
 
     for (int e = threadIdx.x; e < ZERO_BYTES / 4; e += kDecWaves * 64) ((uint32_t*)smem)[e] = 0;
@@ -665,6 +683,8 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
     // UN loads are in flight at its start, steps 0..CH-UN-1 each issue the load UN steps ahead,
     // so the wait counts are exact and nothing is carried over a loop edge in registers.
     const v4u ones = v4u{MT::one2, MT::one2, MT::one2, MT::one2};
+    auto run = [&](auto one_step_tag) {
+    constexpr bool ONE_STEP = decltype(one_step_tag)::value;
     for (int sb = s_begin; sb < s_end; sb += CH) {
         if (sb != s_begin) {
 #pragma unroll
@@ -689,11 +709,12 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
                 }
                 if constexpr (WBITS == 4) {
                     v4u e0, e1, o0, o1;
-                    convert_w4<ADT>(w, e0, e1, o0, o1);
+                    if constexpr (RQBF) dq_w4_bf16<false, ONE_STEP>(w, bq_s, bq_z, bq_c, e0, e1, o0, o1);
+                    else convert_w4<ADT>(w, e0, e1, o0, o1);
                     // refill the queue slot only after its old value is dead, so that both live
                     // in the same registers
                     if (i + UN < CH) wq[i % UN] = load_w(step + UN);
-                    if constexpr (REFQ) {
+                    if constexpr (REFQ != 0 && !RQBF) {
                         e0 = ref_dq_f16<RQZ>(e0, rq_c, rq_z[0], rq_s[0]);
                         e1 = ref_dq_f16<RQZ>(e1, rq_c, rq_z[0], rq_s[0]);
                         o0 = ref_dq_f16<RQZ>(o0, rq_c, rq_z[NH - 1], rq_s[NH - 1]);
@@ -707,9 +728,10 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
                     if constexpr (!REFQ) asum = MT::mma(ones, a1, asum);
                 } else {
                     v4u s0, s1;
-                    convert_w8<ADT>(w, s0, s1);
+                    if constexpr (RQBF) dq_w8_bf16<ONE_STEP>(w, bq_s[0], bq_z[0], bq_c[0], s0, s1);
+                    else convert_w8<ADT>(w, s0, s1);
                     if (i + UN < CH) wq[i % UN] = load_w(step + UN);
-                    if constexpr (REFQ) {
+                    if constexpr (REFQ != 0 && !RQBF) {
                         s0 = ref_dq_f16<RQZ>(s0, rq_c, rq_z[0], rq_s[0]);
                         s1 = ref_dq_f16<RQZ>(s1, rq_c, rq_z[0], rq_s[0]);
                     }
@@ -729,6 +751,13 @@ __global__ __launch_bounds__(kDecWaves * 64) void gemm_wo_decode_lds_kernel(cons
         }
         a_real += CH * 256;
         if constexpr (G128) sz_addr += CH * NC * 4;
+    }
+    };
+    if constexpr (RQBF && REFQ == 2) {
+        if (whole_zp) run(std::true_type{});
+        else run(std::false_type{});
+    } else {
+        run(std::true_type{});
     }
     if constexpr (!G128) {
         if (s_begin < s_end) fold(sz_addr);
@@ -1454,19 +1483,26 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
         if (smem > 64 * 1024) return false;   // beyond what a launch may ask for without raising the kernel's limit
 #define FNN_DEC(G, MPV, ...)                                                                         \
     do {                                                                                             \
-        note_kernel("gemm_wo_decode_lds_kernel", WBITS, MPV, full16 ? 16 : full8 ? 8 : -16);             \
+        note_kernel(refq ? "gemm_wo_decode_lds_kernel(per-weight rounding)" : "gemm_wo_decode_lds_kernel", WBITS, MPV, \
+                    full16 ? 16 : full8 ? 8 : -16);                                                  \
         if (full16) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, true, ##__VA_ARGS__><<<grid, block, smem, st>>>(p); \
         else if (full8) gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 8, true, ##__VA_ARGS__><<<grid, block, smem, st>>>(p); \
         else gemm_wo_decode_lds_kernel<WBITS, ADT, G, MPV, 16, false, ##__VA_ARGS__><<<grid, block, smem, st>>>(p);  \
     } while (0)
-        // fp16 activations with per-channel fp16 scales: the reference's own per-weight rounding
-        bool refq = false;
+        // per-channel scales (and zero points) of the activations' 16-bit type, or fp16 everything with small
+        // groups: the reference's own per-weight rounding
+        // (not int4 weights under bf16: see launch_wo_panel)
+        constexpr bool CAN_REFQ = ADT == FNN_F16 || WBITS == 8;
+        const bool refq = (CAN_REFQ && p.group == 0 && p.scale_dtype == ADT && (!p.zp || p.zp_dtype == ADT)) || small_groups;
         if constexpr (ADT == FNN_F16) {
-            refq = (p.group == 0 && p.scale_dtype == FNN_F16) || small_groups;
             if (small_groups && p.zp) FNN_DEC(false, 8, 4);
             else if (small_groups) FNN_DEC(false, 8, 3);
-            else if (refq && p.zp) FNN_DEC(false, 8, 2);
-            else if (refq) FNN_DEC(false, 8, 1);
+        }
+        if constexpr (CAN_REFQ) {
+            if (refq && !small_groups) {
+                if (p.zp) FNN_DEC(false, 8, 2);
+                else FNN_DEC(false, 8, 1);
+            }
         }
         if (refq) {}
         else if (p.group == 0) FNN_DEC(false, 8);

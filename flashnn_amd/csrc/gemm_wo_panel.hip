@@ -44,7 +44,9 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // single pass over the weights.
 // REFQ (1, or 2 with zero points; fp16 activations, per-channel fp16 scales and zero points): every weight is dequantised and rounded to
 // fp16 as the reference's torch path does before the dot product (ref_dq_f16 in wo_common.h); the MFMAs
-// against ones and the fold at the end are then not needed.  (The same with tables per group of 128 - a
+// against ones and the fold at the end are then not needed.  With bf16 activations and per-channel bf16 tables
+// the same with both roundings to bf16 (ref_dq_bf16: fp32 arithmetic; the short form where every zero point of
+// the wave's rows is whole, the two-step form otherwise, chosen per wave).  (The same with tables per group of 128 - a
 // lane fetching its row's scale and zero point slab by slab, bf16 rows converted to fp16 by a pass of their
 // own - was built and measured on A16W4, K = 8192, N = 28672: 16 rows 28.0 -> 38.5 us, 64 rows 52.5 -> 56.5 us.
 // Three more instructions per pair of weights where the fold costs two per output and slab: at these row
@@ -54,7 +56,9 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // table row (G128 is set as well: the table path is the same, with twice the rows).
 template <int WBITS, int ADT, bool G128, int SDT, int MB, int RT, int D, bool NTL, bool MOE = false, int REFQ = 0, int GSUB = 1>
 __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, const int passes, const MoeArgs q) {
-    static_assert(!REFQ || (ADT == FNN_F16 && !G128 && !MOE), "reference rounding: fp16, per-channel");
+    static_assert(!REFQ || (!G128 && !MOE), "reference rounding: per-channel tables of the activations' type");
+    // bf16 activations with bf16 tables: both roundings to bf16, worked in fp32 (ref_dq_bf16 in wo_common.h)
+    constexpr bool RQBF = REFQ != 0 && ADT == FNN_BF16;
     static_assert(GSUB == 1 || (GSUB == 2 && G128 && !MOE), "groups of 64: plain calls with group tables");
     // Gathered form with group tables: the reference's mixture-of-experts launcher lays them out
     // [expert][channel][group] (flashnn/triton_kernels/fused_moe_a16w4.py:336-344), the transpose of the
@@ -205,13 +209,24 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
     // REFQ: the scale and zero point of the weight row this lane feeds to the MFMAs (row li of the tile)
     v2h rq_s[NH], rq_z[NH];
     const v2h rq_c = pair_of_f16_bits(WBITS == 4 ? 0x6408u : 0x6480u);   // 1032 / 1152: what the conversion adds
+    float bq_s[2], bq_z[2], bq_c[2];                                     // the same as fp32 numbers (bf16 tables)
+    bool whole_zp = true;    // wave-uniform: every zero point of the wave's rows is whole and at most 128 (one-step form)
     if constexpr (REFQ) {
 #pragma unroll
         for (int h = 0; h < NH; ++h) {
             const int n = NH * (row0 + li) + h;
-            rq_s[h] = pair_of_f16_bits(((const uint16_t*)p.scale)[n]);
-            rq_z[h] = pair_of_f16_bits(p.zp ? ((const uint16_t*)p.zp)[n] : 0u);
+            const uint32_t sb = ((const uint16_t*)p.scale)[n], zb = p.zp ? ((const uint16_t*)p.zp)[n] : 0u;
+            if constexpr (RQBF) {
+                bq_s[h] = bf16_bits_to_f32(sb);
+                bq_z[h] = bf16_bits_to_f32(zb);
+                bq_c[h] = -((WBITS == 4 ? 8.f : 128.f) + bq_z[h]) * bq_s[h];
+                whole_zp = whole_zp && bf16_zp_is_whole(bq_z[h]);
+            } else {
+                rq_s[h] = pair_of_f16_bits(sb);
+                rq_z[h] = pair_of_f16_bits(zb);
+            }
         }
+        if constexpr (RQBF && REFQ == 2) whole_zp = __builtin_amdgcn_ballot_w64(!whole_zp) == 0;
     }
 
     v4f outv[MB][NH], accg[MB][NH], asum[MB];
@@ -273,7 +288,9 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
 
     // All activation fragments of the slab are requested first, the weights are converted while
     // those reads are in flight, and the MFMAs then run back to back behind a single wait.
-    auto compute = [&](const char* stage, const v4u w0, const v4u w1, const bool last, const tab_t s_first, const tab_t z_first) {
+    auto compute = [&](auto one_step_tag, const char* stage, const v4u w0, const v4u w1, const bool last, const tab_t s_first,
+                       const tab_t z_first) {
+        constexpr bool ONE_STEP = decltype(one_step_tag)::value;
         v4u bf[2][MB][2];
 #pragma unroll
         for (int s = 0; s < 2; ++s)
@@ -295,9 +312,14 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         }
         if constexpr (WBITS == 4) {
             v4u e[2][2], o[2][2];
-            convert_w4_nat<ADT>(w0, e[0][0], e[0][1], o[0][0], o[0][1]);
-            convert_w4_nat<ADT>(w1, e[1][0], e[1][1], o[1][0], o[1][1]);
-            if constexpr (REFQ) {
+            if constexpr (RQBF) {
+                dq_w4_bf16<true, ONE_STEP>(w0, bq_s, bq_z, bq_c, e[0][0], e[0][1], o[0][0], o[0][1]);
+                dq_w4_bf16<true, ONE_STEP>(w1, bq_s, bq_z, bq_c, e[1][0], e[1][1], o[1][0], o[1][1]);
+            } else {
+                convert_w4_nat<ADT>(w0, e[0][0], e[0][1], o[0][0], o[0][1]);
+                convert_w4_nat<ADT>(w1, e[1][0], e[1][1], o[1][0], o[1][1]);
+            }
+            if constexpr (REFQ != 0 && !RQBF) {
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -321,9 +343,14 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
             }
         } else {
             v4u c[2][2];
-            convert_w8<ADT>(w0, c[0][0], c[0][1]);
-            convert_w8<ADT>(w1, c[1][0], c[1][1]);
-            if constexpr (REFQ) {
+            if constexpr (RQBF) {
+                dq_w8_bf16<ONE_STEP>(w0, bq_s[0], bq_z[0], bq_c[0], c[0][0], c[0][1]);
+                dq_w8_bf16<ONE_STEP>(w1, bq_s[0], bq_z[0], bq_c[0], c[1][0], c[1][1]);
+            } else {
+                convert_w8<ADT>(w0, c[0][0], c[0][1]);
+                convert_w8<ADT>(w1, c[1][0], c[1][1]);
+            }
+            if constexpr (REFQ != 0 && !RQBF) {
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -356,8 +383,14 @@ __global__ __launch_bounds__(512) void gemm_wo_panel_kernel(const WoArgs p, cons
         wq[W][1] = load_w((JJ) + D, 1);                                    \
         __builtin_amdgcn_sched_barrier(0);                                 \
         if (mine_) {                                                       \
-            compute(CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1]), \
-                    !G128 && part_tail && (JJ) == nsl - 1, sq[Q][0], zq[Q][0]); \
+            bool two_step_ = false;                                        \
+            if constexpr (RQBF && REFQ == 2) two_step_ = !whole_zp;        \
+            if (two_step_)                                                 \
+                compute(std::integral_constant<bool, !(RQBF && REFQ == 2)>{}, CUR, *(const v4u*)(wmine + wrd[0]), \
+                        *(const v4u*)(wmine + wrd[1]), !G128 && part_tail && (JJ) == nsl - 1, sq[Q][0], zq[Q][0]); \
+            else                                                           \
+                compute(std::true_type{}, CUR, *(const v4u*)(wmine + wrd[0]), *(const v4u*)(wmine + wrd[1]), \
+                        !G128 && part_tail && (JJ) == nsl - 1, sq[Q][0], zq[Q][0]); \
             if constexpr (TABLDS) fold(lds_tab(0, (JJ)), lds_tab(1, (JJ))); \
             else if constexpr (G128) fold(sq[Q][GSUB - 1], zq[Q][GSUB - 1]); \
         }                                                                  \
@@ -600,9 +633,12 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);
     p.m_base = 0;
-    // fp16 activations with per-channel fp16 scales (and zero points): the reference's own per-weight rounding
-    constexpr bool CAN_REFQ = ADT == FNN_F16;
-    const bool refq = CAN_REFQ && p.group == 0 && p.scale_dtype == FNN_F16 && (!p.zp || p.zp_dtype == FNN_F16);
+    // per-channel scales (and zero points) of the activations' 16-bit type: the reference's own per-weight rounding.
+    // Not int4 weights under bf16: rounding to bf16 takes about three vector instructions per weight where the plain
+    // conversion of a nibble takes 0.75, which cost 13 to 34 % at 1 to 64 rows, for weights of at most 8 scale steps
+    // whose rounding moves an output 16 times less than an int8 weight's (int8 under bf16: -8 to +9 %).
+    constexpr bool CAN_REFQ = ADT == FNN_F16 || WBITS == 8;
+    const bool refq = CAN_REFQ && p.group == 0 && p.scale_dtype == ADT && (!p.zp || p.zp_dtype == ADT);
     note_kernel(refq ? "gemm_wo_panel_kernel(per-weight rounding)" : "gemm_wo_panel_kernel", WBITS, mb, rt);
 #define FNN_PANEL3(G, SDTV, MBV, RTV, NTLV)                                                              \
     do {                                                                                                 \

@@ -153,6 +153,49 @@ __device__ __forceinline__ void bytes_to_f32(uint32_t x, float (&f)[4]) {
     f[3] = (float)(x >> 24);
 }
 
+// Whole operand groups through ref_dq_bf16: c = -(off + zp) * s (used by the one-step form only).
+// 16 int8 (k .. k+15 of one row) -> two bf16 MFMA operands in natural k order (as convert_w8)
+template <bool ONE_STEP>
+__device__ __forceinline__ void dq_w8_bf16(const v4u w, float s, float zp, float c, v4u& s0, v4u& s1) {
+    uint32_t o[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        float f[4];
+        bytes_to_f32(w[q] ^ 0x80808080u, f);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            o[2 * q + i] = ONE_STEP ? ref_dq_bf16_merged(f[2 * i], f[2 * i + 1], s, c) : ref_dq_bf16(f[2 * i], f[2 * i + 1], 128.f, zp, s);
+    }
+    s0 = v4u{o[0], o[1], o[2], o[3]};
+    s1 = v4u{o[4], o[5], o[6], o[7]};
+}
+// 16 bytes = 16 k of two channels (index 0: the even channel, low nibbles) -> bf16 operands; NAT: natural k order
+// (as convert_w4_nat), else the order (0,2)(1,3)(4,6)(5,7) of convert_w4
+template <bool NAT, bool ONE_STEP>
+__device__ __forceinline__ void dq_w4_bf16(const v4u w, const float (&s)[2], const float (&zp)[2], const float (&c)[2],
+                                           v4u& e0, v4u& e1, v4u& o0, v4u& o1) {
+    uint32_t e[8], o[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t x = w[q] ^ 0x88888888u;      // two's complement -> offset by 8
+        float fe[4], fo[4];
+        bytes_to_f32(x & 0x0F0F0F0Fu, fe);
+        bytes_to_f32((x >> 4) & 0x0F0F0F0Fu, fo);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int k0 = NAT ? 2 * i : i, k1 = NAT ? 2 * i + 1 : i + 2;
+            e[2 * q + i] = ONE_STEP ? ref_dq_bf16_merged(fe[k0], fe[k1], s[0], c[0]) : ref_dq_bf16(fe[k0], fe[k1], 8.f, zp[0], s[0]);
+            o[2 * q + i] = ONE_STEP ? ref_dq_bf16_merged(fo[k0], fo[k1], s[1], c[1]) : ref_dq_bf16(fo[k0], fo[k1], 8.f, zp[1], s[1]);
+        }
+    }
+    e0 = v4u{e[0], e[1], e[2], e[3]};
+    e1 = v4u{e[4], e[5], e[6], e[7]};
+    o0 = v4u{o[0], o[1], o[2], o[3]};
+    o1 = v4u{o[4], o[5], o[6], o[7]};
+}
+// whether a bf16 zero point lets the one-step form stand for the reference's two roundings
+__device__ __forceinline__ bool bf16_zp_is_whole(float z) { return z == rintf(z) && fabsf(z) <= 128.f; }
+
 constexpr int FNN_I8 = 3;   // type code of int8 zero points (mixture-of-experts entry point only)
 
 // The bias as the reference adds it: its int8 branch casts the product to the output type and then adds the

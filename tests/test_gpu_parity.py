@@ -776,7 +776,8 @@ WO_BREACHES = []   # (case, outputs beyond the stated tolerance, outputs) of the
 # rtol = atol = 1e-2 although the kernel is the more accurate of the two.  Only these kernels may leave the
 # stated tolerance, only on a bounded share of the outputs, and only towards the float64 value; every kernel
 # that says it rounds per weight - the tiled kernel for more than 64 rows (fp16 tables, or bf16 tables with bf16
-# activations) and the few-row kernels with per-channel fp16 tables - is held to the tolerance without exception.
+# activations) and the few-row kernels with per-channel tables of the activations' type (fp16; bf16 over int8
+# weights) - is held to the tolerance without exception.
 FP32_SCALING_KERNELS = {"gemm_wo_panel_kernel", "gemm_wo_stream_kernel", "gemm_wo_any_kernel", "gemm_wo_decode_kernel",
                         "gemm_wo_decode_lds_kernel", "gemm_wo_gemv_kernel", "gemm_wo_gemv_flat_kernel",
                         "gemm_wo_tile_kernel"}
@@ -1150,6 +1151,52 @@ def test_weight_only_tiled_zero_points_whole_or_not(bits, group, kind, ty):
                                   _tag(ty), _tag(ty), group, bits == 4)
         assert (np.abs(got - want) <= ATOL + RTOL * np.abs(want)).all()
     assert _lib.last_kernel().startswith("gemm_wo_tile_kernel(per-weight rounding)"), _lib.last_kernel()
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 9, 33, 64])
+@pytest.mark.parametrize("kind", ["none", "whole", "quarter", "large"])
+def test_a16w8_bf16_tables_round_per_weight(M, kind):
+    """int8 weights under bf16 rows with per-channel bf16 tables, 1 to 64 rows: the decode and panel kernels round
+    every weight to bf16 as the reference does (fp32 arithmetic), in one step where the zero points of a wave's rows are
+    whole, in two where one is fractional or large - chosen per wave, so the single large one leaves the rest on the
+    short form."""
+    N, K = 1024, 2048
+    bf = torch.bfloat16
+    act, w, qw, scale, zp, bias = _wo_inputs(M, N, K, 0, 8, bf, bf, kind != "none", M == 8, seed=900 + M)
+    if kind == "quarter":
+        zp = (zp.float() + 0.25).to(bf)
+    elif kind == "large":
+        zp = zp.clone()
+        zp[100] = 600.0
+    if kind != "large":
+        _wo_check(act, w, qw, scale, zp, bias, 0, 8, bf, strict=True)
+    else:
+        # (outputs of the size of 600 * scale * sum(a): only the tolerance is held, as in the tiled kernel's test)
+        d = lambda t: None if t is None else t.to(DEV)
+        got = flashnn_amd.GemmWeightOnly(bf)(d(act), d(qw), d(scale), d(bias), d(zp)).float().cpu().numpy()
+        want = O.weight_only_gemm(O.to_np(act), w.numpy(), O.to_np(scale), O.to_np(zp), None if bias is None else O.to_np(bias),
+                                  O.BF16, O.BF16, 0, False)
+        assert (np.abs(got - want) <= ATOL + RTOL * np.abs(want) + 2.0 ** -7 * np.abs(want)).all()
+    assert "per-weight rounding" in _lib.last_kernel(), _lib.last_kernel()
+
+
+@pytest.mark.parametrize("M", [4, 16])
+def test_a16w8_bf16_one_hot_few_rows(M):
+    """One-hot bf16 rows pick single int8 weights: each output is twice bf16((q - zp) * scale), bit for bit (decode
+    kernel at 4 rows, panel kernel at 16)."""
+    N, K = 512, 1024
+    g = torch.Generator().manual_seed(79)
+    bf = torch.bfloat16
+    w = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    scale = torch.empty(N).uniform_(1e-3, 1e-2, generator=g).to(bf)
+    zp = torch.randint(-64, 64, (N,), generator=g).to(bf)
+    ks = torch.randint(0, K, (M,), generator=g)
+    act = torch.zeros(M, K, dtype=bf)
+    act[torch.arange(M), ks] = 2.0
+    out = flashnn_amd.GemmWeightOnly(bf)(act.to(DEV), w.to(DEV), scale.to(DEV), None, zp.to(DEV))
+    assert "per-weight rounding" in _lib.last_kernel(), _lib.last_kernel()
+    want = 2.0 * ((w[:, ks].float() - zp.float()[:, None]) * scale.float()[:, None]).to(bf).float()   # [N, M]
+    assert torch.equal(out.float().cpu(), want.t().contiguous())
 
 
 @pytest.mark.parametrize("ty", [torch.float16, torch.bfloat16])
