@@ -37,6 +37,8 @@ _SIGNATURES = {
     "fnn_gemm_weight_only_workspace_bytes": [_i64] * 4 + [_int] * 2,
     "fnn_gemm_a16w8_ws": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr, _size, _ptr],
     "fnn_gemm_a16w4_ws": [_ptr] * 6 + [_i64] * 7 + [_int] * 5 + [_ptr, _size, _ptr],
+    "fnn_gemm_a16w8_tiled": [_ptr] * 6 + [_i64] * 7 + [_int] * 7 + [_ptr],
+    "fnn_gemm_a16w4_tiled": [_ptr] * 6 + [_i64] * 7 + [_int] * 7 + [_ptr],
     "fnn_a16w4_prepacked_bytes": [_i64] * 3,
     "fnn_a16w4_prepack": [_ptr] * 4 + [_i64] * 4 + [_int] * 2 + [_ptr],
     "fnn_gemm_a16w4_prepacked": [_ptr] * 4 + [_i64] * 6 + [_int] * 3 + [_ptr],

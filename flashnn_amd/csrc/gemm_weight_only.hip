@@ -1674,7 +1674,7 @@ static int run_wo(const char* fn, void* out, const void* act, const void* qw, co
                   const void* bias, const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda,
                   int64_t ldw, int64_t ldc, int64_t group, int act_dtype, int out_dtype,
                   int scale_dtype, int zp_dtype, int bias_dtype, void* stream, void* workspace = nullptr,
-                  size_t ws_bytes = 0) {
+                  size_t ws_bytes = 0, int block_m = 0, int block_n = 0) {
     // an empty tensor has no address: pointers are only required when there is something to compute
     if (M != 0 && N != 0 && (!out || !act || !qw || !scale)) { set_error("%s: null pointer argument", fn); return FNN_ERR_ARG; }
     if (M < 0 || N < 0 || K <= 0 || lda < K || ldw < K || ldc < N || group < 0) {
@@ -1701,6 +1701,29 @@ static int run_wo(const char* fn, void* out, const void* act, const void* qw, co
     p.out_dtype = out_dtype; p.scale_dtype = scale_dtype; p.zp_dtype = zp_dtype; p.bias_dtype = bias_dtype;
     if (ws_bytes > 0 && !workspace) { set_error("%s: a workspace size without a workspace", fn); return FNN_ERR_ARG; }
     p.cvt_ws = workspace; p.cvt_ws_bytes = ws_bytes;
+    if (block_m != 0 || block_n != 0) {
+        // Blocks named by the caller (a recorded configuration, or a candidate being timed): the few-row kernel
+        // with block_m activation rows per pass and block_n output channels per workgroup, for up to 64 rows -
+        // the range in which it is the launcher's own choice from two rows on.  Refused where the launcher's
+        // choice rounds every weight as the reference does and this kernel would not (groups of 64, up to 8 rows,
+        // fp16 throughout), so that a named block never changes how the result is rounded.
+        constexpr int NH = WBITS == 4 ? 2 : 1;
+        const bool rounds_elsewhere = group == 64 && M <= 8 && act_dtype == FNN_F16 && scale_dtype == FNN_F16 &&
+                                      (!zp || zp_dtype == FNN_F16);
+        if (M > 64 || block_m % 16 != 0 || block_n % (16 * NH) != 0 || rounds_elsewhere) {
+            set_error("%s: blocks of %d rows x %d channels are not available for M=%lld group=%lld", fn, block_m, block_n,
+                      (long long)M, (long long)group);
+            return FNN_ERR_UNSUPPORTED;
+        }
+        p.force_mb = block_m / 16;
+        p.force_rt = block_n / (16 * NH);
+        const Call call(fn);
+        if (!launch_wo_panel(p, WBITS, act_dtype, (hipStream_t)stream)) {
+            set_error("%s: the few-row kernel does not take this problem with blocks of %d rows x %d channels", fn, block_m, block_n);
+            return FNN_ERR_UNSUPPORTED;
+        }
+        return call.done();
+    }
     const Call call(fn);
     if (act_dtype == FNN_F16) dispatch_wo<WBITS, FNN_F16>(p, (hipStream_t)stream);
     else dispatch_wo<WBITS, FNN_BF16>(p, (hipStream_t)stream);
@@ -1727,6 +1750,24 @@ extern "C" int fnn_gemm_a16w4(void* out, const void* act, const void* qw, const 
                               void* stream) {
     return run_wo<4>("fnn_gemm_a16w4", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group,
                      act_dtype, out_dtype, scale_dtype, zp_dtype, bias_dtype, stream);
+}
+
+extern "C" int fnn_gemm_a16w8_tiled(void* out, const void* act, const void* qw, const void* scale, const void* bias,
+                                    const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                                    int64_t group, int act_dtype, int out_dtype, int scale_dtype, int zp_dtype,
+                                    int bias_dtype, int block_m, int block_n, void* stream) {
+    if (block_m <= 0 || block_n <= 0) { set_error("fnn_gemm_a16w8_tiled: block_m and block_n must be positive"); return FNN_ERR_ARG; }
+    return run_wo<8>("fnn_gemm_a16w8_tiled", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group, act_dtype,
+                     out_dtype, scale_dtype, zp_dtype, bias_dtype, stream, nullptr, 0, block_m, block_n);
+}
+
+extern "C" int fnn_gemm_a16w4_tiled(void* out, const void* act, const void* qw, const void* scale, const void* bias,
+                                    const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                                    int64_t group, int act_dtype, int out_dtype, int scale_dtype, int zp_dtype,
+                                    int bias_dtype, int block_m, int block_n, void* stream) {
+    if (block_m <= 0 || block_n <= 0) { set_error("fnn_gemm_a16w4_tiled: block_m and block_n must be positive"); return FNN_ERR_ARG; }
+    return run_wo<4>("fnn_gemm_a16w4_tiled", out, act, qw, scale, bias, zp, M, N, K, lda, ldw, ldc, group, act_dtype,
+                     out_dtype, scale_dtype, zp_dtype, bias_dtype, stream, nullptr, 0, block_m, block_n);
 }
 
 extern "C" size_t fnn_gemm_weight_only_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t group, int act_dtype,

@@ -628,7 +628,14 @@ static bool launch_panel_t(WoArgs& p, hipStream_t st) {
         if (!tables16) return false;
     }
     int mb = 1;
-    const int rt = choose_rows(wrows, p.M, (int)((p.K + 127) / 128), &mb, WBITS);
+    int rt = choose_rows(wrows, p.M, (int)((p.K + 127) / 128), &mb, WBITS);
+    if (p.force_rt != 0 || p.force_mb != 0) {
+        // blocks named by the caller: one of the built pairs, and weight rows that divide into such tiles
+        rt = p.force_rt;
+        mb = p.force_mb;
+        const bool built = (rt == 4 && (mb == 1 || mb == 2 || mb == 4)) || (rt == 2 && (mb == 1 || mb == 2)) || (rt == 1 && mb == 1);
+        if (!built || wrows % (16 * rt) != 0) return false;
+    }
     const int tiles = wrows / (16 * rt);
     const int passes = (p.M + mb * 16 - 1) / (mb * 16);
     const dim3 grid(((tiles + 7) / 8) * 8 * passes);

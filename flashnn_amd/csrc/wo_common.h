@@ -24,6 +24,8 @@ struct WoArgs {
     size_t cvt_ws_bytes;
     const float* act_unscale;   // per activation row: what the output is multiplied by (NULL: nothing); set where
                                 // the rows were scaled by a power of two on their way from bf16 to fp16
+    int force_rt, force_mb;     // the panel kernel's blocks named by the caller: 16 force_rt weight rows per workgroup,
+                                // 16 force_mb activation rows per pass (0: the launcher chooses)
 };
 
 // s if group == 128 << s (the group sizes whose tables the 128-value slabs of the panel and tiled kernels can

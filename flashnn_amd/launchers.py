@@ -231,7 +231,7 @@ def hip_gemm_a8w8_int32(a, b, tile=(0, 0, 0)):
     return acc
 
 
-def _weight_only(fn_name, out, act, quant_w, scale_w, bias, zero_points, n_out):
+def _weight_only(fn_name, out, act, quant_w, scale_w, bias, zero_points, n_out, tile=None):
     assert quant_w.dtype == torch.int8, "Weight must be int8 type"
     assert act.is_contiguous(), "Activation must be contiguous"
     assert quant_w.is_contiguous(), "Weight must be contiguous"
@@ -277,30 +277,54 @@ def _weight_only(fn_name, out, act, quant_w, scale_w, bias, zero_points, n_out):
             _lib.dtype_code(bias.dtype) if bias is not None else 0)
     # scratch for bf16 rows converted to fp16 (so that every weight is rounded as the reference rounds it): taken
     # from torch's caching allocator per call, which hands it to later calls on this stream in stream order
-    need = 0
-    if M > 64 and act.dtype == torch.bfloat16:
-        need = int(lib.fnn_gemm_weight_only_workspace_bytes(M, N, K, group, _lib.dtype_code(act.dtype),
-                                                            _lib.dtype_code(scale_w.dtype)))
-    if need:
-        ws = torch.empty(need, dtype=torch.uint8, device=act.device)
-        _lib.check(getattr(lib, fn_name + "_ws")(*args, ws.data_ptr(), need, _lib.current_stream(act.device)))
+    def run_default():
+        need = 0
+        if M > 64 and act.dtype == torch.bfloat16:
+            need = int(lib.fnn_gemm_weight_only_workspace_bytes(M, N, K, group, _lib.dtype_code(act.dtype),
+                                                                _lib.dtype_code(scale_w.dtype)))
+        if need:
+            ws = torch.empty(need, dtype=torch.uint8, device=act.device)
+            _lib.check(getattr(lib, fn_name + "_ws")(*args, ws.data_ptr(), need, _lib.current_stream(act.device)))
+        else:
+            _lib.check(getattr(lib, fn_name)(*args, _lib.current_stream(act.device)))
+
+    def run_named(t):
+        bm, bn = tuned_configs.as_config(t)[:2]
+        if bm == 0:
+            return run_default()
+        return _lib.check(getattr(lib, fn_name + "_tiled")(*args, bm, bn, _lib.current_stream(act.device)))
+
+    # Up to 64 rows the blocks of the few-row kernel can be named: a shape-keyed record, written by a tuning run
+    # under the name of the reference's kernel for the call (gemm_a16w8.py:84, :180; gemm_a16w4.py:84, :210) with
+    # the shape it is tuned by there (key M, N, K; gemm_a16w8.py:322-336), and the group size where there is one
+    if M <= 64:
+        prefix = fn_name[4:] + ("_per_channel" if group == 0 else f"_sub_channel_g{group}")
+        if tile is None:
+            tile = tuned_configs.CACHE.shape_tile(prefix, M, N, K)
+        if tile is None and get_autotune_triton_kernels():
+            tile = tuned_configs.tune(f"{prefix}_{M}_{N}_{K}", tuned_configs.weight_only_candidates(N // quant_w.shape[0]),
+                                      run_named)
+    if tile is None:
+        run_default()
     else:
-        _lib.check(getattr(lib, fn_name)(*args, _lib.current_stream(act.device)))
+        run_named(tile)
     return out
 
 
-def hip_gemm_a16w8_forward(out, act, quant_w, scale_w, bias=None, zero_points=None):
+def hip_gemm_a16w8_forward(out, act, quant_w, scale_w, bias=None, zero_points=None, tile=None):
     """Replaces triton_gemm_a16w8_forward (flashnn/triton_kernels/gemm_a16w8.py:275-338).
-    `out` need not be zeroed."""
+    `out` need not be zeroed.  `tile` = (rows per pass, channels per workgroup) names the blocks of the few-row
+    kernel (up to 64 rows) and bypasses the tuned-configuration lookup (not part of the reference's signature)."""
     return _weight_only("fnn_gemm_a16w8", out, act, quant_w, scale_w, bias, zero_points,
-                        quant_w.shape[0])
+                        quant_w.shape[0], tile)
 
 
-def hip_gemm_a16w4_forward(out, act, quant_w, scale_w, bias=None, zero_points=None):
+def hip_gemm_a16w4_forward(out, act, quant_w, scale_w, bias=None, zero_points=None, tile=None):
     """Replaces triton_gemm_a16w4_forward (flashnn/triton_kernels/gemm_a16w4.py:336-406).
-    quant_w is [N/2, K] with channel 2j in the low and 2j+1 in the high nibble of row j."""
+    quant_w is [N/2, K] with channel 2j in the low and 2j+1 in the high nibble of row j.  `tile` as in
+    hip_gemm_a16w8_forward."""
     return _weight_only("fnn_gemm_a16w4", out, act, quant_w, scale_w, bias, zero_points,
-                        quant_w.shape[0] * 2)
+                        quant_w.shape[0] * 2, tile)
 
 
 class PrepackedInt4:

@@ -3,7 +3,9 @@ compile_and_cache_kernels and configs/triton_autotune_best_configs.json play in 
 (flashnn/triton_kernels/triton_utils.py:14-24, 38-80, 84-151).
 
 A kernel launch is named by a method name ("gemm_a8w8_M_N_K", the reference's own,
-triton_kernels/gemm_a8w8.py:199).  The first time a method name is met while tuning is switched on
+triton_kernels/gemm_a8w8.py:199; the weight-only GEMMs of up to 64 rows, which the reference tunes in-process
+by M, N, K - gemm_a16w8.py:322-336 - are named after its kernels: "gemm_a16w8_per_channel_M_N_K",
+"gemm_a16w4_sub_channel_g128_M_N_K").  The first time a method name is met while tuning is switched on
 (set_autotune_triton_kernels(True), as in the reference) the candidates are timed on the caller's
 operands and the best one is recorded, in memory and in the JSON file; afterwards, and in later
 processes, the recorded configuration is used without timing anything.  With tuning switched off
@@ -29,6 +31,16 @@ JSON_FILENAME = "hip_autotune_best_configs.json"
 # admit (parts shorter than four slabs, M or N too small) are refused by the library and skipped by tune().
 A8W8_CANDIDATES = [(0, 0, 0, 0), (256, 256, 0, 1), (256, 192, 0, 1), (256, 128, 0, 1), (128, 128, 0, 1), (64, 128, 0, 1),
                    (128, 128, 0, 2), (128, 128, 0, 3), (128, 128, 0, 4), (128, 128, 0, 6), (128, 128, 0, 8)]
+
+
+def weight_only_candidates(channels_per_weight_row):
+    """Candidate (rows per pass, channels per workgroup, 0, 1) of the few-row weight-only kernel, the BLOCK_M and
+    BLOCK_N of the reference's lists (gemm_a16w8.py:15-80, gemm_a16w4.py:15-80); (0, 0, 0, 0) = the library's
+    choice, which comes first because every shape admits it.  A workgroup takes 16, 32 or 64 weight rows (one or
+    two channels each) and at most as many activation rows per pass; pairs a shape does not divide into are
+    refused by the library and skipped by tune()."""
+    c = channels_per_weight_row
+    return [(0, 0, 0, 0)] + [(16 * mb, 16 * rt * c, 0, 1) for rt in (4, 2, 1) for mb in (4, 2, 1) if mb <= rt]
 
 
 def as_config(tile):

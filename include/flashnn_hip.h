@@ -170,6 +170,25 @@ int fnn_gemm_a16w4_ws(void* out, const void* act, const void* qw, const void* sc
                       void* workspace, size_t ws_bytes, void* stream);
 
 /*
+ * fnn_gemm_a16w8 / fnn_gemm_a16w4 with the blocks of the few-row kernel named by the caller: block_m activation
+ * rows per pass over the weights (16, 32 or 64) and block_n output channels per workgroup (16, 32 or 64 weight
+ * rows: int8 16 / 32 / 64 channels, int4 32 / 64 / 128), block_m not above the weight rows of a workgroup.  The
+ * counterpart of the BLOCK_M / BLOCK_N of the reference's autotune lists for these kernels
+ * (flashnn/triton_kernels/gemm_a16w8.py:15-80, gemm_a16w4.py:15-80), for a tuned-configuration cache to time and
+ * record; up to 64 rows.  FNN_ERR_UNSUPPORTED where the pair is not built, the shape does not divide into such
+ * blocks, or the library's own choice for the call rounds every weight as the reference does and this kernel
+ * would not: a named block never changes the rounding of the result, only the order of the fp32 additions.
+ */
+int fnn_gemm_a16w8_tiled(void* out, const void* act, const void* qw, const void* scale, const void* bias,
+                         const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                         int64_t group, int act_dtype, int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
+                         int block_m, int block_n, void* stream);
+int fnn_gemm_a16w4_tiled(void* out, const void* act, const void* qw, const void* scale, const void* bias,
+                         const void* zp, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                         int64_t group, int act_dtype, int out_dtype, int scale_dtype, int zp_dtype, int bias_dtype,
+                         int block_m, int block_n, void* stream);
+
+/*
  * fnn_gemm_a16w4 on weights repacked once by the caller (made for the decode of one or a few tokens).  The
  * reference keeps int4 weights as [N/2, K] bytes with [K/group, N] tables beside them
  * (flashnn/quant_gemm.py:174-204; its Triton launcher, flashnn/triton_kernels/gemm_a16w4.py:336-406, reads

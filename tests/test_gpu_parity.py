@@ -1153,6 +1153,111 @@ def test_weight_only_tiled_zero_points_whole_or_not(bits, group, kind, ty):
     assert _lib.last_kernel().startswith("gemm_wo_tile_kernel(per-weight rounding)"), _lib.last_kernel()
 
 
+def _close_to(got, want, out_ty):
+    """Two fp32 summation orders of one dot product, each rounded once to the output type."""
+    got, want = got.float().cpu().numpy(), want.float().cpu().numpy()
+    step = 2.0 ** -7 if out_ty == torch.bfloat16 else 2.0 ** -10
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    return (np.abs(got - want) <= step * np.abs(want) + 1e-3 * rms).all()
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("group", [0, 128])
+def test_weight_only_named_blocks(bits, group):
+    """Every pair of blocks of the few-row kernel, named through the `_tiled` entry points, gives the result of the
+    library's own choice up to the order of the fp32 additions, on the kernel variant it names; pairs the shape does
+    not divide into, more than 64 rows, and a call whose default path rounds differently are refused."""
+    from flashnn_amd import tuned_configs as TC
+    M, N, K = 40, 2048, 2048
+    act_ty = torch.float16 if group == 0 else torch.bfloat16
+    act, w, qw, scale, zp, bias = _wo_inputs(M, N, K, group, bits, act_ty, torch.float16, True, True, seed=77)
+    d = lambda t: t.to(DEV)
+    fwd = launchers.hip_gemm_a16w8_forward if bits == 8 else launchers.hip_gemm_a16w4_forward
+    plain = torch.empty(M, N, dtype=act_ty, device=DEV)
+    fwd(plain, d(act), d(qw), d(scale), d(bias), d(zp))
+    assert _lib.last_kernel().startswith("gemm_wo_panel_kernel"), _lib.last_kernel()
+    rounding = "(per-weight rounding)" in _lib.last_kernel()
+    cands = TC.weight_only_candidates(2 if bits == 4 else 1)
+    assert cands[0] == (0, 0, 0, 0) and len(cands) == 7
+    for cand in cands[1:]:
+        out = torch.full((M, N), float("nan"), dtype=act_ty, device=DEV)
+        fwd(out, d(act), d(qw), d(scale), d(bias), d(zp), tile=cand)
+        mb, rt = cand[0] // 16, cand[1] // (16 * (2 if bits == 4 else 1))
+        assert _lib.last_kernel() == f"gemm_wo_panel_kernel{'(per-weight rounding)' if rounding else ''}<{bits},{mb},{rt}>", (cand, _lib.last_kernel())
+        assert _close_to(out, plain, act_ty), cand
+    out = torch.empty(M, N, dtype=act_ty, device=DEV)
+    for bad in ((48, 64), (16, 24), (64, 32 * (2 if bits == 4 else 1)), (16, 256)):     # not built: rows above the tile's, odd sizes
+        with pytest.raises(_lib.FlashnnHipError):
+            fwd(out, d(act), d(qw), d(scale), d(bias), d(zp), tile=bad)
+    # weight rows that do not divide into 64-row tiles
+    n2 = 48 * (2 if bits == 4 else 1)
+    out2 = torch.empty(M, n2, dtype=act_ty, device=DEV)
+    rows = n2 // (2 if bits == 4 else 1)
+    with pytest.raises(_lib.FlashnnHipError):
+        fwd(out2, d(act), d(qw[:rows]), d(scale[..., :n2].contiguous()), None, None, tile=cands[1])
+    fwd(out2, d(act), d(qw[:rows]), d(scale[..., :n2].contiguous()), None, None, tile=cands[-1])   # 16-row tiles do
+    # more than 64 rows
+    act65 = torch.randn(65, K).to(act_ty)
+    with pytest.raises(_lib.FlashnnHipError):
+        fwd(torch.empty(65, N, dtype=act_ty, device=DEV), d(act65), d(qw), d(scale), None, None, tile=cands[1])
+
+
+def test_weight_only_named_blocks_never_change_the_rounding():
+    """Groups of 64 with up to 8 fp16 rows run on the decode kernel, which rounds every weight as the reference does;
+    the few-row kernel would scale in fp32, so its blocks cannot be named for such a call."""
+    M, N, K = 4, 1024, 2048
+    act, w, qw, scale, zp, bias = _wo_inputs(M, N, K, 64, 8, torch.float16, torch.float16, True, False, seed=78)
+    d = lambda t: t.to(DEV)
+    out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+    with pytest.raises(_lib.FlashnnHipError):
+        launchers.hip_gemm_a16w8_forward(out, d(act), d(qw), d(scale), None, d(zp), tile=(16, 64))
+    launchers.hip_gemm_a16w8_forward(out, d(act), d(qw), d(scale), None, d(zp))
+    assert "per-weight rounding" in _lib.last_kernel(), _lib.last_kernel()
+
+
+def test_weight_only_tuned_config_cache(tmp_path, monkeypatch):
+    """With tuning on, the first weight-only launch of a shape with up to 64 rows times the block pairs of the few-row
+    kernel and records the best under the name of the reference's kernel for the call; the next launch, and a fresh
+    reader of the file, use the record; more than 64 rows are not tuned."""
+    import json
+    from flashnn_amd import tuned_configs as TC
+    path = tmp_path / "best.json"
+    monkeypatch.setenv("FLASHNN_AMD_TUNED_CONFIGS", str(path))
+    TC.CACHE.reset()
+    M, N, K = 24, 4096, 2048
+    d = lambda t: None if t is None else t.to(DEV)
+    try:
+        for bits, group, name in ((8, 0, f"gemm_a16w8_per_channel_{M}_{N}_{K}"), (4, 128, f"gemm_a16w4_sub_channel_g128_{M}_{N}_{K}")):
+            act, w, qw, scale, zp, bias = _wo_inputs(M, N, K, group, bits, torch.bfloat16, torch.float16, True, False, seed=79)
+            op = flashnn_amd.GemmWeightOnly(torch.bfloat16)
+            plain = op(d(act), d(qw), d(scale), None, d(zp))
+            flashnn_amd.set_autotune_triton_kernels(True)
+            try:
+                tuned = op(d(act), d(qw), d(scale), None, d(zp))
+            finally:
+                flashnn_amd.set_autotune_triton_kernels(False)
+            data = json.load(open(path))
+            assert name in data, list(data)
+            tile = TC.deserialize_best_config(data[name])
+            assert tile in TC.weight_only_candidates(2 if bits == 4 else 1)
+            again = op(d(act), d(qw), d(scale), None, d(zp))
+            if tile[0]:
+                assert _lib.last_kernel().endswith(f"<{bits},{tile[0] // 16},{tile[1] // (16 * (2 if bits == 4 else 1))}>"), _lib.last_kernel()
+            assert _close_to(tuned, plain, torch.bfloat16) and _close_to(again, plain, torch.bfloat16)
+            assert TC.TunedConfigs().lookup(name) == tile
+        n_records = len(json.load(open(path)))
+        act, w, qw, scale, zp, bias = _wo_inputs(80, 1024, 1024, 0, 8, torch.float16, torch.float16, False, False, seed=80)
+        flashnn_amd.set_autotune_triton_kernels(True)
+        try:
+            flashnn_amd.GemmWeightOnly(torch.float16)(d(act), d(qw), d(scale), None, None)
+        finally:
+            flashnn_amd.set_autotune_triton_kernels(False)
+        assert len(json.load(open(path))) == n_records
+    finally:
+        monkeypatch.undo()
+        TC.CACHE.reset()
+
+
 @pytest.mark.parametrize("M", [1, 3, 8, 9, 33, 64])
 @pytest.mark.parametrize("kind", ["none", "whole", "quarter", "large"])
 def test_a16w8_bf16_tables_round_per_weight(M, kind):
