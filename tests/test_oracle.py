@@ -560,3 +560,44 @@ def test_fused_moe_a16w4_exact_and_reductions():
                             np.array([8]), False, 1, BM, O.F16, O.F16)
     ref = O.weight_only_gemm_f64(O.to_np(a), w[1].numpy(), O.to_np(scale)[1], zp[1].numpy(), None, 0)
     np.testing.assert_allclose(one, ref, rtol=2e-3, atol=1e-5)
+
+
+def test_one_step_dequantisation_equals_the_two_roundings():
+    """The kernels that round every weight as the torch path does take a short form where the zero points are whole:
+    one fp16 subtraction of (offset + zp) from the offset-coded weight, or, for bf16 tables, one exact fp32
+    u * s - (off + zp) * s rounded once to bf16.  Both must give the bits of `((q - zp) * s)` evaluated in the table
+    type with each operation rounded (flashnn/quant_gemm.py:14-17) - checked here with torch's own 16-bit arithmetic
+    over every int8 weight, every whole zero point in range and random scales; and a fractional or larger zero
+    point must be able to differ, which is why the kernels test for it."""
+    g = torch.Generator().manual_seed(5)
+    q = torch.arange(-128, 128, dtype=torch.float32).reshape(-1, 1, 1)
+    # bf16: zero points -128 .. 128, scales over several binades
+    zp = torch.arange(-128, 129, dtype=torch.float32).reshape(1, -1, 1)
+    s = (torch.empty(64).uniform_(1e-3, 1e-2, generator=g) * 2.0 ** torch.randint(-6, 7, (64,), generator=g)).bfloat16().reshape(1, 1, -1)
+    want = (q.bfloat16() - zp.bfloat16()) * s                                   # two bf16 operations
+    u, off = q.double() + 128.0, 128.0
+    exact = u * s.double() - (off + zp.double()) * s.double()                    # what one fp32 fma returns: see below
+    assert torch.equal(exact.float().double(), exact)                            # ... exactly, in fp32
+    assert torch.equal(((u * s.double()).float()).double(), u * s.double())      # and both products are fp32 numbers
+    assert torch.equal((((off + zp.double()) * s.double()).float()).double(), (off + zp.double()) * s.double())
+    assert torch.equal(exact.float().bfloat16(), want)
+    # fp16: zero points -512 .. 512 under the offset 1152 (int8) of the exponent-trick conversion
+    zp = torch.arange(-512, 513, dtype=torch.float32).reshape(1, -1, 1)
+    s = torch.empty(16).uniform_(1e-3, 1e-2, generator=g).half().reshape(1, 1, -1)
+    want = (q.half() - zp.half()) * s
+    x = (q + 1152.0).half()
+    assert torch.equal(x.float(), q + 1152.0)
+    sub = (torch.tensor(1152.0).half() + zp.half())                              # formed once per channel
+    assert torch.equal(sub.float(), 1152.0 + zp)
+    assert torch.equal((x - sub) * s, want)
+    # the odd int4 channel's offset of 72, in steps of 1/16 under the exponent of 64
+    q4 = torch.arange(-8, 8, dtype=torch.float32).reshape(-1, 1, 1)
+    x = (q4 + 72.0).half()
+    sub = (torch.tensor(72.0).half() + zp.half())
+    assert torch.equal(sub.float(), 72.0 + zp) and torch.equal((x - sub) * s, (q4.half() - zp.half()) * s)
+    # not so beyond the range: q - zp no longer fits the type and the reference's first rounding shows
+    zp_bad = torch.tensor([300.0, 3.3]).bfloat16().reshape(1, -1, 1)
+    s1 = torch.tensor([0.0078125 * 1.3]).bfloat16().reshape(1, 1, -1)
+    two = (q.bfloat16() - zp_bad) * s1
+    one = ((q.double() - zp_bad.double()) * s1.double()).float().bfloat16()
+    assert not torch.equal(one[:, 0], two[:, 0]) and not torch.equal(one[:, 1], two[:, 1])
