@@ -1368,9 +1368,10 @@ static void launch_stream(WoArgs& p, hipStream_t st) {
 // the decode kernels keep a copy of the activation rows in LDS up to this size
 constexpr size_t kDecodeActLdsBytes = 33 * 1024;
 
-// gemv_only: take the one-wave-per-tile kernel or nothing
+// gemv_only: take the one-wave-per-tile kernel or nothing; lds_only: nothing where the activations do not fit the
+// kernel's LDS copy (the kernel without that copy is not wanted)
 template <int WBITS, int ADT>
-static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
+static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only, bool lds_only = false) {
     constexpr int NH = WBITS == 4 ? 2 : 1;
     if (p.M > 8 || p.K % 128 != 0) return false;
     // groups of 32 or 64: only with fp16 activations and fp16 tables (every weight dequantised to fp16 first)
@@ -1513,7 +1514,7 @@ static bool launch_decode(WoArgs& p, hipStream_t st, bool gemv_only) {
 #undef FNN_DEC
         return true;
     }
-    if (small_groups) return false;      // the kernel below walks groups of whole 128-value steps
+    if (small_groups || lds_only) return false;      // the kernel below walks groups of whole 128-value steps
     const size_t smem = fixed + (act_lds ? act_bytes : 0);
     if (smem > 64 * 1024) return false;
     note_kernel("gemm_wo_decode_kernel", WBITS, p.group, act_lds);
@@ -1632,6 +1633,16 @@ static void dispatch_wo(WoArgs& p, hipStream_t st) {
     // whose waves share the activations through LDS; the other decode kernels for a single row and
     // for the shapes the panel kernel does not take.
     if (p.M <= 4 && (WBITS == 4 || p.M == 1) && launch_decode<WBITS, ADT>(p, st, true)) return;
+    // 2 to 4 rows over at most 4096 weight rows: such a call is a handful of memory latencies, and the decode kernel
+    // (512 workgroups at most, K split over the waves of each, the activations copied to LDS once) gets through them
+    // sooner than the panel kernel's slab pipeline with its barrier per slab.  Measured under a captured graph with
+    // rotating weights, panel / decode kernel, us - int8 per channel N=K=4096: M=2 8.7 / 6.8, M=4 8.6 / 7.6; N=2048
+    // K=2048 5.9 / 4.4; N=2048 K=8192 M=2 10.2 / 6.5; int4 g128 N=K=4096 8.7 / 6.4 and 8.7 / 6.9; N=8192 K=4096 9.6 /
+    // 8.2 and 9.5 / 9.1.  With more weight rows every workgroup's own copy of the activations (M K 2 bytes against the
+    // 8 K bytes of its weights) costs more than the latencies saved: int8 N=8192 K=2048 7.7 / 8.7, N=4608 K=3584
+    // 8.7 / 9.5.  Inside the rule the decode kernel is behind by at most 9 % (int4 N=4608 K=3584 M=4 8.5 / 9.3).
+    // Both kernels round alike (per weight with per-channel tables of the activations' type, in fp32 otherwise).
+    if (p.M >= 2 && p.M <= 4 && (WBITS == 4 ? p.N / 2 : p.N) <= 4096 && launch_decode<WBITS, ADT>(p, st, false, true)) return;
     // More than 64 rows: the tiled kernel dequantises every weight once per 128 or 256 rows (the panel kernel
     // takes 64 a pass), but a tile is one workgroup walking all of K: with 128 tiles or fewer half the CUs
     // or more stand idle while the others each need about 1.3 us per 128 values of K, and 64-row passes of the

@@ -864,7 +864,25 @@ def test_weight_only_reference_test_shape():
             for with_bias in (False, True):
                 case = _wo_inputs(3, 1024, 4096, group, 8, torch.float16, torch.float16, with_zp, with_bias, seed=9)
                 _wo_check(*case, group, 8, torch.float16, strict=True)
-                assert _lib.last_kernel().startswith("gemm_wo_decode_lds_kernel" if group else "gemm_wo_panel_kernel(per-weight")
+                assert _lib.last_kernel().startswith("gemm_wo_decode_lds_kernel(per-weight rounding)"), _lib.last_kernel()
+
+
+@pytest.mark.parametrize("bits,group,M,N,K,kernel", [
+    (8, 0, 2, 4096, 4096, "gemm_wo_decode_lds_kernel"), (8, 0, 4, 4096, 4096, "gemm_wo_decode_lds_kernel"),
+    (4, 128, 4, 8192, 2048, "gemm_wo_decode_lds_kernel"), (4, 0, 3, 2048, 1024, "gemm_wo_decode_lds_kernel"),
+    (8, 128, 2, 2048, 8192, "gemm_wo_decode_lds_kernel"),
+    (8, 0, 4, 4608, 1024, "gemm_wo_panel_kernel"),          # more than 4096 weight rows
+    (8, 0, 3, 2048, 8192, "gemm_wo_panel_kernel"),          # three rows of 8192 values do not fit the LDS copy
+    (8, 0, 5, 4096, 4096, "gemm_wo_panel_kernel"),          # five rows
+    (4, 128, 4, 8704, 1024, "gemm_wo_panel_kernel")])
+def test_weight_only_two_to_four_rows_over_few_weight_rows(bits, group, M, N, K, kernel):
+    """2 to 4 activation rows over at most 4096 weight rows run on the decode kernel where its LDS copy of the
+    activations fits, on the panel kernel otherwise; both round alike."""
+    for act_ty in (torch.float16, torch.bfloat16):
+        case = _wo_inputs(M, N, K, group, bits, act_ty, torch.float16, True, M == 2, seed=300 + M)
+        _wo_check(*case, group, bits, act_ty, cols=np.r_[0:128, N - 128:N])
+        assert _lib.last_kernel().startswith(kernel), _lib.last_kernel()
+        assert ("per-weight rounding" in _lib.last_kernel()) == (group == 0 and act_ty == torch.float16), _lib.last_kernel()
 
 
 @pytest.mark.parametrize("bits", [8, 4])
