@@ -430,10 +430,21 @@ template <int MODE>
 static bool launch_skinny_t(A8W8Args& p, hipStream_t st) {
     // a single activation row gains nothing from shared slabs (measured 14.0 against 16.5 us at K = N = 8192)
     // (it takes the shared-slab kernel all the same when K is no multiple of 128, which only that one handles)
-    if ((p.M > 1 || p.K % 128 != 0) && launch_a8_panel_t<MODE>(p, st)) return true;
-    if (p.M > 64 || p.K % 128 != 0 || p.lda % 16 != 0 || p.ldb % 16 != 0 ||
-        ((uintptr_t)p.a % 16) != 0 || ((uintptr_t)p.b % 16) != 0)
-        return false;
+    const bool skinny_ok = p.M <= 64 && p.K % 128 == 0 && p.lda % 16 == 0 && p.ldb % 16 == 0 &&
+                           ((uintptr_t)p.a % 16) == 0 && ((uintptr_t)p.b % 16) == 0;
+    // Up to 16 rows, two kinds of shapes on which this kernel (16 channels per workgroup, K split over its waves,
+    // no barrier per slab) beats the shared-slab kernel; both kernels timed over 60 shapes under a captured graph
+    // with rotating weights, shared-slab / this kernel, us.  Few workgroups - N <= 4096, one per CU or fewer, at any
+    // K (N=K=2048 4.6 / 3.5, N=K=4096 M=2..8 6.7 / 6.3, M=16 7.1 / 6.8, N=4096 K=11008 11.5 / 10.5, N=1536 K=8960
+    // 7.8 / 6.0), or N <= 8192 with K <= 3072 (N=8192 K=2048 6.3 / 5.3): the call is a handful of latencies.  And up
+    // to 8 rows of K >= 8192 over N >= 8192: N=12288 25.6 / 20.0, N=16384 33.7 / 25.1, N=28672 49.3 / 40.1, N=32768
+    // 58.4 / 44.7; K=11008 N=12288 33.3 / 28.7.  Elsewhere the shared-slab kernel is level or ahead (N=4608 K=4096
+    // 6.8 / 7.2, N=12288 K=4096 11.9 / 13.5, N=28672 K=4096 23.7 / 25.9; from 17 rows on everywhere).
+    const bool few_workgroups = p.N <= 4096 || (p.N <= 8192 && p.K <= 3072);
+    const bool long_rows = p.M <= 8 && p.K >= 8192 && p.N >= 8192;
+    const bool prefer = skinny_ok && p.M <= 16 && (few_workgroups || long_rows);
+    if (!prefer && (p.M > 1 || p.K % 128 != 0) && launch_a8_panel_t<MODE>(p, st)) return true;
+    if (!skinny_ok) return false;
     const dim3 grid((p.N + 15) / 16), block(kSkWaves * 64);
     note_kernel("gemm_a8w8_skinny_kernel", (p.M + 15) / 16);
     if (p.M <= 16) gemm_a8w8_skinny_kernel<1, MODE><<<grid, block, 0, st>>>(p);

@@ -218,6 +218,26 @@ def test_a8w8_between_one_and_two_rounds_of_few_row_workgroups(M, N, K, kernel):
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
 
 
+@pytest.mark.parametrize("M,N,K,kernel", [(2, 4096, 4096, "skinny"), (16, 4096, 1024, "skinny"), (9, 1024, 11008, "skinny"),
+                                          (16, 8192, 3072, "skinny"), (8, 8192, 8192, "skinny"), (3, 16384, 8192, "skinny"),
+                                          (17, 4096, 4096, "panel"), (16, 4112, 4096, "panel"), (16, 8192, 3200, "panel"),
+                                          (9, 16384, 8192, "panel"), (8, 16384, 8064, "panel"), (8, 8176, 8192, "panel"),
+                                          (4, 4096, 1056, "panel")])
+def test_a8w8_up_to_16_rows_which_few_row_kernel(M, N, K, kernel):
+    """Up to 16 rows: the kernel that splits K over the waves of a 16-channel workgroup where there are few
+    workgroups (N <= 4096, or N <= 8192 with K <= 3072) and for up to 8 rows of K >= 8192 over N >= 8192; the
+    shared-slab kernel next to those ranges (and for any K that is no multiple of 128).  Same bits either way."""
+    a, b = _rand_i8((M, K), 63), _rand_i8((N, K), 64)
+    acc = flashnn_amd.launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
+    assert _lib.last_kernel().startswith(f"gemm_a8w8_{kernel}_kernel"), _lib.last_kernel()
+    assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
+    g = torch.Generator().manual_seed(65)
+    ar, ac = (torch.rand(M, generator=g) * 0.05).half(), (torch.rand(N, generator=g) * 0.05).half()
+    out = flashnn_amd.GemmA8W8(torch.bfloat16)(a.to(DEV), b.to(DEV), ar.to(DEV), ac.to(DEV)).float().cpu().numpy()
+    assert _lib.last_kernel().startswith(f"gemm_a8w8_{kernel}_kernel"), _lib.last_kernel()
+    assert np.array_equal(out, O.gemm_a8w8_epilogue_fp32(acc, O.to_np(ar), O.to_np(ac), O.BF16))
+
+
 @pytest.mark.parametrize("M,N,tile", [(100, 33024, "256,192"), (128, 38912, "256,192"), (65, 32768, "128,128"), (129, 33024, None)])
 def test_a8w8_few_rows_over_a_little_more_than_one_round_of_tiles(M, N, tile):
     """Up to 128 rows over 32769 .. 38912 channels take one round of 256x192 tiles (rows beyond M are padding)
