@@ -1912,6 +1912,61 @@ def test_c_abi_row_strides(hip_lib):
     assert bool((qbuf[:, :8] == 5).all()) and bool((qbuf[:, 8 + 1024:] == 5).all())
 
 
+SEEN_STRIDED_KERNELS = set()
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("group", [0, 128])
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 2048), (3, 1024, 2048), (3, 8704, 1024), (8, 2048, 1152), (16, 2048, 2048),
+                                   (40, 1056, 2304), (70, 512, 1024), (200, 16512, 512), (1, 256, 18944), (24, 528, 512)])
+def test_weight_only_c_abi_row_strides(hip_lib, bits, group, M, N, K):
+    """The weight-only entry points take row strides (lda >= K, ldw >= K, ldc >= N): activations, weights and output
+    that are column slices of wider buffers give the bits of the contiguous call, on every kernel family (decode,
+    GEMV, panel, tiled, stream), and nothing is written outside the output's columns."""
+    if group and K % group:
+        pytest.skip("K is no multiple of the group size")
+    act_ty = torch.float16 if (M + bits) % 2 else torch.bfloat16
+    act, w, qw, scale, zp, bias = _wo_inputs(M, N, K, group, bits, act_ty, torch.float16, True, True, seed=400 + M)
+    dev = torch.device(DEV)
+    rows = qw.shape[0]
+    abuf = torch.zeros(M, K + 64, dtype=act_ty, device=DEV)
+    wbuf = torch.zeros(rows, K + 48, dtype=torch.int8, device=DEV)
+    a, q = abuf[:, 8:8 + K], wbuf[:, 16:16 + K]                      # 16-byte aligned starts, strided rows
+    a.copy_(act.to(DEV)); q.copy_(qw.to(DEV))
+    obuf = torch.full((M, N + 24), 7.0, dtype=act_ty, device=DEV)
+    out = obuf[:, 8:8 + N]
+    sc, z, b = scale.to(DEV), zp.to(DEV), bias.to(DEV)
+    fn = hip_lib.fnn_gemm_a16w8 if bits == 8 else hip_lib.fnn_gemm_a16w4
+    code = _lib.dtype_code
+    rc = fn(out.data_ptr(), a.data_ptr(), q.data_ptr(), sc.data_ptr(), b.data_ptr(), z.data_ptr(), M, N, K,
+            a.stride(0), q.stride(0), out.stride(0), group, code(act_ty), code(act_ty), code(sc.dtype), code(z.dtype),
+            code(b.dtype), _lib.current_stream(dev))
+    assert rc == 0, hip_lib.fnn_last_error()
+    strided_kernel = _lib.last_kernel()
+    plain = torch.empty(M, N, dtype=act_ty, device=DEV)
+    ac, qc = a.contiguous(), q.contiguous()
+    rc = fn(plain.data_ptr(), ac.data_ptr(), qc.data_ptr(), sc.data_ptr(), b.data_ptr(), z.data_ptr(), M, N, K,
+            K, K, N, group, code(act_ty), code(act_ty), code(sc.dtype), code(z.dtype), code(b.dtype),
+            _lib.current_stream(dev))
+    assert rc == 0, hip_lib.fnn_last_error()
+    torch.cuda.synchronize()
+    assert _lib.last_kernel() == strided_kernel, (strided_kernel, _lib.last_kernel())
+    assert torch.equal(out, plain), strided_kernel
+    SEEN_STRIDED_KERNELS.add(strided_kernel.split("<")[0].split("(")[0])
+    assert bool((obuf[:, :8] == 7).all()) and bool((obuf[:, 8 + N:] == 7).all()), strided_kernel
+    # ... and the contiguous call is the operator's result
+    via_op = flashnn_amd.GemmWeightOnly(act_ty)(ac, qc, sc, b, z)
+    assert torch.equal(via_op, plain) or M > 64      # (beyond 64 bf16 rows the operator adds the conversion scratch)
+
+
+def test_weight_only_c_abi_row_strides_reached_every_kernel_family():
+    """(runs after the cases above: they must have gone through the decode, panel, tiled and stream kernels)"""
+    if len(SEEN_STRIDED_KERNELS) == 0:
+        pytest.skip("the strided cases did not run in this session")
+    for family in ("gemm_wo_decode_lds_kernel", "gemm_wo_panel_kernel", "gemm_wo_tile_kernel", "gemm_wo_stream_kernel"):
+        assert family in SEEN_STRIDED_KERNELS, (family, sorted(SEEN_STRIDED_KERNELS))
+
+
 # ----------------------------------------------------------------------------- empty inputs
 def test_empty_inputs_through_the_operators():
     """No rows (or no channels) is a valid call: nothing is launched, the outputs have the right shapes."""
