@@ -1912,6 +1912,31 @@ def test_c_abi_row_strides(hip_lib):
     assert bool((qbuf[:, :8] == 5).all()) and bool((qbuf[:, 8 + 1024:] == 5).all())
 
 
+@pytest.mark.parametrize("M,N,K,kernel", [(1, 1024, 2048, "skinny"), (8, 1024, 2048, "skinny"), (1, 528, 1056, "panel"),
+                                          (32, 2048, 1024, "panel"), (64, 8192, 1152, "panel"), (300, 520, 1056, "ring"),
+                                          (40, 20480, 512, "ring"), (5, 100, 96, "any")])
+def test_a8w8_c_abi_row_strides_on_every_kernel(hip_lib, M, N, K, kernel):
+    """Strided operand and output rows (16-byte aligned starts) through each A8W8 kernel: the bits of the oracle, and
+    nothing written outside the output's columns."""
+    abuf, bbuf = _rand_i8((M, K + 64), 45).to(DEV), _rand_i8((N, K + 32), 46).to(DEV)
+    a, b = abuf[:, 16:16 + K], bbuf[:, 32:32 + K]
+    g = torch.Generator().manual_seed(47)
+    ar = (torch.rand(M, generator=g) * 0.05).half().to(DEV)
+    ac = (torch.rand(N, generator=g) * 0.05).half().to(DEV)
+    obuf = torch.full((M, N + 40), 7.0, dtype=torch.bfloat16, device=DEV)
+    out = obuf[:, 8:8 + N]
+    rc = hip_lib.fnn_gemm_a8w8(out.data_ptr(), a.data_ptr(), b.data_ptr(), ar.data_ptr(), ac.data_ptr(), M, N, K,
+                               a.stride(0), b.stride(0), out.stride(0), _lib.dtype_code(torch.bfloat16), 0, 0,
+                               _lib.current_stream(torch.device(DEV)))
+    assert rc == 0, hip_lib.fnn_last_error()
+    torch.cuda.synchronize()
+    assert _lib.last_kernel().startswith(f"gemm_a8w8_{kernel}_kernel"), _lib.last_kernel()
+    want = O.gemm_a8w8_epilogue_fp32(O.gemm_a8w8_acc(a.cpu().numpy(), b.cpu().numpy()), O.to_np(ar.cpu()),
+                                     O.to_np(ac.cpu()), O.BF16)
+    assert np.array_equal(out.float().cpu().numpy(), want)
+    assert bool((obuf[:, :8] == 7).all()) and bool((obuf[:, 8 + N:] == 7).all())
+
+
 SEEN_STRIDED_KERNELS = set()
 
 
