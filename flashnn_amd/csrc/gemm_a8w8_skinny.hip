@@ -406,7 +406,13 @@ static bool launch_a8_panel_t(A8W8Args& p, hipStream_t st) {
         for (int m = cand == 1 ? 1 : cand; m >= m_lo; m >>= 1) {
             if (m > need && m > m_lo) continue;               // more row blocks than there are rows
             const int64_t wgs = (int64_t)(p.N / (16 * cand)) * ((p.M + m * 16 - 1) / (m * 16));
-            const double cost = (double)((wgs + 255) / 256) * (8.0 + (double)((KT * cand + 7) / 8) * per_iter[m]);
+            double cost = (double)((wgs + 255) / 256) * (8.0 + (double)((KT * cand + 7) / 8) * per_iter[m]);
+            // Weight rows a multiple of 8 KiB apart: a workgroup's 64 rows then start in the same few memory channels,
+            // and 32-row workgroups stream them better (forced pairs under a captured graph, M=16, K=8192, 64 / 32
+            // rows per workgroup, us: N=12288 25.6 / 24.1, N=16384 33.8 / 26.1, N=28672 50.8 / 47.0, N=32768 58.5 /
+            // 49.8; at K=4096 and K=11008 the 64-row workgroups are level or ahead: N=16384 14.9 / 16.3, 38.6 / 38.8)
+            // (measured for up to 16 rows only)
+            if (cand == 4 && p.M <= 16 && p.ldb % 8192 == 0) cost *= 1.3;
             if (rt == 0 || cost < best) { best = cost; rt = cand; mb = m; }
         }
     }

@@ -222,14 +222,17 @@ def test_a8w8_between_one_and_two_rounds_of_few_row_workgroups(M, N, K, kernel):
                                           (16, 8192, 3072, "skinny"), (8, 8192, 8192, "skinny"), (3, 16384, 8192, "skinny"),
                                           (17, 4096, 4096, "panel"), (16, 4112, 4096, "panel"), (16, 8192, 3200, "panel"),
                                           (9, 16384, 8192, "panel"), (8, 16384, 8064, "panel"), (8, 8176, 8192, "panel"),
-                                          (4, 4096, 1056, "panel")])
+                                          (4, 4096, 1056, "panel"), (16, 16384, 8192, "panel<1,2"), (16, 16384, 4096, "panel<2,4"),
+                                          (16, 16384, 8320, "panel<2,4")])
 def test_a8w8_up_to_16_rows_which_few_row_kernel(M, N, K, kernel):
     """Up to 16 rows: the kernel that splits K over the waves of a 16-channel workgroup where there are few
     workgroups (N <= 4096, or N <= 8192 with K <= 3072) and for up to 8 rows of K >= 8192 over N >= 8192; the
-    shared-slab kernel next to those ranges (and for any K that is no multiple of 128).  Same bits either way."""
+    shared-slab kernel next to those ranges (and for any K that is no multiple of 128) - with 32 instead of 64 weight
+    rows per workgroup where the rows lie a multiple of 8 KiB apart.  Same bits either way."""
     a, b = _rand_i8((M, K), 63), _rand_i8((N, K), 64)
     acc = flashnn_amd.launchers.hip_gemm_a8w8_int32(a.to(DEV), b.to(DEV)).cpu().numpy()
-    assert _lib.last_kernel().startswith(f"gemm_a8w8_{kernel}_kernel"), _lib.last_kernel()
+    kernel, _, blocks = kernel.partition("<")
+    assert _lib.last_kernel().startswith(f"gemm_a8w8_{kernel}_kernel" + ("<" + blocks if blocks else "")), _lib.last_kernel()
     assert np.array_equal(acc, O.gemm_a8w8_acc(a.numpy(), b.numpy()))
     g = torch.Generator().manual_seed(65)
     ar, ac = (torch.rand(M, generator=g) * 0.05).half(), (torch.rand(N, generator=g) * 0.05).half()
