@@ -677,6 +677,33 @@ def test_fused_moe_a8w8_many_rows_bit_exact(shape, out_ty):
             assert (want == 3.0).any()
 
 
+@pytest.mark.parametrize("shape", [(16, 8, 1024, 1024, 2, 16), (1024, 8, 1024, 1024, 2, 64), (9, 4, 48, 80, 2, 16)])
+def test_fused_moe_a8w8_strided_operands(shape):
+    """Tokens, expert weights and output that are column slices of wider buffers (the launcher passes their row and
+    expert strides): the bits of the call on contiguous copies, on the few-row, the tiled and the guarded kernel, and
+    nothing written outside the output's columns."""
+    M, E, N, K, top_k, BM = shape
+    g = torch.Generator().manual_seed(M + 7)
+    abuf = torch.randint(-128, 128, (M, K + 64), dtype=torch.int8, generator=g).to(DEV)
+    bbuf = torch.randint(-128, 128, (E, N + 3, K + 32), dtype=torch.int8, generator=g).to(DEV)
+    a, b = abuf[:, 16:16 + K], bbuf[:, 1:1 + N, 16:16 + K]
+    ar = (torch.rand(M, generator=g) * 0.05).half().to(DEV)
+    ac = (torch.rand(E, N, generator=g) * 0.05).float().to(DEV)
+    w, ids = torch.topk(torch.softmax(torch.randn(M, E, generator=g), -1), top_k, dim=-1)
+    w = w.float().contiguous()
+    s_, e_, used = workloads.moe_align_block_size(ids, BM, E)
+    cbuf = torch.full((M, top_k, N + 24), 3.0, dtype=torch.float16, device=DEV)
+    c = cbuf[:, :, 8:8 + N]
+    args = (ar, ac, w.to(DEV), ids.to(DEV), s_.to(DEV), e_.to(DEV), used.to(DEV), True, top_k, BM)
+    flashnn_amd.fused_moe_a8w8_forward(a, b, c, *args)
+    strided_kernel = _lib.last_kernel()
+    plain = torch.full((M, top_k, N), 3.0, dtype=torch.float16, device=DEV)
+    flashnn_amd.fused_moe_a8w8_forward(a.contiguous(), b.contiguous(), plain, *args)
+    assert _lib.last_kernel() == strided_kernel, (strided_kernel, _lib.last_kernel())
+    assert torch.equal(c, plain), strided_kernel
+    assert bool((cbuf[:, :, :8] == 3).all()) and bool((cbuf[:, :, 8 + N:] == 3).all())
+
+
 @pytest.mark.parametrize("act_ty", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("group,zp_kind", [(0, "float"), (0, None), (0, "int8"), (128, "float"), (128, None), (128, "int8"),
                                            (64, "int8")])
