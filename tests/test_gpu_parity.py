@@ -752,6 +752,34 @@ def test_fused_moe_a16w4_close(shape, group, zp_kind, act_ty):
     assert bool((got2[rest] == 3.0).all()) and not bool((got2[first] == 3.0).all())
 
 
+@pytest.mark.parametrize("group", [0, 128])
+@pytest.mark.parametrize("shape", [(16, 8, 512, 1024, 2, 16), (1024, 8, 256, 1024, 2, 128), (9, 3, 16, 128, 2, 16)])
+def test_fused_moe_a16w4_strided_operands(shape, group):
+    """Tokens, packed expert weights and output as column slices of wider buffers: the bits of the call on contiguous
+    copies, on the few-row, the tiled and the guarded kernel; nothing written outside the output's columns."""
+    M, E, N2, K, top_k, BM = shape
+    g = torch.Generator().manual_seed(M + 11)
+    abuf = torch.randn(M, K + 64, generator=g).half().to(DEV)
+    bbuf = torch.randint(-128, 128, (E, N2 + 3, K + 32), dtype=torch.int8, generator=g).to(DEV)
+    a, b = abuf[:, 8:8 + K], bbuf[:, 2:2 + N2, 16:16 + K]
+    sshape = (E, 2 * N2) if group == 0 else (E, 2 * N2, K // group)
+    scale = torch.empty(sshape).uniform_(1e-3, 1e-2, generator=g).half().to(DEV)
+    zp = torch.randint(-3, 4, sshape, generator=g).half().to(DEV)
+    tw, ids = torch.topk(torch.softmax(torch.randn(M, E, generator=g), -1), top_k, dim=-1)
+    tw = tw.float().contiguous()
+    s_, e_, used = workloads.moe_align_block_size(ids, BM, E)
+    cbuf = torch.full((M, top_k, 2 * N2 + 24), 3.0, dtype=torch.float16, device=DEV)
+    c = cbuf[:, :, 8:8 + 2 * N2]
+    args = (scale, zp, tw.to(DEV), ids.to(DEV), s_.to(DEV), e_.to(DEV), used.to(DEV), True, top_k, BM)
+    flashnn_amd.fused_moe_a16w4_forward(a, b, c, *args)
+    strided_kernel = _lib.last_kernel()
+    plain = torch.full((M, top_k, 2 * N2), 3.0, dtype=torch.float16, device=DEV)
+    flashnn_amd.fused_moe_a16w4_forward(a.contiguous(), b.contiguous(), plain, *args)
+    assert _lib.last_kernel() == strided_kernel, (strided_kernel, _lib.last_kernel())
+    assert torch.equal(c, plain), strided_kernel
+    assert bool((cbuf[:, :, :8] == 3).all()) and bool((cbuf[:, :, 8 + 2 * N2:] == 3).all())
+
+
 @pytest.mark.parametrize("act_ty", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("zp_kind", ["float", None])
 @pytest.mark.parametrize("group", [0, 128])
