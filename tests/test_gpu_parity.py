@@ -1995,6 +1995,45 @@ def test_a8w8_c_abi_row_strides_on_every_kernel(hip_lib, M, N, K, kernel):
     assert bool((obuf[:, :8] == 7).all()) and bool((obuf[:, 8 + N:] == 7).all())
 
 
+@pytest.mark.parametrize("M,K", [(33, 1024), (5, 8192), (4096, 1024), (7, 1000)])
+def test_norm_entry_points_c_abi_row_strides(hip_lib, M, K):
+    """RMSNorm, LayerNorm and their quantising forms with input and output rows that are column slices of wider
+    buffers (ldx > K, ldo > K): the bits of the contiguous call, nothing written outside the output's columns (one
+    workgroup per row, one wave per row, and the any-length kernels)."""
+    dev = torch.device(DEV)
+    st = _lib.current_stream(dev)
+    g = torch.Generator().manual_seed(M + K)
+    xbuf = torch.randn(M, K + 64, generator=g).bfloat16().to(DEV)
+    x = xbuf[:, 8:8 + K]
+    xc = x.contiguous()
+    gamma = torch.empty(K).uniform_(0.5, 1.5, generator=g).to(DEV)
+    beta = torch.randn(K, generator=g).to(DEV)
+    code = _lib.dtype_code
+    def run(call, out_ty, fill):
+        obuf = torch.full((M, K + 32), fill, dtype=out_ty, device=DEV)
+        o = obuf[:, 16:16 + K]
+        plain = torch.empty(M, K, dtype=out_ty, device=DEV)
+        s1, s2 = torch.empty(M, dtype=torch.bfloat16, device=DEV), torch.empty(M, dtype=torch.bfloat16, device=DEV)
+        assert call(o, x, s1) == 0, hip_lib.fnn_last_error()
+        assert call(plain, xc, s2) == 0, hip_lib.fnn_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(o, plain)
+        assert bool((obuf[:, :16] == fill).all()) and bool((obuf[:, 16 + K:] == fill).all())
+        return s1, s2
+    bf, f32 = code(torch.bfloat16), code(torch.float32)
+    run(lambda o, i, s: hip_lib.fnn_rmsnorm(o.data_ptr(), i.data_ptr(), gamma.data_ptr(), 1e-6, M, K, i.stride(0), o.stride(0),
+                                            bf, f32, st), torch.bfloat16, 7.0)
+    run(lambda o, i, s: hip_lib.fnn_layernorm(o.data_ptr(), i.data_ptr(), gamma.data_ptr(), beta.data_ptr(), 1e-5, M, K,
+                                              i.stride(0), o.stride(0), bf, f32, st), torch.bfloat16, 7.0)
+    s1, s2 = run(lambda o, i, s: hip_lib.fnn_rmsnorm_dquant(o.data_ptr(), s.data_ptr(), i.data_ptr(), gamma.data_ptr(), 1e-6, M, K,
+                                                            i.stride(0), o.stride(0), bf, f32, st), torch.int8, 5)
+    assert torch.equal(s1, s2)
+    s1, s2 = run(lambda o, i, s: hip_lib.fnn_layernorm_dquant(o.data_ptr(), s.data_ptr(), i.data_ptr(), gamma.data_ptr(),
+                                                              beta.data_ptr(), 1e-5, M, K, i.stride(0), o.stride(0), bf, f32, st),
+                 torch.int8, 5)
+    assert torch.equal(s1, s2)
+
+
 SEEN_STRIDED_KERNELS = set()
 
 
