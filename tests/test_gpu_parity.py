@@ -2034,6 +2034,36 @@ def test_norm_entry_points_c_abi_row_strides(hip_lib, M, K):
     assert torch.equal(s1, s2)
 
 
+@pytest.mark.parametrize("M", [1, 4, 16, 40, 64, 100])
+def test_a16w4_prepacked_c_abi_row_strides(hip_lib, M):
+    """The packed int4 GEMM with activation and output rows that are column slices of wider buffers: the bits of the
+    contiguous call (one row, and 16, 32 and 64 rows per pass), nothing written outside the output's columns."""
+    N, K = 2048, 1024
+    g = torch.Generator().manual_seed(500 + M)
+    w = torch.randint(-8, 8, (N, K), generator=g, dtype=torch.int8)
+    qw = torch.from_numpy(O.pack_int4(w.numpy())).to(DEV)
+    scale = torch.empty(K // 128, N).uniform_(1e-3, 1e-2, generator=g).half().to(DEV)
+    zp = torch.randint(-4, 4, (K // 128, N), generator=g).half().to(DEV)
+    packed = launchers.hip_a16w4_prepack(qw, scale, zp)
+    bias = torch.randn(N, generator=g).bfloat16().to(DEV)
+    abuf = torch.randn(M, K + 64, generator=g).bfloat16().to(DEV)
+    a = abuf[:, 8:8 + K]
+    ac = a.contiguous()
+    obuf = torch.full((M, N + 24), 7.0, dtype=torch.bfloat16, device=DEV)
+    out = obuf[:, 8:8 + N]
+    plain = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    bf = _lib.dtype_code(torch.bfloat16)
+    st = _lib.current_stream(torch.device(DEV))
+    for o, i in ((out, a), (plain, ac)):
+        rc = hip_lib.fnn_gemm_a16w4_prepacked(o.data_ptr(), i.data_ptr(), packed.buffer.data_ptr(), bias.data_ptr(), M, N, K,
+                                              i.stride(0), o.stride(0), 128, bf, bf, bf, st)
+        assert rc == 0, hip_lib.fnn_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(out, plain), _lib.last_kernel()
+    assert bool((obuf[:, :8] == 7).all()) and bool((obuf[:, 8 + N:] == 7).all())
+    assert torch.equal(launchers.hip_gemm_a16w4_prepacked_forward(torch.empty_like(plain), ac, packed, bias), plain)
+
+
 SEEN_STRIDED_KERNELS = set()
 
 
